@@ -1,0 +1,147 @@
+"""Builds the HIP kernels into one shared library for gfx950.
+
+`build()` compiles every `.hip` file beside this script with hipcc, in
+parallel, and links `liyab_amd/_lib/libliyab_hip.so`; it prints a line per
+file so that a first call in a fresh checkout shows progress. When the
+package folder cannot be written to, the library goes to a per-user folder
+under the system's temporary directory instead. Nothing here needs a GPU:
+hipcc cross-compiles.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import List, Optional
+
+CSRC = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(CSRC)
+LIB_NAME = "libliyab_hip.so"
+ARCH = "gfx950"
+FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fno-gpu-rdc",
+    # packed 32-bit float instructions are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def sources() -> List[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def headers() -> List[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h"))
+
+
+def source_hash() -> str:
+    h = hashlib.sha256()
+    for p in sources() + headers():
+        h.update(os.path.basename(p).encode())
+        with open(p, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def hipcc_path() -> Optional[str]:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def _writable(d: str) -> bool:
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def lib_dirs() -> List[str]:
+    """Where the library may live, in the order they are tried."""
+    user = f"liyab_amd_{os.getuid()}_{source_hash()}"
+    return [os.path.join(PKG, "_lib"), os.path.join(tempfile.gettempdir(), user)]
+
+
+def find_library() -> Optional[str]:
+    for d in lib_dirs():
+        p = os.path.join(d, LIB_NAME)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def is_stale(lib_path: str) -> bool:
+    try:
+        with open(lib_path + ".hash") as f:
+            return f.read().strip() != source_hash()
+    except OSError:
+        return True
+
+
+def _say(msg: str, quiet: bool) -> None:
+    if not quiet:
+        print(f"[liyab_amd build] {msg}", file=sys.stderr, flush=True)
+
+
+def build(quiet: bool = False, jobs: Optional[int] = None) -> str:
+    """Compiles and links; returns the library's path."""
+    hipcc = hipcc_path()
+    if hipcc is None:
+        raise RuntimeError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernels cannot be built")
+    out_dir = next((d for d in lib_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError("no writable folder for the kernel library: tried " + ", ".join(lib_dirs()))
+    obj_dir = os.path.join(out_dir, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    env = dict(os.environ)
+    if not env.get("HOME") or not os.access(env.get("HOME", ""), os.W_OK):
+        env["HOME"] = out_dir  # the compiler driver wants some home folder
+    srcs = sources()
+    jobs = jobs or min(len(srcs), max(1, min(16, os.cpu_count() or 1)))
+    t0 = time.time()
+    _say(f"compiling {len(srcs)} HIP files for {ARCH} with {jobs} jobs into {out_dir}", quiet)
+
+    def compile_one(src: str) -> str:
+        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
+        t = time.time()
+        r = subprocess.run([hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj], env=env, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {os.path.basename(src)}:\n{r.stdout}\n{r.stderr}")
+        _say(f"  {os.path.basename(src)} done in {time.time() - t:.0f} s", quiet)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(compile_one, srcs))
+    lib = os.path.join(out_dir, LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs], env=env,
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, lib)
+    with open(lib + ".hash", "w") as f:
+        f.write(source_hash())
+    shutil.rmtree(obj_dir, ignore_errors=True)
+    _say(f"built {lib} in {time.time() - t0:.0f} s", quiet)
+    return lib
+
+
+if __name__ == "__main__":
+    print(build())

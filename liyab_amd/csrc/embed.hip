@@ -1,0 +1,119 @@
+// Token embedding gather (+ learned positions) and the write of keys and
+// values into cache pages.
+//
+// x[t] = scale * tok[id_t] (+ pos[p_t]): the reference's `embed` followed by
+// `add_positions` (src/core/transformer.cpp:5495-5512, 2791-2808), one pass
+// over the row. The sum is formed in 32-bit and the residual stream it
+// starts is 32-bit on both paths.
+#include "common.h"
+
+namespace liyab {
+
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ tok, const T* __restrict__ pos,
+                             const int* __restrict__ ids, const int* __restrict__ positions, int d, float scale) {
+    const int t = blockIdx.x;
+    const int64_t id = ids[t];
+    const T* trow = tok + id * d;
+    const T* prow = pos != nullptr ? pos + static_cast<int64_t>(positions[t]) * d : nullptr;
+    float* out = x + static_cast<int64_t>(t) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = to_float<T>(trow[i]) * scale;
+        if (prow != nullptr) v += to_float<T>(prow[i]);
+        out[i] = v;
+    }
+}
+
+// x[t] += table[p_t]  (a residual position encoding applied on its own)
+template <typename T>
+__global__ void add_rows_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ rows, int d) {
+    const int t = blockIdx.x;
+    const T* r = table + static_cast<int64_t>(rows[t]) * d;
+    float* out = x + static_cast<int64_t>(t) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] += to_float<T>(r[i]);
+}
+
+// Token t's keys and values, read from its row of the projection output at
+// column offsets k_off and v_off, go to slot[t] = page * page_size + offset
+// of a cache laid out [page][kv_head][page_size][head_dim]
+// (the reference's store_kv, src/core/transformer.cpp:2875-2890).
+template <typename T>
+__global__ void kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc, const T* __restrict__ src, int64_t src_stride,
+                                int k_off, int v_off, const int* __restrict__ slots, int n_kv_head, int hd,
+                                int page_size) {
+    const int t = blockIdx.x;
+    const int64_t slot = slots[t];
+    if (slot < 0) return;
+    const int64_t page = slot / page_size;
+    const int off = static_cast<int>(slot % page_size);
+    const T* row = src + static_cast<int64_t>(t) * src_stride;
+    const int kv_dim = n_kv_head * hd;
+    for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) {
+        const int h = i / hd, e = i % hd;
+        const int64_t dst = ((page * n_kv_head + h) * page_size + off) * hd + e;
+        kc[dst] = row[k_off + i];
+        vc[dst] = row[v_off + i];
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+extern "C" int liyab_embed(float* x, const void* tok, const void* pos, int dtype, const int* ids, const int* positions,
+                           int n, int d, float scale, hipStream_t stream) {
+    LIYAB_REQUIRE(x && tok && ids, "embed: null pointer");
+    LIYAB_REQUIRE(pos == nullptr || positions != nullptr, "embed: a position table needs positions");
+    LIYAB_REQUIRE(d > 0 && n >= 0, "embed: bad sizes n=%d d=%d", n, d);
+    if (n == 0) return 0;
+    const int threads = d >= 256 ? 256 : 64;
+    if (dtype == kF32) {
+        embed_kernel<float><<<n, threads, 0, stream>>>(x, static_cast<const float*>(tok), static_cast<const float*>(pos),
+                                                       ids, positions, d, scale);
+    } else if (dtype == kBF16) {
+        embed_kernel<bf16_t><<<n, threads, 0, stream>>>(x, static_cast<const bf16_t*>(tok),
+                                                        static_cast<const bf16_t*>(pos), ids, positions, d, scale);
+    } else {
+        return fail(1, "embed: unknown dtype %d", dtype);
+    }
+    return check_launch("embed");
+}
+
+extern "C" int liyab_add_rows(float* x, const void* table, int dtype, const int* rows, int n, int d,
+                              hipStream_t stream) {
+    LIYAB_REQUIRE(x && table && rows, "add_rows: null pointer");
+    LIYAB_REQUIRE(d > 0 && n >= 0, "add_rows: bad sizes n=%d d=%d", n, d);
+    if (n == 0) return 0;
+    const int threads = d >= 256 ? 256 : 64;
+    if (dtype == kF32) {
+        add_rows_kernel<float><<<n, threads, 0, stream>>>(x, static_cast<const float*>(table), rows, d);
+    } else if (dtype == kBF16) {
+        add_rows_kernel<bf16_t><<<n, threads, 0, stream>>>(x, static_cast<const bf16_t*>(table), rows, d);
+    } else {
+        return fail(1, "add_rows: unknown dtype %d", dtype);
+    }
+    return check_launch("add_rows");
+}
+
+extern "C" int liyab_kv_write(void* kc, void* vc, const void* src, int dtype, int64_t src_stride, int k_off, int v_off,
+                              const int* slots, int n, int n_kv_head, int hd, int page_size, hipStream_t stream) {
+    LIYAB_REQUIRE(kc && vc && src && slots, "kv_write: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n_kv_head > 0 && hd > 0 && page_size > 0, "kv_write: bad sizes");
+    LIYAB_REQUIRE(k_off >= 0 && v_off >= 0 && k_off + n_kv_head * hd <= src_stride && v_off + n_kv_head * hd <= src_stride,
+                  "kv_write: column offsets %d/%d with %d values do not fit a row of %lld", k_off, v_off, n_kv_head * hd,
+                  static_cast<long long>(src_stride));
+    if (n == 0) return 0;
+    const int threads = n_kv_head * hd >= 256 ? 256 : 64;
+    if (dtype == kF32) {
+        kv_write_kernel<float><<<n, threads, 0, stream>>>(static_cast<float*>(kc), static_cast<float*>(vc),
+                                                          static_cast<const float*>(src), src_stride, k_off, v_off,
+                                                          slots, n_kv_head, hd, page_size);
+    } else if (dtype == kBF16) {
+        kv_write_kernel<bf16_t><<<n, threads, 0, stream>>>(static_cast<bf16_t*>(kc), static_cast<bf16_t*>(vc),
+                                                           static_cast<const bf16_t*>(src), src_stride, k_off, v_off,
+                                                           slots, n_kv_head, hd, page_size);
+    } else {
+        return fail(1, "kv_write: unknown dtype %d", dtype);
+    }
+    return check_launch("kv_write");
+}

@@ -1,0 +1,201 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+The counterpart of the reference's `Transformer::forward_batch`
+(src/core/transformer.cpp:6589-6769): items of many tokens (a portion of a
+prompt, continuing where the request's cache ends) beside items of one token
+(decoding), each of a different request (:6607-6647); rows are the items
+concatenated, a row's position is its request's length plus its index in
+the item (:6689-6697); every block runs over all rows at once and only
+attention looks at a row's own request; logits are computed for the wanted
+rows only (:6738-6767); lengths advance after the pass (:6726-6735) and a
+step that cannot get its pages changes nothing.
+
+Everything that varies from step to step reaches the kernels through one
+block of int32 metadata copied to the device in a single transfer.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.pages import UNMAPPED, CacheManager
+from ..cache.storage import CacheStorage
+from ..errors import ContextFull, InvalidArgument
+from ..parts.base import GroupStep, StepContext, StepHost, Workspace
+
+
+@dataclass
+class StepItem:
+    """A request's next tokens and the places among them whose logits are wanted."""
+
+    rid: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)
+
+
+class _Staging:
+    """A few pinned host buffers used in turn, each with the event of its last copy."""
+
+    def __init__(self, device, depth: int = 4):
+        self.device = device
+        self.depth = depth
+        self.host: List[Optional[torch.Tensor]] = [None] * depth
+        self.events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self.turn = 0
+
+    def next(self, n: int) -> torch.Tensor:
+        i = self.turn
+        self.turn = (self.turn + 1) % self.depth
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        buf = self.host[i]
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1024), dtype=torch.int32, pin_memory=True)
+            self.host[i] = buf
+        self._last = i
+        return buf
+
+    def copied(self) -> None:
+        ev = self.events[self._last]
+        if ev is None:
+            ev = self.events[self._last] = torch.cuda.Event()
+        ev.record()
+
+
+class StepFunction:
+    def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0"):
+        self.model = model
+        self.manager = manager
+        self.storage = storage
+        self.device = torch.device(device)
+        self.workspace = Workspace(self.device)
+        self._staging = _Staging(self.device)
+        self._meta_dev: Optional[torch.Tensor] = None
+        self.steps = 0
+        self.tokens = 0
+
+    # -- validation -----------------------------------------------------------
+    def _validate(self, items: Sequence[StepItem]) -> None:
+        if not items:
+            raise InvalidArgument("a step needs at least one item")
+        seen = set()
+        V = self.model.vocab_size
+        for it in items:
+            if it.rid in seen:
+                raise InvalidArgument(f"request {it.rid!r} appears twice in one step")
+            seen.add(it.rid)
+            if not self.manager.is_open(it.rid):
+                raise InvalidArgument(f"request {it.rid!r} is not open")
+            n = len(it.tokens)
+            if n == 0:
+                raise InvalidArgument(f"request {it.rid!r} brings no tokens")
+            for t in it.tokens:
+                if not (0 <= int(t) < V):
+                    raise InvalidArgument(f"token id {t} of request {it.rid!r} is outside [0, {V})")
+            for w in it.want:
+                if not (0 <= int(w) < n):
+                    raise InvalidArgument(f"request {it.rid!r} wants logits at place {w} of {n} tokens")
+            end = self.manager.length(it.rid) + n
+            if end > self.model.max_positions:
+                raise ContextFull(
+                    f"position {end - 1} is past the model's {self.model.max_positions} learned positions")
+
+    # -- the step -------------------------------------------------------------
+    def run(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
+        """Runs the items as one batch from the cache earlier steps left.
+        Returns float32 logits [wanted, vocab] on the device, rows in the order
+        of the items and of each item's `want`, or None when nothing is wanted.
+        The tensor is workspace memory: valid until the next step."""
+        self._validate(items)
+        mgr = self.manager
+        first = [mgr.length(it.rid) for it in items]
+        q_lens = [len(it.tokens) for it in items]
+        mgr.reserve([(it.rid, f + n) for it, f, n in zip(items, first, q_lens)])
+
+        S, N = len(items), sum(q_lens)
+        R = sum(len(it.want) for it in items)
+        W = mgr.max_blocks
+        G = len(mgr.groups)
+        page = mgr.page_size
+        starts = np.zeros(S + 1, dtype=np.int64)
+        np.cumsum(q_lens, out=starts[1:])
+
+        # layout of the metadata block (int32 words)
+        off = {}
+        cur = 0
+        for name, size in (("token_ids", N), ("positions", N), ("tok_seq", N), ("seq_starts", S + 1),
+                           ("context_lens", S), ("state_slots", S), ("logit_rows", max(R, 1))):
+            off[name] = (cur, size)
+            cur += size
+        for g in range(G):
+            off[f"bt{g}"] = (cur, S * W)
+            cur += S * W
+            off[f"slots{g}"] = (cur, N)
+            cur += N
+        total = cur
+        host_t = self._staging.next(total)
+        host = host_t.numpy()
+
+        def view(name):
+            o, size = off[name]
+            return host[o:o + size]
+
+        tok, pos, seq = view("token_ids"), view("positions"), view("tok_seq")
+        rows = view("logit_rows")
+        rows[:] = 0
+        r = 0
+        for i, it in enumerate(items):
+            a, b = int(starts[i]), int(starts[i + 1])
+            tok[a:b] = np.asarray(it.tokens, dtype=np.int32)
+            pos[a:b] = np.arange(first[i], first[i] + q_lens[i], dtype=np.int32)
+            seq[a:b] = i
+            for w in it.want:
+                rows[r] = a + int(w)
+                r += 1
+        view("seq_starts")[:] = starts
+        view("context_lens")[:] = [f + n for f, n in zip(first, q_lens)]
+        view("state_slots")[:] = [mgr.slot(it.rid) for it in items]
+        for g in range(G):
+            bt = view(f"bt{g}").reshape(S, W)
+            bt[:] = UNMAPPED
+            sl = view(f"slots{g}")
+            for i, it in enumerate(items):
+                table = np.asarray(mgr.block_table(it.rid, g), dtype=np.int32)
+                bt[i, :len(table)] = table
+                a, b = int(starts[i]), int(starts[i + 1])
+                p = pos[a:b]
+                pages = table[p // page]
+                if (pages < 0).any():
+                    raise AssertionError("a token of this step maps to a released page")
+                sl[a:b] = pages * page + p % page
+
+        if self._meta_dev is None or self._meta_dev.numel() < total:
+            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        dev = self._meta_dev
+        dev[:total].copy_(host_t[:total], non_blocking=True)
+        self._staging.copied()
+
+        def dview(name):
+            o, size = off[name]
+            return dev[o:o + size]
+
+        ctx = StepContext(
+            n_tokens=N, n_seqs=S,
+            token_ids=dview("token_ids"), positions=dview("positions"), tok_seq=dview("tok_seq"),
+            seq_starts=dview("seq_starts"), context_lens=dview("context_lens"), state_slots=dview("state_slots"),
+            logit_rows=dview("logit_rows"), n_logit_rows=R,
+            groups=[GroupStep(block_tables=dview(f"bt{g}").view(S, W), slots=dview(f"slots{g}")) for g in range(G)],
+            host=StepHost(q_lens=q_lens, starts=[int(s) for s in starts[:-1]], first_pos=first,
+                          max_q_len=max(q_lens), max_context=max(f + n for f, n in zip(first, q_lens))),
+            workspace=self.workspace, dtype=self.model.dtype, page_size=page,
+        )
+        logits = self.model.forward(ctx, self.storage)
+        for it, f, n in zip(items, first, q_lens):
+            mgr.commit(it.rid, f + n)
+        self.steps += 1
+        self.tokens += N
+        return logits

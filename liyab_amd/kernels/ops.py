@@ -1,0 +1,265 @@
+"""The kernels as functions over torch tensors.
+
+Each function checks on the host that shapes, dtypes and layouts are what
+its kernel and grid assume, then launches on torch's current stream. Torch
+supplies the device memory and the stream; every computation is the
+library's own kernel. Nothing here runs without the GPU and the library.
+"""
+
+from __future__ import annotations
+
+import struct
+from typing import Optional
+
+import torch
+
+from ..errors import KernelError
+from . import lib as _lib
+
+F32, BF16 = 0, 1
+EPI_NONE, EPI_GELU_TANH, EPI_GELU_ERF, EPI_RESIDUAL = 0, 1, 2, 3
+ACTIVATION_EPILOGUE = {"none": EPI_NONE, "gelu_tanh": EPI_GELU_TANH, "gelu_erf": EPI_GELU_ERF}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise KernelError(f"the kernels take float32 or bfloat16, not {dt}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{what} must be on the GPU")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+    _dev(t, what)
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{what} must be contiguous int32")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{what} holds {t.numel()} values, {n} are needed")
+
+
+def _f32vec(t: Optional[torch.Tensor], what: str, n: int) -> None:
+    if t is None:
+        return
+    _dev(t, what)
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n:
+        raise KernelError(f"{what} must be {n} contiguous float32 values, got {tuple(t.shape)} {t.dtype}")
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    _dev(t, what)
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{what} must be 2-D with contiguous rows, got shape {tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def check_device() -> None:
+    _lib.call("liyab_check_device")
+
+
+def fill_(t: torch.Tensor, value: float | int) -> torch.Tensor:
+    _dev(t, "fill target")
+    if not t.is_contiguous():
+        raise KernelError("fill target must be contiguous")
+    if t.dtype == torch.float32:
+        bits = struct.unpack("<I", struct.pack("<f", float(value)))[0]
+        size = 4
+    elif t.dtype == torch.int32:
+        bits = int(value) & 0xFFFFFFFF
+        size = 4
+    elif t.dtype == torch.bfloat16:
+        bits = struct.unpack("<I", struct.pack("<f", float(value)))[0]
+        bits = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) & 0xFFFF if value == value else 0x7FC0
+        size = 2
+    else:
+        raise KernelError(f"fill: unsupported dtype {t.dtype}")
+    _lib.call("liyab_fill", t.data_ptr(), size, bits, t.numel(), _stream())
+    return t
+
+
+def add_into_(residual: torch.Tensor, x: torch.Tensor) -> None:
+    """residual (float32) += x, elementwise."""
+    _dev(residual, "residual")
+    _dev(x, "x")
+    if residual.dtype != torch.float32 or not residual.is_contiguous() or not x.is_contiguous():
+        raise KernelError("add_into: residual must be contiguous float32 and x contiguous")
+    if residual.numel() != x.numel():
+        raise KernelError(f"add_into: {residual.numel()} vs {x.numel()} values")
+    _lib.call("liyab_add_into", residual.data_ptr(), x.data_ptr(), dtype_code(x.dtype), x.numel(), _stream())
+
+
+def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0,
+          pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
+    """out[t] = scale * table[ids[t]] (+ pos_table[positions[t]]); out is float32 [n, d].
+    The caller has checked ids against the table's rows (and positions against pos_table's)."""
+    _dev(out, "out")
+    n, d = out.shape
+    if out.dtype != torch.float32 or not out.is_contiguous():
+        raise KernelError("embed: out must be contiguous float32")
+    if table.dim() != 2 or table.shape[1] != d or not table.is_contiguous():
+        raise KernelError(f"embed: table {tuple(table.shape)} does not have rows of {d}")
+    _i32(ids, "ids", n)
+    if pos_table is not None:
+        if pos_table.dtype != table.dtype or pos_table.dim() != 2 or pos_table.shape[1] != d or not pos_table.is_contiguous():
+            raise KernelError("embed: the position table must match the token table's dtype and width")
+        if positions is None:
+            raise KernelError("embed: a position table needs positions")
+        _i32(positions, "positions", n)
+    _lib.call("liyab_embed", out.data_ptr(), table.data_ptr(), _ptr(pos_table), dtype_code(table.dtype),
+              ids.data_ptr(), _ptr(positions), n, d, float(scale), _stream())
+
+
+def add_rows_(x: torch.Tensor, table: torch.Tensor, rows: torch.Tensor) -> None:
+    """x[t] += table[rows[t]]; x is float32 [n, d]."""
+    _dev(x, "x")
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("add_rows: x must be contiguous float32")
+    if table.dim() != 2 or table.shape[1] != d or not table.is_contiguous():
+        raise KernelError(f"add_rows: table {tuple(table.shape)} does not have rows of {d}")
+    _i32(rows, "rows", n)
+    _lib.call("liyab_add_rows", x.data_ptr(), table.data_ptr(), dtype_code(table.dtype), rows.data_ptr(), n, d, _stream())
+
+
+def layernorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+              eps: float, rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = LayerNorm(x[rows[r]] or x[r]); x float32 [*, d], out [n, d] float32 or bfloat16."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = out.shape
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError("layernorm: x must be contiguous float32 [*, d] and out contiguous [n, d]")
+    _f32vec(weight, "norm weight", d)
+    _f32vec(bias, "norm bias", d)
+    if rows is not None:
+        _i32(rows, "rows", n)
+    elif x.shape[0] < n:
+        raise KernelError("layernorm: fewer input rows than output rows")
+    _lib.call("liyab_layernorm", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
+              _ptr(rows), n, d, float(eps), _stream())
+
+
+def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
+                residual: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> None:
+    """out = epilogue(a . w^T + bias), or residual += a . w^T + bias.
+    a [M, K] and w [N, K] share a dtype; rows of a and out may be strided."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    if w.dim() != 2 or w.shape[1] != K or not w.is_contiguous() or w.dtype != a.dtype:
+        raise KernelError(f"gemm: w {tuple(w.shape)} {w.dtype} does not fit a {tuple(a.shape)} {a.dtype}")
+    N = w.shape[0]
+    _f32vec(bias, "bias", N)
+    ldo = ldr = 0
+    out_code = F32
+    if epilogue == EPI_RESIDUAL:
+        if residual is None or residual.dtype != torch.float32 or tuple(residual.shape) != (M, N):
+            raise KernelError("gemm: the residual epilogue needs a float32 residual [M, N]")
+        ldr = _rows(residual, "residual")
+    else:
+        if out is None or tuple(out.shape) != (M, N):
+            raise KernelError("gemm: out must be [M, N]")
+        ldo = _rows(out, "out")
+        out_code = dtype_code(out.dtype)
+    _lib.call("liyab_gemm_simple", _ptr(out), out_code, ldo, a.data_ptr(), lda, w.data_ptr(), dtype_code(a.dtype),
+              _ptr(bias), _ptr(residual), ldr, M, N, K, epilogue, _stream())
+
+
+def kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, src: torch.Tensor, k_off: int, v_off: int,
+             slots: torch.Tensor) -> None:
+    """Writes token t's keys src[t, k_off:k_off+Hkv*hd] and values to slot slots[t] of caches
+    laid out [pages, kv_heads, page_size, head_dim]. Slots are page * page_size + offset; the
+    caller has checked them against the cache's pages."""
+    _dev(k_cache, "k_cache")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("kv_write: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
+    if src.dtype != k_cache.dtype or v_cache.dtype != k_cache.dtype:
+        raise KernelError("kv_write: source and caches must share a dtype")
+    stride = _rows(src, "src")
+    n = src.shape[0]
+    _i32(slots, "slots", n)
+    _, hkv, page, hd = k_cache.shape
+    if k_off + hkv * hd > src.shape[1] or v_off + hkv * hd > src.shape[1]:
+        raise KernelError("kv_write: column offsets pass the source's width")
+    _lib.call("liyab_kv_write", k_cache.data_ptr(), v_cache.data_ptr(), src.data_ptr(), dtype_code(src.dtype), stride,
+              k_off, v_off, slots.data_ptr(), n, hkv, hd, page, _stream())
+
+
+def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
+                      scale: float, window: int = 0) -> None:
+    """out[t, h*hd:(h+1)*hd] = softmax(scale * q_th . K[:pos_t+1]) V for the request tok_seq[t].
+    q is [n, >= n_head*hd] (a view into a wider projection output is fine)."""
+    n = out.shape[0]
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
+    _, hkv, page, hd = k_cache.shape
+    os_ = _rows(out, "out")
+    qs = _rows(q, "q")
+    if q.shape[0] != n or q.shape[1] < n_head * hd or out.shape[1] != n_head * hd:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {n_head} heads of {hd}")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("attention: q, out and the caches must share a dtype")
+    _dev(block_tables, "block_tables")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
+    _i32(tok_seq, "tok_seq", n)
+    _i32(tok_pos, "tok_pos", n)
+    _lib.call("liyab_attention_generic", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
+              dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], tok_seq.data_ptr(),
+              tok_pos.data_ptr(), n, float(scale), int(window), n_head, hkv, hd, page, _stream())
+
+
+def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
+    ld = _rows(logits, "logits")
+    rows, V = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("argmax: logits must be float32")
+    _i32(out, "out", rows)
+    _lib.call("liyab_argmax", out.data_ptr(), logits.data_ptr(), ld, rows, V, _stream())
+
+
+def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+           top_p: torch.Tensor, uniform: torch.Tensor) -> None:
+    """Per-row sampling; temperature/top_p float32 [rows], top_k int32 [rows], uniform float64 [rows] in [0, 1)."""
+    ld = _rows(logits, "logits")
+    rows, V = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("sample: logits must be float32")
+    _i32(out, "out", rows)
+    _f32vec(temperature, "temperature", rows)
+    _f32vec(top_p, "top_p", rows)
+    _i32(top_k, "top_k", rows)
+    _dev(uniform, "uniform")
+    if uniform.dtype != torch.float64 or uniform.numel() != rows or not uniform.is_contiguous():
+        raise KernelError("sample: uniform must be contiguous float64 [rows]")
+    _lib.call("liyab_sample", out.data_ptr(), logits.data_ptr(), ld, rows, V, temperature.data_ptr(),
+              top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(), _stream())
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
+         residual: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> None:
+    """The product kernel for these operands: matrix cores for bfloat16 shapes they take,
+    the plain tiled kernel for float32 and everything else."""
+    gemm_simple(a, w, bias, out=out, residual=residual, epilogue=epilogue)
+
+
+def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0) -> None:
+    """Attention of the step's tokens over their requests' cached keys and values; the kernel
+    is chosen from the step's shape (`ctx` is the step's StepContext)."""
+    attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
+                      window=window)

@@ -1,0 +1,68 @@
+"""The attention mixer over paged keys and values."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..cache.pages import KVSpec
+from ..cache.storage import LayerCache
+from ..kernels import ops
+from .base import StepContext
+from .linear import linear
+from .registry import register_mixer
+
+
+class Attention:
+    """Causal self-attention with a fused, biased QKV projection and a biased
+    output projection: the reference's attention_mixer for a block with
+    `fused_qkv` (src/core/transformer.cpp:3083-3140). In order: qkv = h . Wqkv^T
+    + b split [q | k | v] (:2657-2673, bias :1263-1273); the step's keys and
+    values go to their cache slots before any score is computed, so a portion's
+    later tokens see its earlier ones through the cache (:3083-3128); scores,
+    softmax and weighted values over positions [0, pos] or the last `window`
+    (:2162-2453); out = att . Wo^T + bo added into the residual (:3139-3140,
+    :5647). Head counts, head size, scale and window are the spec's; queries
+    may outnumber key/value heads by a whole factor."""
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.spec = spec
+        self.dtype = dtype
+        self.width = spec.width
+        self.n_head, self.n_kv_head, self.head_dim = spec.n_head, spec.n_kv_head, spec.head_dim
+        if self.n_head % self.n_kv_head != 0:
+            raise ValueError(f"{self.n_head} query heads are no multiple of {self.n_kv_head} key/value heads")
+        self.scale = float(spec.scale)
+        self.window = int(spec.window)
+        self.q_dim = self.n_head * self.head_dim
+        self.kv_dim = self.n_kv_head * self.head_dim
+        qkv_out = self.q_dim + 2 * self.kv_dim
+        t = spec.tensors
+        self.qkv_weight = store.fetch(t["qkv_weight"], (qkv_out, self.width), "matrix")
+        self.qkv_bias = store.fetch(t["qkv_bias"], (qkv_out,), "vector") if "qkv_bias" in t else None
+        self.out_weight = store.fetch(t["out_weight"], (self.width, self.q_dim), "matrix")
+        self.out_bias = store.fetch(t["out_bias"], (self.width,), "vector") if "out_bias" in t else None
+
+    def cache_spec(self) -> Optional[KVSpec]:
+        return KVSpec(self.n_kv_head, self.head_dim, self.window)
+
+    def state_spec(self):
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache: LayerCache, state, residual: torch.Tensor,
+                writes_cache: bool = True) -> None:
+        n = h.shape[0]
+        ws = ctx.workspace
+        group = ctx.groups[cache.group]
+        qkv = ws.get("qkv", (n, self.q_dim + 2 * self.kv_dim), self.dtype)
+        linear(h, self.qkv_weight, self.qkv_bias, out=qkv)
+        if writes_cache:
+            ops.kv_write(cache.k, cache.v, qkv, self.q_dim, self.q_dim + self.kv_dim, group.slots)
+        att = ws.get("att", (n, self.q_dim), self.dtype)
+        ops.attention(att, qkv, cache.k, cache.v, group.block_tables, ctx, n_head=self.n_head, scale=self.scale,
+                      window=self.window)
+        linear(att, self.out_weight, self.out_bias, residual=residual)
+
+
+register_mixer("attention", Attention)

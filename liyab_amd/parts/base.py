@@ -1,0 +1,93 @@
+"""What every part sees of a step, and the interfaces parts implement.
+
+A step is a flat batch of tokens of several requests (the reference's
+`Segment` list flattened: src/core/transformer.h:890-902, rows concatenated
+in src/core/transformer.cpp:6689-6693). `StepContext` carries, per token,
+its request and position, per request its block table and state slot, and
+the rows whose logits are wanted. Parts read what they need from it; none
+knows which model it is in or what else the batch holds.
+
+Interfaces (duck-typed; the registries in `registry.py` map a spec's `kind`
+to a class constructed as `cls(spec, store, dtype)`):
+
+  norm:      forward(x_f32 [n, d], ctx, rows=None) -> [n or len(rows), d] in the compute dtype
+  mixer:     cache_spec() -> KVSpec | None;  state_spec() -> StateSpec | None
+             forward(h, ctx, cache, state, residual, writes_cache=True): adds its output into `residual`
+  ffn:       forward(h, ctx, residual): adds its output into `residual`
+  position:  where == "residual": add(ctx, x);  fused_table() -> table | None
+  block:     cls(layer_spec, mixer, ffn, norm_mixer, norm_ffn); forward(x, ctx, cache, state, writes_cache)
+
+`residual` is the float32 residual stream [n, d]; a part adds into it in
+place (the sum is 32-bit whatever the compute dtype), which lets an output
+projection fold the addition into its epilogue.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers that keep their addresses from step to step."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = f"{name}/{dtype}"
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            cap = max(n, 1)
+            if buf is not None:
+                cap = max(cap, 2 * buf.numel())
+            buf = torch.empty(cap, dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:n].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+@dataclass
+class GroupStep:
+    """A cache group's view of the step."""
+
+    block_tables: torch.Tensor  # int32 [n_seqs, max_blocks]; -1 where unmapped
+    slots: torch.Tensor  # int32 [n_tokens]: page * page_size + offset of each token
+
+
+@dataclass
+class StepHost:
+    """The same facts on the host, for choosing kernels and grids."""
+
+    q_lens: List[int]  # tokens of each request in this step
+    starts: List[int]  # row of each request's first token
+    first_pos: List[int]  # position of each request's first token
+    max_q_len: int
+    max_context: int  # longest context after this step
+
+
+@dataclass
+class StepContext:
+    n_tokens: int
+    n_seqs: int
+    token_ids: torch.Tensor  # int32 [n_tokens]
+    positions: torch.Tensor  # int32 [n_tokens]
+    tok_seq: torch.Tensor  # int32 [n_tokens]: index of the token's request in this step
+    seq_starts: torch.Tensor  # int32 [n_seqs + 1]
+    context_lens: torch.Tensor  # int32 [n_seqs]: positions each request holds after this step
+    state_slots: torch.Tensor  # int32 [n_seqs]
+    logit_rows: torch.Tensor  # int32 [n_rows]
+    n_logit_rows: int
+    groups: List[GroupStep]
+    host: StepHost
+    workspace: Workspace
+    dtype: torch.dtype
+    page_size: int

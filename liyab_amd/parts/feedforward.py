@@ -1,0 +1,35 @@
+"""Feed-forward parts."""
+
+from __future__ import annotations
+
+import torch
+
+from .base import StepContext
+from .linear import linear
+from .registry import register_ffn
+
+
+class DenseFFN:
+    """The ungated feed-forward: m = act(h . Wup^T + b_up) . Wdown^T + b_down,
+    added into the residual (the reference's dense_ffn for FfnKind::Ungated,
+    src/core/transformer.cpp:4903-4913; residual :5692). `activation` is
+    "gelu_tanh" (:123-130) or "gelu_erf" (:134-142)."""
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.dtype = dtype
+        self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
+        if self.activation not in ("gelu_tanh", "gelu_erf"):
+            raise ValueError(f"unknown activation '{self.activation}'")
+        t = spec.tensors
+        self.up_weight = store.fetch(t["up_weight"], (self.inner, self.width), "matrix")
+        self.up_bias = store.fetch(t["up_bias"], (self.inner,), "vector") if "up_bias" in t else None
+        self.down_weight = store.fetch(t["down_weight"], (self.width, self.inner), "matrix")
+        self.down_bias = store.fetch(t["down_bias"], (self.width,), "vector") if "down_bias" in t else None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, residual: torch.Tensor) -> None:
+        inner = ctx.workspace.get("ffn_inner", (h.shape[0], self.inner), self.dtype)
+        linear(h, self.up_weight, self.up_bias, out=inner, activation=self.activation)
+        linear(inner, self.down_weight, self.down_bias, residual=residual)
+
+
+register_ffn("dense_ffn", DenseFFN)

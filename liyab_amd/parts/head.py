@@ -1,0 +1,34 @@
+"""The output head."""
+
+from __future__ import annotations
+
+import torch
+
+from .base import StepContext
+from .linear import linear
+from .registry import register_head
+
+
+class LMHead:
+    """logits = h . W^T (+ bias), times logit_scale when it is not 1: the
+    reference's compute_logits after the final norm (src/core/transformer.cpp:2622-2638,
+    finish_logits :2613-2620). W may be the token embedding's table (a tied
+    head, :1100-1104): the store hands out the same device tensor for the same
+    name, so a tied table is resident once. Logits are float32."""
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.width, self.vocab_size = spec.width, spec.vocab_size
+        self.logit_scale = float(spec.logit_scale)
+        if self.logit_scale != 1.0:
+            raise NotImplementedError("a logit scale other than 1 is not implemented")
+        t = spec.tensors
+        self.weight = store.fetch(t["weight"], (self.vocab_size, self.width), "table")
+        self.bias = store.fetch(t["bias"], (self.vocab_size,), "vector") if "bias" in t else None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        logits = ctx.workspace.get("logits", (h.shape[0], self.vocab_size), torch.float32)
+        linear(h, self.weight, self.bias, out=logits)
+        return logits
+
+
+register_head("lm_head", LMHead)
