@@ -12,4 +12,15 @@ from .errors import (  # noqa: F401
     Unsupported,
 )
 
+from .sampling import SamplingParams  # noqa: F401
+
 __version__ = "0.1.0"
+
+
+def __getattr__(name):
+    # the engine needs torch and the GPU library: import it on first use
+    if name in ("Engine", "EngineCore", "StepItem", "GenerationResult", "GenerationStats"):
+        from . import engine
+
+        return getattr(engine, name)
+    raise AttributeError(name)

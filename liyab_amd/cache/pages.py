@@ -180,12 +180,20 @@ class CacheManager:
         r = self._requests[rid]
         return [max(0, self._pages_for(new_length) - len(t)) for t in r.tables]
 
-    def can_reserve(self, wants: Sequence[Tuple[Hashable, int]]) -> bool:
+    def can_reserve(self, wants: Sequence[Tuple[Hashable, int]], new_lengths: Sequence[int] = ()) -> bool:
+        """Whether `reserve(wants)` would succeed, with requests that are not
+        open yet and would come to hold `new_lengths` positions counted in."""
         need = [0] * len(self.groups)
         for rid, new_length in wants:
             for gi, n in enumerate(self.pages_needed(rid, new_length)):
                 need[gi] += n
+        for length in new_lengths:
+            for gi in range(len(self.groups)):
+                need[gi] += self._pages_for(length)
         return all(n <= g.pool.free_pages for n, g in zip(need, self.groups))
+
+    def free_slots(self) -> int:
+        return len(self._free_slots)
 
     def reserve(self, wants: Sequence[Tuple[Hashable, int]]) -> None:
         """Maps pages so that each request can hold `new_length` positions.

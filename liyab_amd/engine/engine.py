@@ -1,0 +1,180 @@
+"""The engine: requests in, tokens out.
+
+The Python entry point, in the manner of the reference's C++ `Engine`
+(include/liyab/engine.h:634-1052): `Engine(model, ...)` for `Engine::create`,
+`generate(prompt ids, SamplingParams, on_token)` for `generate_tokens`
+(src/core/engine.cpp:3804-3810), statistics named as `GenerationStats`
+(include/liyab/types.h:238-292: prompt_tokens, prefill_ms, ttft_ms,
+generated_tokens, decode_ms, tokens_per_second, kv_cache_bytes). Where the
+reference runs each open sequence on its caller's thread, this engine is
+one loop: `add_request` any number of prompts, then `step()` until none is
+unfinished; `generate` does that for one or several prompts.
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
+
+from ..errors import InvalidArgument
+from ..sampling import Sampler, SamplingParams
+from .core import EngineCore
+from .scheduler import Request, Scheduled, Scheduler
+from .step import StepItem
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    prefill_ms: float = 0.0
+    ttft_ms: float = 0.0
+    generated_tokens: int = 0
+    decode_ms: float = 0.0
+    tokens_per_second: float = 0.0
+    kv_cache_bytes: int = 0
+    preemptions: int = 0
+
+
+@dataclass
+class GenerationResult:
+    rid: Hashable
+    prompt: List[int]
+    tokens: List[int]
+    finish_reason: Optional[str]
+    stats: GenerationStats = field(default_factory=GenerationStats)
+
+
+class Engine:
+    def __init__(self, model: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
+                 num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_num_seqs: int = 64,
+                 max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None):
+        """`model`: a folder with config.json and model.safetensors. `ctx`: the
+        context length (default: the model's). `prefill_chunk`: the longest
+        portion of a prompt in one step (the reference's 256,
+        src/core/engine.cpp:2863-2864). `num_pages` / `max_tokens` size the
+        page pool."""
+        self.core = EngineCore(model, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
+                               max_tokens=max_tokens, max_requests=max_num_seqs, context_length=ctx)
+        self.scheduler = Scheduler(self.core.manager, max_num_seqs=max_num_seqs,
+                                   max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
+                                   eos_token_id=self.core.model.plan.eos_token_id, on_open=self._reset_slot)
+        self.sampler = Sampler(self.core.device)
+        self._requests: Dict[Hashable, Request] = {}
+        self._t_first: Dict[Hashable, float] = {}
+        self._t_start: Dict[Hashable, float] = {}
+        self._t_end: Dict[Hashable, float] = {}
+        self._next_id = 0
+        self.stop_at_eos = True
+
+    # -- plumbing ---------------------------------------------------------------
+    def _reset_slot(self, rid: Hashable) -> None:
+        if self.core.storage.states:
+            self.core.storage.reset_slot(self.core.manager.slot(rid))
+
+    @property
+    def config(self):
+        return self.core.config
+
+    # -- continuous batching ------------------------------------------------------
+    def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    rid: Optional[Hashable] = None) -> Hashable:
+        params = params or SamplingParams()
+        prompt = [int(t) for t in prompt_ids]
+        V = self.core.vocab_size
+        for t in prompt:
+            if not (0 <= t < V):
+                raise InvalidArgument(f"token id {t} is outside [0, {V})")  # src/core/transformer.cpp:6195-6197
+        if rid is None:
+            rid = f"req-{self._next_id}"
+            self._next_id += 1
+        if rid in self._requests and self._requests[rid].state != "finished":
+            raise InvalidArgument(f"request {rid!r} is still running")
+        r = Request(rid=rid, prompt=prompt, params=params, seed=params.resolved_seed())
+        self.scheduler.add(r)
+        self._requests[rid] = r
+        self._t_start[rid] = time.perf_counter()
+        return rid
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    def step(self, on_token: Optional[Callable[[Hashable, int], Optional[bool]]] = None) -> List[Request]:
+        """One scheduler iteration: a batch, a model step, sampling. Returns the
+        requests that finished in it."""
+        batch = self.scheduler.schedule()
+        if not batch:
+            return []
+        items = []
+        for s in batch:
+            toks = s.request.tokens[s.first:s.first + s.count]
+            items.append(StepItem(s.request.rid, toks, [s.count - 1] if s.wants_logits else []))
+        logits = self.core.step(items)
+        sampled: Dict[Hashable, int] = {}
+        wanting = [s.request for s in batch if s.wants_logits]
+        if wanting:
+            tokens = self.sampler.sample(logits, [r.params for r in wanting], [r.seed for r in wanting],
+                                         [len(r.generated) for r in wanting])
+            now = time.perf_counter()
+            for r, t in zip(wanting, tokens):
+                sampled[r.rid] = int(t)
+                if not r.generated:
+                    self._t_first.setdefault(r.rid, now)
+        cb = None
+        if on_token is not None:
+            cb = lambda r, t: on_token(r.rid, t)  # noqa: E731
+        if not self.stop_at_eos:
+            saved, self.scheduler.eos_token_id = self.scheduler.eos_token_id, None
+            done = self.scheduler.update(batch, sampled, cb)
+            self.scheduler.eos_token_id = saved
+        else:
+            done = self.scheduler.update(batch, sampled, cb)
+        now = time.perf_counter()
+        for r in done:
+            self._t_end[r.rid] = now
+        return done
+
+    def abort(self, rid: Hashable) -> None:
+        r = self._requests.get(rid)
+        if r is not None and r.state != "finished":
+            self.scheduler.finish(r, "cancelled")
+
+    def result(self, rid: Hashable) -> GenerationResult:
+        r = self._requests[rid]
+        end = time.perf_counter()
+        t0 = self._t_start.get(rid, end)
+        t1 = self._t_first.get(rid, end)
+        st = GenerationStats(prompt_tokens=len(r.prompt), generated_tokens=len(r.generated),
+                             prefill_ms=(t1 - t0) * 1e3, ttft_ms=(t1 - t0) * 1e3,
+                             decode_ms=(self._t_end.get(rid, end) - t1) * 1e3,
+                             kv_cache_bytes=self.core.storage.bytes_per_token() * (r.n_tokens - 1),
+                             preemptions=r.preemptions)
+        if st.decode_ms > 0 and st.generated_tokens > 1:
+            # the reference's generated * 1000 / decode_ms (src/core/engine.cpp:4447-4448), over the
+            # tokens that decoding steps produced (the first comes out of the prompt's last portion)
+            st.tokens_per_second = (st.generated_tokens - 1) * 1000.0 / st.decode_ms
+        return GenerationResult(rid=rid, prompt=r.prompt, tokens=list(r.generated), finish_reason=r.finish_reason,
+                                stats=st)
+
+    # -- generation ---------------------------------------------------------------
+    def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 on_token: Optional[Callable[[Hashable, int], Optional[bool]]] = None):
+        """Generates for one prompt (a list of ids -> one GenerationResult) or
+        several (a list of lists -> a list of results, batched continuously).
+        `on_token(rid, token)` returning False stops that request."""
+        single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
+        plist = [prompts] if single else list(prompts)
+        if not plist:
+            raise InvalidArgument("no prompt was given")
+        if params is None or isinstance(params, SamplingParams):
+            params_list = [params or SamplingParams()] * len(plist)
+        else:
+            params_list = list(params)
+            if len(params_list) != len(plist):
+                raise InvalidArgument("one SamplingParams per prompt is needed")
+        rids = [self.add_request(p, sp) for p, sp in zip(plist, params_list)]
+        while any(self._requests[r].state != "finished" for r in rids):
+            self.step(on_token)
+        results = [self.result(r) for r in rids]
+        return results[0] if single else results

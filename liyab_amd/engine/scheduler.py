@@ -1,0 +1,232 @@
+"""The scheduler: admission, prompt portions under a token budget, decoding,
+finishing, and what happens when pages run out.
+
+The reference schedules by threads: each generating thread submits the pass
+it needs and one of them runs the merged batch (src/core/engine.cpp:1842-2041);
+prompts go in portions of 256 tokens (:2863-2864), a decoding request brings
+one token a pass (:4311-4334), and a request stops at an end-of-generation
+token, at max_tokens or on its callback's word (:4351-4393). When the cache
+cannot grow the reference fails the request (src/core/kv_cache.cpp:249-252,
+src/core/engine.cpp:3878-3882). Here one loop owns all requests:
+
+  * every step first gives each decoding request its one token, then hands
+    the rest of the token budget to prompt portions in order of admission
+    (a portion is as small as the budget leaves, down to one token), then
+    admits waiting requests first come, first served, while a request slot,
+    budget and pages for the first portion are there;
+  * when a request cannot get its pages, the most recently admitted running
+    request is preempted: its pages and slot go back, it returns to the head
+    of the waiting queue and is recomputed from its prompt plus what it has
+    generated. A request is never preempted for its own sake by a later one,
+    and a request that could not fit the pool alone is refused on arrival.
+
+The scheduler decides on the host from the cache manager's counts only; it
+runs nothing on the GPU and is tested without one.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..cache.pages import CacheManager
+from ..errors import InvalidArgument, OutOfPages
+from ..sampling import SamplingParams
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    seed: int = 0
+    generated: List[int] = field(default_factory=list)
+    computed: int = 0  # tokens of prompt + generated that are in the cache
+    state: str = WAITING
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    arrival: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.generated
+
+    @property
+    def n_tokens(self) -> int:
+        return len(self.prompt) + len(self.generated)
+
+    @property
+    def remaining(self) -> int:
+        return self.n_tokens - self.computed
+
+
+@dataclass
+class Scheduled:
+    request: Request
+    first: int  # index of the first token run in this step
+    count: int  # how many tokens
+    wants_logits: bool  # the portion reaches the request's last token
+
+
+@dataclass
+class SchedulerStats:
+    steps: int = 0
+    batched_tokens: int = 0
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    preemptions: int = 0
+    pages_in_use_peak: int = 0
+
+
+class Scheduler:
+    def __init__(self, manager: CacheManager, *, max_num_seqs: int, max_batched_tokens: int, prefill_chunk: int,
+                 eos_token_id: Optional[int] = None, on_open: Optional[Callable[[Hashable], None]] = None):
+        if max_num_seqs <= 0 or max_batched_tokens <= 0 or prefill_chunk <= 0:
+            raise InvalidArgument("max_num_seqs, max_batched_tokens and prefill_chunk must be positive")
+        self.manager = manager
+        self.max_num_seqs = min(max_num_seqs, manager.max_requests)
+        self.max_batched_tokens = max_batched_tokens
+        self.prefill_chunk = prefill_chunk
+        self.eos_token_id = eos_token_id
+        self.on_open = on_open
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []
+        self.stats = SchedulerStats()
+        self._arrivals = 0
+
+    # -- arrival --------------------------------------------------------------
+    def add(self, request: Request) -> None:
+        if not request.prompt:
+            raise InvalidArgument("the prompt is empty")  # src/core/engine.cpp:3867-3871
+        if request.params.max_tokens <= 0:
+            raise InvalidArgument("max_tokens must be positive")
+        if len(request.prompt) >= self.manager.max_positions + 1:
+            raise InvalidArgument(
+                f"the prompt has {len(request.prompt)} tokens; the context holds {self.manager.max_positions}")
+        # the most positions it can come to hold: every token but the last sampled one is run
+        most = min(len(request.prompt) + request.params.max_tokens - 1, self.manager.max_positions)
+        need = -(-most // self.manager.page_size)
+        for g in self.manager.groups:
+            if g.spec.window <= 0 and need > g.pool.num_pages:
+                raise OutOfPages(
+                    f"request {request.rid!r} may need {need} pages; the pool has {g.pool.num_pages} in all")
+        request.state = WAITING
+        request.arrival = self._arrivals
+        self._arrivals += 1
+        self.waiting.append(request)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # -- one step's decisions ---------------------------------------------------
+    def _open(self, r: Request) -> None:
+        self.manager.open(r.rid)
+        if self.on_open is not None:
+            self.on_open(r.rid)
+
+    def _preempt(self, r: Request) -> None:
+        self.manager.close(r.rid)
+        self.running.remove(r)
+        r.computed = 0
+        r.state = WAITING
+        r.preemptions += 1
+        self.stats.preemptions += 1
+        self.waiting.appendleft(r)
+
+    def schedule(self) -> List[Scheduled]:
+        """Chooses this step's batch and opens/preempts requests accordingly.
+        Pages are only counted here; the step function maps them."""
+        budget = self.max_batched_tokens
+        batch: List[Scheduled] = []
+        wants: List = []
+
+        def fits(r: Request, count: int) -> bool:
+            return self.manager.can_reserve(wants + [(r.rid, r.computed + count)])
+
+        def take(r: Request, count: int) -> None:
+            nonlocal budget
+            batch.append(Scheduled(r, r.computed, count, r.computed + count == r.n_tokens))
+            wants.append((r.rid, r.computed + count))
+            budget -= count
+
+        # running requests: decoding ones first, then prompt portions, each in order of admission
+        order = [r for r in self.running if r.remaining == 1] + [r for r in self.running if r.remaining > 1]
+        for r in order:
+            if r.state != RUNNING or budget <= 0:
+                continue
+            count = min(r.remaining, self.prefill_chunk, budget)
+            while not fits(r, count):
+                victim = self.running[-1]
+                if victim is r:
+                    # nobody later to take pages from: shrink the portion or wait
+                    while count > 1 and not fits(r, count):
+                        count -= 1
+                    if not fits(r, count):
+                        count = 0
+                    break
+                for s in [s for s in batch if s.request is victim]:
+                    batch.remove(s)
+                    wants.remove((victim.rid, victim.computed + s.count))
+                    budget += s.count
+                self._preempt(victim)
+            if count > 0 and r.state == RUNNING:
+                take(r, count)
+        # admission, first come first served
+        while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
+            r = self.waiting[0]
+            count = min(r.remaining, self.prefill_chunk, budget)
+            if self.manager.free_slots() == 0 or not self.manager.can_reserve(wants, new_lengths=[count]):
+                break
+            self._open(r)
+            self.waiting.popleft()
+            r.state = RUNNING
+            self.running.append(r)
+            take(r, count)
+        if not batch and self.has_unfinished():
+            raise OutOfPages("no request can make progress: the page pool is too small for any of them")
+        self.stats.steps += 1
+        n = sum(s.count for s in batch)
+        self.stats.batched_tokens += n
+        self.stats.decode_tokens += sum(1 for s in batch if s.count == 1 and s.wants_logits and s.request.generated)
+        self.stats.prefill_tokens = self.stats.batched_tokens - self.stats.decode_tokens
+        return batch
+
+    # -- after the step -----------------------------------------------------------
+    def update(self, batch: Sequence[Scheduled], sampled: Dict[Hashable, int],
+               on_token: Optional[Callable[[Request, int], bool]] = None) -> List[Request]:
+        """Records what the step computed and sampled; returns requests that finished."""
+        done = []
+        for s in batch:
+            r = s.request
+            r.computed += s.count
+            if not s.wants_logits:
+                continue
+            token = sampled[r.rid]
+            r.generated.append(token)
+            reason = None
+            if self.eos_token_id is not None and token == self.eos_token_id:
+                reason = "stop"
+            elif len(r.generated) >= r.params.max_tokens:
+                reason = "length"
+            elif r.n_tokens > self.manager.max_positions:
+                reason = "context"  # the next token would pass the last position
+            if on_token is not None and on_token(r, token) is False and reason is None:
+                reason = "callback"
+            if reason is not None:
+                self.finish(r, reason)
+                done.append(r)
+        self.stats.pages_in_use_peak = max(self.stats.pages_in_use_peak,
+                                           max((g.pool.peak_in_use for g in self.manager.groups), default=0))
+        return done
+
+    def finish(self, r: Request, reason: str) -> None:
+        if r.state == RUNNING:
+            self.manager.close(r.rid)
+            self.running.remove(r)
+        elif r.state == WAITING:
+            self.waiting.remove(r)
+        r.state = FINISHED
+        r.finish_reason = reason

@@ -1,0 +1,97 @@
+"""Sampling parameters, the per-token random numbers, and the device sampler.
+
+Parameters and their defaults are the reference's `SamplingParams`
+(include/liyab/types.h:215-222): temperature 0.8 (<= 0 is greedy), top_k 40
+(<= 0 off), top_p 0.95 (>= 1 off), seed 0 = pick one at random, max_tokens
+256. The order temperature -> top-k -> top-p -> renormalise -> draw is the
+reference's (src/core/sampling.cpp:16-79) and runs in the sampling kernel.
+
+The reference gives each generation its own `mt19937_64` (src/core/engine.cpp:3893),
+which makes a request's draws independent of what else runs. Here the same
+property comes from a counter-based generator: the uniform number for a
+request's k-th generated token is a pure function of (seed, k), so it is
+also the same after a preemption and recompute.
+"""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+_MASK = (1 << 64) - 1
+
+
+@dataclass
+class SamplingParams:
+    temperature: float = 0.8
+    top_k: int = 40
+    top_p: float = 0.95
+    seed: int = 0
+    max_tokens: int = 256
+
+    @property
+    def greedy(self) -> bool:
+        return not (self.temperature > 0.0)
+
+    def resolved_seed(self) -> int:
+        """The seed in use: a fresh random one when `seed` is 0."""
+        if self.seed != 0:
+            return self.seed & _MASK
+        return int.from_bytes(os.urandom(8), "little") | 1
+
+
+def uniform(seed: int, index: int) -> float:
+    """A number in [0, 1) for token `index` of a request with `seed`:
+    splitmix64's output function over a counter, top 53 bits."""
+    z = (seed * 0x9E3779B97F4A7C15 + (index + 1) * 0xD1B54A32D192ED03) & _MASK
+    z = (z + 0x9E3779B97F4A7C15) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    z ^= z >> 31
+    return (z >> 11) * (1.0 / (1 << 53))
+
+
+class Sampler:
+    """Samples one token per logits row on the device."""
+
+    def __init__(self, device):
+        import torch
+
+        self.device = torch.device(device)
+        self._cap = 0
+
+    def _buffers(self, rows: int):
+        import torch
+
+        if rows > self._cap:
+            cap = max(rows, 64, 2 * self._cap)
+            self._out = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self._temp = torch.empty(cap, dtype=torch.float32, device=self.device)
+            self._topk = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self._topp = torch.empty(cap, dtype=torch.float32, device=self.device)
+            self._u = torch.empty(cap, dtype=torch.float64, device=self.device)
+            self._cap = cap
+
+    def sample(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int]) -> List[int]:
+        """One token per row of `logits` [rows, vocab] (float32, device).
+        `seeds[r]` is row r's resolved seed and `indices[r]` how many tokens
+        its request has generated so far."""
+        import torch
+
+        from ..kernels import ops
+
+        rows = logits.shape[0]
+        if not (len(params) == len(seeds) == len(indices) == rows):
+            raise ValueError("one SamplingParams, seed and index per logits row is needed")
+        self._buffers(rows)
+        out = self._out[:rows]
+        if all(p.greedy for p in params):
+            ops.argmax(out, logits)
+        else:
+            self._temp[:rows].copy_(torch.tensor([float(p.temperature) for p in params], dtype=torch.float32))
+            self._topk[:rows].copy_(torch.tensor([int(p.top_k) for p in params], dtype=torch.int32))
+            self._topp[:rows].copy_(torch.tensor([float(p.top_p) for p in params], dtype=torch.float32))
+            self._u[:rows].copy_(torch.tensor([uniform(s, i) for s, i in zip(seeds, indices)], dtype=torch.float64))
+            ops.sample(out, logits, self._temp[:rows], self._topk[:rows], self._topp[:rows], self._u[:rows])
+        return out.tolist()

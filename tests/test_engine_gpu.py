@@ -1,0 +1,285 @@
+"""The engine against the plain implementation, under every way of cutting and batching the
+work, in 32-bit and in bfloat16 (needs the GPU)."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_gpt2 as plain
+import trace_tools as tt
+from conftest import CONFIGS, ROOT, TOL
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+
+def make_requests(name):
+    """Token sequences of the workloads: prompt + continuation, teacher-forced."""
+    cfg, _ = CONFIGS[name]
+    V, P = cfg["vocab_size"], cfg["n_positions"]
+    if name == "A":
+        lens = {"a0": 7 + 24, "a1": 19 + 24, "a2": 1 + 24, "a3": P, "a4": 70}
+        seed = 1
+    else:
+        lens = {"b0": 1 + 32, "b1": 13 + 32, "b2": 64 + 32, "b3": 100 + 32, "b4": 200 + 32, "b5": P}
+        seed = 3
+    reqs = {}
+    for i, (rid, n) in enumerate(lens.items()):
+        reqs[rid] = tt.random_tokens(seed * 100 + i, n, V) if i != 4 else tt.stream_tokens(seed, n, V)
+    return reqs
+
+
+@pytest.fixture(scope="module")
+def reference(plain_models):
+    """{(model, dtype): {rid: logits [T, V]}} from the plain implementation. The bfloat16 path
+    holds its matrices in bfloat16, so its reference uses the matrices rounded the same way."""
+    out = {}
+    for name in ("A", "B"):
+        config, tensors = plain_models[name]
+        reqs = make_requests(name)
+        out[(name, "float32")] = {rid: plain.forward(config, tensors, toks) for rid, toks in reqs.items()}
+        rounded = plain.round_weights_to_bf16(tensors)
+        out[(name, "bfloat16")] = {rid: plain.forward(config, rounded, toks) for rid, toks in reqs.items()}
+    return out
+
+
+def make_core(model_dir, dtype, max_tokens, page_size=16, poison=True):
+    import torch
+
+    from liyab_amd.engine import EngineCore
+
+    core = EngineCore(model_dir, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8)
+    if poison:  # free pages hold NaN: a kernel that reads past a request's length shows it
+        for c in core.storage.layers.values():
+            c.k.fill_(float("nan"))
+            c.v.fill_(float("nan"))
+        torch.cuda.synchronize()
+    return core
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_each_request_alone_and_whole(name, dtype, model_dirs, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_whole(reqs)
+    core = make_core(model_dirs[name], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    for rid, toks in reqs.items():
+        assert sorted(got[rid]) == list(range(len(toks)))
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"whole {name} {dtype}")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_bulk_then_last_32_one_by_one(name, dtype, model_dirs, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_bulk_tail(reqs, tail=32)
+    core = make_core(model_dirs[name], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"bulk+tail {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("sizes", [(5,), (48,), (5, 2, 17, 3, 48, 2, 31, 7)])
+def test_portions_of_changing_size(name, dtype, sizes, model_dirs, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_portions(reqs, sizes)
+    core = make_core(model_dirs[name], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"portions {sizes} {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_mixed_batches_with_pages_used_again(name, dtype, seed, model_dirs, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_mixed(reqs, seed=seed)
+    assert any(len(st["entries"]) >= 2 for st in steps), "no step held several requests"
+    assert any(len(st["entries"]) >= 2 and {len(t) for _, t, _ in st["entries"]} > {1} and
+               any(len(t) == 1 for _, t, _ in st["entries"]) for st in steps), "no step mixed a portion with a single token"
+    most = tt.max_live_tokens(steps)
+    total = sum(-(-len(t) // 64) * 64 for t in reqs.values())
+    assert most < total, "the pool would hold every request at once: no page would be used again"
+    core = make_core(model_dirs[name], dtype, most)
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"mixed {name} {dtype}")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding_from_the_first_token(name, dtype, model_dirs, reference):
+    """Every token of the longest request one by one, from position 0 to the last position."""
+    reqs = make_requests(name)
+    rid = "a3" if name == "A" else "b5"
+    one = {rid: reqs[rid]}
+    steps = tt.schedule_bulk_tail(one, tail=len(one[rid]))
+    core = make_core(model_dirs[name], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, one, reference[(name, dtype)], TOL[dtype], f"decode all {name} {dtype}")
+    # the first tokens of a sequence: position 0 attends to itself only
+    assert sorted(got[rid])[:4] == [0, 1, 2, 3]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_context_full_and_bad_ids(dtype, model_dirs):
+    from liyab_amd import ContextFull, InvalidArgument
+    from liyab_amd.engine import StepItem
+
+    cfg, _ = CONFIGS["A"]
+    core = make_core(model_dirs["A"], dtype, 256)
+    core.open("x")
+    core.step([StepItem("x", [1] * cfg["n_positions"], [])])
+    with pytest.raises(ContextFull):
+        core.step([StepItem("x", [1], [0])])
+    core.open("y")
+    with pytest.raises(InvalidArgument):
+        core.step([StepItem("y", [cfg["vocab_size"]], [0])])
+    with pytest.raises(InvalidArgument):
+        core.step([StepItem("y", [], [])])
+    with pytest.raises(InvalidArgument):
+        core.step([StepItem("y", [1], [0]), StepItem("y", [2], [0])])
+    assert core.length("y") == 0
+
+
+def test_out_of_pages_changes_nothing(model_dirs):
+    from liyab_amd import OutOfPages
+    from liyab_amd.engine import StepItem
+
+    core = make_core(model_dirs["A"], "float32", 64)  # 4 pages of 16
+    core.open("x")
+    core.open("y")
+    core.step([StepItem("x", [1] * 40, [])])
+    before = core.manager.pages_in_use()
+    with pytest.raises(OutOfPages):
+        core.step([StepItem("x", [2], [0]), StepItem("y", [3] * 20, [])])
+    assert core.manager.pages_in_use() == before and core.length("x") == 40 and core.length("y") == 0
+    core.manager.check()
+
+
+def test_truncate_and_replay_gives_the_same_logits(model_dirs, plain_models):
+    """The reference's rollback check: 70 tokens, back to 65, the last 5 again
+    (tests/test_engine.cpp:3740-3741, 3764-3767)."""
+    cfg, _ = CONFIGS["B"]
+    toks = [3 + (i * 37) % 280 for i in range(70)]
+    core = make_core(model_dirs["B"], "float32", 128)
+    from liyab_amd.engine import StepItem
+
+    core.open("r")
+    first = core.step([StepItem("r", toks, list(range(70)))]).cpu().numpy().copy()
+    core.truncate("r", 65)
+    again = core.step([StepItem("r", toks[65:], list(range(5)))]).cpu().numpy()
+    assert tt.rel_err(again, first[65:]) <= TOL["float32"]
+    config, tensors = plain_models["B"]
+    assert tt.rel_err(first, plain.forward(config, tensors, toks)) <= TOL["float32"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_program_mixed(dtype, model_dirs, reference, tmp_path):
+    """bin/trace_run as a user runs it: a mixed trace with few pages, its files compared."""
+    name = "B"
+    cfg, _ = CONFIGS[name]
+    reqs = make_requests(name)
+    steps = tt.schedule_mixed(reqs, seed=2)
+    # some steps want nothing, some want a few places
+    for st in steps[::3]:
+        st["entries"] = [(rid, toks, want[-1:]) for rid, toks, want in st["entries"]]
+    steps[1]["entries"] = [(rid, toks, []) for rid, toks, want in steps[1]["entries"]]
+    got = tt.run_trace_program(model_dirs[name], dtype, steps, str(tmp_path / "out"), tt.max_live_tokens(steps),
+                               cfg["vocab_size"])
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"trace_run {dtype}")
+
+
+def _near_argmax(ref_row, token, tol):
+    ref_row = np.asarray(ref_row, dtype=np.float64)
+    return ref_row[token] >= ref_row.max() - tol * np.abs(ref_row).max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(name, dtype, model_dirs, plain_models):
+    """Engine.generate with several prompts batched continuously; each token is the plain
+    implementation's greedy choice given the tokens so far (or within tolerance of it)."""
+    from liyab_amd import Engine, SamplingParams
+
+    cfg, _ = CONFIGS[name]
+    config, tensors = plain_models[name]
+    if dtype == "bfloat16":
+        tensors = plain.round_weights_to_bf16(tensors)
+    V = cfg["vocab_size"]
+    n_new = 24 if name == "A" else 32
+    lens = [7, 19, 1] if name == "A" else [1, 13, 64, 100, 200]
+    prompts = [tt.random_tokens(40 + i, n, V) for i, n in enumerate(lens)]
+    engine = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=40, max_num_seqs=4, max_batched_tokens=64,
+                    prefill_chunk=5 if name == "A" else 48)
+    engine.stop_at_eos = False
+    results = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new))
+    for prompt, res in zip(prompts, results):
+        want_n = min(n_new, cfg["n_positions"] - len(prompt) + 1)
+        assert len(res.tokens) == want_n and res.finish_reason in ("length", "context")
+        ref = plain.forward(config, tensors, prompt + res.tokens[:-1])
+        for i, t in enumerate(res.tokens):
+            row = ref[len(prompt) - 1 + i]
+            assert _near_argmax(row, t, TOL[dtype]), f"token {i} of prompt length {len(prompt)}: {t} vs {int(np.argmax(row))}"
+        if dtype == "float32":
+            assert res.tokens == plain.generate_greedy(config, tensors, prompt, n_new)
+    assert engine.core.manager.pages_in_use() == 0
+    engine.core.manager.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_temperature_sampling_alone_and_batched(dtype, model_dirs, plain_models):
+    """Temperature 0.8, sampler seed 4: the same tokens alone and in a batch, and each the
+    plain sampler's draw from the plain logits (unless the draw falls on a boundary)."""
+    from liyab_amd import Engine, SamplingParams
+
+    name = "B"
+    cfg, _ = CONFIGS[name]
+    config, tensors = plain_models[name]
+    V = cfg["vocab_size"]
+    prompts = [tt.random_tokens(60 + i, n, V) for i, n in enumerate([1, 13, 64])]
+    sp = SamplingParams(temperature=0.8, top_k=0, top_p=1.0, seed=4, max_tokens=32)
+    engine = Engine(model_dirs[name], dtype=dtype, page_size=16, max_num_seqs=4, max_batched_tokens=64, prefill_chunk=48)
+    engine.stop_at_eos = False
+    together = engine.generate(prompts, sp)
+    alone = [engine.generate(p, sp) for p in prompts]
+    for a, b in zip(together, alone):
+        assert a.tokens == b.tokens
+    if dtype == "float32":
+        for prompt, res in zip(prompts, together):
+            ref = plain.forward(config, tensors, prompt + res.tokens[:-1])
+            for i, t in enumerate(res.tokens):
+                probs = plain.probabilities(ref[len(prompt) - 1 + i], 0.8)
+                u = plain.uniform(4, i)
+                expect = plain.sample(probs, u)
+                if t != expect:
+                    cdf = np.cumsum(probs)
+                    assert np.abs(cdf - u).min() < 1e-5, f"token {i}: {t} vs {expect}, not a boundary case"
+
+
+def test_command_line_json(model_dirs, plain_models):
+    name = "A"
+    config, tensors = plain_models[name]
+    prompt = tt.random_tokens(77, 9, CONFIGS[name][0]["vocab_size"])
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "liyab-cli"), "-m", model_dirs[name], "-p",
+           ",".join(map(str, prompt)), "-n", "12", "--temp", "0", "--dtype", "float32", "--json"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-3000:]
+    lines = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    assert "load_ms" in lines[0]
+    turn = lines[1]
+    assert turn["prompt_tokens"] == 9 and turn["generated_tokens"] == len(turn["tokens"])
+    expect = plain.generate_greedy(config, tensors, prompt, 12)
+    eos = config.get("eos_token_id")
+    assert turn["tokens"] == expect[:len(turn["tokens"])] and (len(turn["tokens"]) == 12 or turn["tokens"][-1] == eos)
+    assert "decode:" in p.stderr and "prompt: 9 tokens" in p.stderr
