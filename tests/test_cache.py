@@ -1,0 +1,174 @@
+"""The cache manager on the host: pages on demand, reuse, windows, state slots; no page is
+lost, held twice or freed twice under random orders of requests (no GPU)."""
+
+import random
+
+import pytest
+
+from liyab_amd import Busy, ContextFull, InvalidArgument, OutOfPages
+from liyab_amd.cache import UNMAPPED, CacheManager, KVSpec, PagePool
+
+
+def manager(num_pages=64, page_size=16, max_positions=1024, max_requests=8, window=0, groups=None):
+    groups = groups or [(KVSpec(4, 16, window), [0, 1])]
+    return CacheManager(groups, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                        max_positions=max_positions)
+
+
+def test_the_reference_tests_page_counts():
+    """tests/test_kv_cache.cpp:129-149 with 16-token pages and a 1,024 limit."""
+    m = manager()
+    m.open("r")
+    assert m.pages_in_use() == 0
+    m.reserve([("r", 1)])
+    assert m.pages_in_use() == 1
+    m.reserve([("r", 100)])
+    assert m.pages_in_use() == 7  # ceil(100 / 16)
+    with pytest.raises(ContextFull):
+        m.reserve([("r", 1025)])
+    m.commit("r", 100)
+    m.truncate("r", 20)  # pages starting at >= 32 are returned
+    assert m.pages_in_use() == 2
+    before = set(m.block_table("r"))
+    m.reserve([("r", 100)])
+    assert m.pages_in_use() == 7 and m.groups[0].pool.peak_in_use == 7  # freed pages were used again
+    assert before <= set(m.block_table("r"))
+    m.close("r")
+    assert m.pages_in_use() == 0
+    m.check()
+
+
+def test_reserve_is_all_or_nothing_across_requests():
+    m = manager(num_pages=5)
+    m.open("a")
+    m.open("b")
+    m.reserve([("a", 40)])  # 3 pages
+    m.commit("a", 40)
+    assert not m.can_reserve([("a", 50), ("b", 20)])  # 1 + 2 > 2 free
+    with pytest.raises(OutOfPages):
+        m.reserve([("a", 50), ("b", 20)])
+    assert m.pages_in_use() == 3 and m.block_table("b") == [] and len(m.block_table("a")) == 3
+    assert m.can_reserve([("a", 48), ("b", 16)])  # a needs none (48 fits 3 pages), b one
+    m.reserve([("a", 49), ("b", 16)])
+    assert m.pages_in_use() == 5 and m.free_pages() == 0
+    assert not m.can_reserve([], new_lengths=[1]) and m.can_reserve([], new_lengths=[0])
+    m.check()
+
+
+def test_finished_requests_pages_are_used_again_first():
+    m = manager(num_pages=8)
+    m.open("a")
+    m.reserve([("a", 64)])
+    pages_a = list(m.block_table("a"))
+    m.commit("a", 64)
+    m.close("a")
+    m.open("b")
+    m.reserve([("b", 33)])
+    assert set(m.block_table("b")) <= set(pages_a) and m.groups[0].pool.peak_in_use == 4
+    assert m.slot_of_position("b", 0, 17) == m.block_table("b")[1] * 16 + 1
+    m.check()
+
+
+def test_misuse_is_refused():
+    m = manager(max_requests=2)
+    m.open("a")
+    with pytest.raises(InvalidArgument):
+        m.open("a")
+    m.open("b")
+    with pytest.raises(Busy):
+        m.open("c")
+    m.reserve([("a", 10)])
+    with pytest.raises(InvalidArgument):
+        m.commit("a", 17)  # past the reserved pages
+    m.commit("a", 10)
+    with pytest.raises(InvalidArgument):
+        m.reserve([("a", 5)])
+    with pytest.raises(InvalidArgument):
+        m.truncate("a", 11)
+    with pytest.raises(KeyError):
+        m.close("zzz")
+    pool = PagePool(2)
+    p = pool.allocate(1)
+    pool.release(p)
+    with pytest.raises(AssertionError):
+        pool.release(p)  # freed twice
+    with pytest.raises(OutOfPages):
+        pool.allocate(3)
+
+
+def test_state_slots():
+    m = manager(max_requests=3)
+    slots = [m.open(r) for r in "abc"]
+    assert sorted(slots) == [0, 1, 2] and m.free_slots() == 0
+    m.close("b")
+    assert m.open("d") == slots[1]  # the freed slot is used again
+    m.check()
+
+
+def test_window_group_gives_back_pages_the_window_has_passed():
+    spec_all, spec_win = KVSpec(2, 16, 0), KVSpec(2, 16, 40)
+    m = CacheManager([(spec_all, [0, 2]), (spec_win, [1, 3])], page_size=16, num_pages=[64, 6], max_requests=4,
+                     max_positions=1024)
+    assert m.group_of_layer == {0: 0, 2: 0, 1: 1, 3: 1}
+    m.open("r")
+    length = 0
+    for n in (30, 30, 1, 1, 50, 1, 1, 1, 7, 33):
+        m.reserve([("r", length + n)])
+        length += n
+        m.commit("r", length)
+        # group 0 keeps everything
+        assert m.pages_in_use(0) == -(-length // 16)
+        # group 1 keeps exactly the pages a query at position >= length can still see
+        first_needed = max(0, length - 40 + 1)
+        table = m.block_table("r", 1)
+        for lp, page in enumerate(table):
+            assert (page == UNMAPPED) == ((lp + 1) * 16 <= first_needed), (length, lp)
+        m.check()
+    assert m.groups[1].pool.peak_in_use <= 6
+    m.close("r")
+    assert m.pages_in_use(0) == 0 and m.pages_in_use(1) == 0
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_lose_nothing(seed):
+    rng = random.Random(seed)
+    window = rng.choice([0, 0, 24, 70])
+    m = CacheManager([(KVSpec(2, 16, 0), [0]), (KVSpec(2, 16, window), [1])], page_size=rng.choice([4, 16]),
+                     num_pages=[rng.randint(20, 60), rng.randint(20, 60)], max_requests=5, max_positions=300)
+    live, n = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.15 and len(live) < 5:
+            rid = f"r{n}"
+            n += 1
+            m.open(rid)
+            live[rid] = 0
+        elif op < 0.75 and live:
+            k = rng.randint(1, min(3, len(live)))
+            wants = [(rid, live[rid] + rng.choice([1, 1, 1, 2, 9, 40])) for rid in rng.sample(sorted(live), k)]
+            used = [m.pages_in_use(g) for g in range(2)]
+            try:
+                m.reserve(wants)
+            except (OutOfPages, ContextFull):
+                assert [m.pages_in_use(g) for g in range(2)] == used  # nothing changed
+            else:
+                for rid, length in wants:
+                    m.commit(rid, length)
+                    live[rid] = length
+        elif op < 0.85 and live and window == 0:
+            rid = rng.choice(sorted(live))
+            live[rid] = rng.randint(0, live[rid])
+            m.truncate(rid, live[rid])
+        elif live:
+            rid = rng.choice(sorted(live))
+            m.close(rid)
+            del live[rid]
+        m.check()
+        for rid, length in live.items():
+            assert m.length(rid) == length
+            assert sum(p != UNMAPPED for p in m.block_table(rid, 0)) >= -(-length // m.page_size)
+    for rid in list(live):
+        m.close(rid)
+    m.check()
+    assert m.pages_in_use(0) == 0 and m.pages_in_use(1) == 0 and m.free_slots() == 5

@@ -1,0 +1,160 @@
+"""The scheduler's decisions, with the model replaced by a rule for the next token (no GPU)."""
+
+import pytest
+
+from liyab_amd import InvalidArgument, OutOfPages
+from liyab_amd.cache import CacheManager, KVSpec
+from liyab_amd.engine.scheduler import FINISHED, RUNNING, WAITING, Request, Scheduler
+from liyab_amd.sampling import SamplingParams
+
+
+def setup(num_pages=64, page_size=16, max_positions=256, max_num_seqs=4, budget=64, chunk=48, eos=None):
+    m = CacheManager([(KVSpec(2, 16, 0), [0])], page_size=page_size, num_pages=num_pages, max_requests=8,
+                     max_positions=max_positions)
+    return m, Scheduler(m, max_num_seqs=max_num_seqs, max_batched_tokens=budget, prefill_chunk=chunk, eos_token_id=eos)
+
+
+def next_token(r):
+    return (sum(r.tokens) * 31 + len(r.tokens)) % 97  # a pure function of the tokens so far
+
+
+def run(m, s, log=None, limit=10000):
+    """Drives the scheduler as the engine does, mapping pages as the step function would."""
+    steps = 0
+    while s.has_unfinished():
+        batch = s.schedule()
+        assert batch
+        assert sum(b.count for b in batch) <= s.max_batched_tokens
+        assert len({b.request.rid for b in batch}) == len(batch)
+        m.reserve([(b.request.rid, b.first + b.count) for b in batch])  # never fails: schedule() counted the pages
+        for b in batch:
+            assert b.first == m.length(b.request.rid) == b.request.computed
+            m.commit(b.request.rid, b.first + b.count)
+        sampled = {b.request.rid: next_token(b.request) for b in batch if b.wants_logits}
+        if log is not None:
+            log.append([(b.request.rid, b.first, b.count, b.wants_logits) for b in batch])
+        s.update(batch, sampled)
+        m.check()
+        steps += 1
+        assert steps < limit
+    return steps
+
+
+def alone(prompt, max_tokens, max_positions=256):
+    r = Request("x", list(prompt), SamplingParams(temperature=0, max_tokens=max_tokens))
+    while len(r.generated) < max_tokens and r.n_tokens <= max_positions:
+        r.generated.append(next_token(r))
+    return r.generated
+
+
+def test_prompt_portions_decoding_and_finish():
+    m, s = setup(budget=64, chunk=48)
+    r = Request("a", list(range(100)), SamplingParams(temperature=0, max_tokens=5))
+    s.add(r)
+    log = []
+    run(m, s, log)
+    assert [x[0][1:] for x in log[:3]] == [(0, 48, False), (48, 48, False), (96, 4, True)]
+    assert all(x[0][2] == 1 and x[0][3] for x in log[3:]) and len(log) == 3 + 4
+    assert r.state == FINISHED and r.finish_reason == "length" and r.generated == alone(range(100), 5)
+    assert m.pages_in_use() == 0 and not m.is_open("a")
+    assert s.stats.batched_tokens == 100 + 4 and s.stats.decode_tokens == 4 and s.stats.prefill_tokens == 100
+
+
+def test_decodes_first_then_portions_under_the_budget():
+    m, s = setup(budget=20, chunk=48)
+    a = Request("a", [1, 2, 3], SamplingParams(temperature=0, max_tokens=50))
+    s.add(a)
+    log = []
+    b = Request("b", list(range(60)), SamplingParams(temperature=0, max_tokens=3))
+    batch = s.schedule()  # a's prompt alone
+    m.reserve([("a", 3)]); m.commit("a", 3); s.update(batch, {"a": next_token(a)})
+    s.add(b)
+    run(m, s, log)
+    first = log[0]
+    assert first[0] == ("a", 3, 1, True)  # the decoding request comes first, with its one token
+    assert first[1] == ("b", 0, 19, False)  # the portion is what the budget leaves
+    assert log[1][1] == ("b", 19, 19, False) and log[3][1] == ("b", 57, 3, True)
+    assert a.generated == alone([1, 2, 3], 50) and b.generated == alone(range(60), 3)
+
+
+def test_admission_first_come_first_served_and_slots():
+    m, s = setup(max_num_seqs=2, budget=64, chunk=64)
+    rs = [Request(f"r{i}", [i + 1] * 10, SamplingParams(temperature=0, max_tokens=4)) for i in range(4)]
+    for r in rs:
+        s.add(r)
+    batch = s.schedule()
+    assert [b.request.rid for b in batch] == ["r0", "r1"] and [r.state for r in rs] == [RUNNING, RUNNING, WAITING, WAITING]
+    m.reserve([(b.request.rid, b.count) for b in batch])
+    for b in batch:
+        m.commit(b.request.rid, b.count)
+    s.update(batch, {b.request.rid: next_token(b.request) for b in batch})
+    run(m, s)
+    assert all(r.generated == alone(r.prompt, 4) for r in rs)
+
+
+def test_stops_at_eos_and_at_the_last_position():
+    m, s = setup(max_positions=32, eos=next_token(Request("p", [5, 6, 7], SamplingParams())))
+    r = Request("a", [5, 6, 7], SamplingParams(temperature=0, max_tokens=10))
+    s.add(r)
+    run(m, s)
+    assert r.finish_reason == "stop" and len(r.generated) == 1
+    m, s = setup(max_positions=32)
+    r = Request("a", list(range(30)), SamplingParams(temperature=0, max_tokens=10))
+    s.add(r)
+    run(m, s)
+    assert r.finish_reason == "context" and len(r.generated) == 3 and r.n_tokens == 33  # positions 0..31 were run
+    m, s = setup()
+    r = Request("a", [1, 2], SamplingParams(temperature=0, max_tokens=10))
+    s.add(r)
+    batch = s.schedule()
+    m.reserve([("a", 2)]); m.commit("a", 2)
+    s.update(batch, {"a": 9}, on_token=lambda req, tok: False)
+    assert r.finish_reason == "callback" and m.pages_in_use() == 0
+
+
+def test_refusals_on_arrival():
+    m, s = setup(num_pages=4, max_positions=64)
+    with pytest.raises(InvalidArgument, match="empty"):
+        s.add(Request("a", [], SamplingParams()))
+    with pytest.raises(InvalidArgument, match="max_tokens"):
+        s.add(Request("a", [1], SamplingParams(max_tokens=0)))
+    with pytest.raises(InvalidArgument, match="context holds"):
+        s.add(Request("a", [1] * 65, SamplingParams()))
+    m, s = setup(num_pages=2, max_positions=256)
+    with pytest.raises(OutOfPages, match="may need 3 pages"):
+        s.add(Request("a", [1] * 30, SamplingParams(max_tokens=4)))  # 33 positions > 2 pages: could never fit
+    s.add(Request("b", [1] * 30, SamplingParams(max_tokens=3)))  # 32 positions: fits alone
+
+
+def test_when_pages_run_out_the_latest_request_is_preempted_and_recomputed():
+    """8 pages of 16; three requests that each grow to 5 pages cannot all stay. The most recently
+    admitted one gives its pages back, waits at the head of the queue and is recomputed from
+    its prompt plus what it had generated; everyone's tokens are those it generates alone."""
+    m, s = setup(num_pages=8, budget=64, chunk=32, max_num_seqs=3)
+    rs = [Request(f"r{i}", [i + 3] * 30, SamplingParams(temperature=0, max_tokens=45)) for i in range(3)]
+    for r in rs:
+        s.add(r)
+    log = []
+    run(m, s, log)
+    assert s.stats.preemptions >= 1
+    assert rs[0].preemptions == 0  # the earliest request is never the victim of a later one
+    assert rs[2].preemptions >= 1
+    for r in rs:
+        assert r.generated == alone(r.prompt, 45), r.rid
+        assert r.state == FINISHED
+    # a preempted request starts again from position 0 with its generated tokens as prompt
+    restarts = [e for step in log for e in step if e[0] == "r2" and e[1] == 0]
+    assert len(restarts) == 1 + rs[2].preemptions
+    assert s.stats.pages_in_use_peak <= 8 and m.pages_in_use() == 0
+    m.check()
+
+
+def test_no_request_starves_under_pressure():
+    m, s = setup(num_pages=6, budget=32, chunk=16, max_num_seqs=4)
+    rs = [Request(f"r{i}", [i + 1] * (5 + 7 * i), SamplingParams(temperature=0, max_tokens=30)) for i in range(6)]
+    for r in rs:
+        s.add(r)
+    steps = run(m, s)
+    assert steps < 2000
+    for r in rs:
+        assert r.generated == alone(r.prompt, 30)
