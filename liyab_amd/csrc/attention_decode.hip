@@ -1,0 +1,235 @@
+// Attention for tokens taken one at a time (decoding, short prompt portions)
+// over paged bfloat16 keys and values, with the keys of a token cut into
+// splits so that few tokens still fill the chip.
+//
+// Grid (token, query head, split). A workgroup of 4 waves walks its split's
+// keys; LPK lanes share a key (each holds 8 consecutive dimensions, 16
+// bytes), so a wave takes 64 / LPK keys a pass, read straight from the pages
+// through the block table. Each lane group keeps a running maximum, sum and
+// weighted values (the reference's per-span partial softmax,
+// src/core/transformer.cpp:2327-2358); groups, then waves, then splits are
+// merged in a fixed order by rescaling to the common maximum (:2367-2385).
+// The reference cuts a token's keys by its position only (:2136-2139,
+// 2225-2227) to keep bits equal; here the number of splits follows the batch
+// (more splits when few tokens are in flight), which moves results by
+// rounding only. Scores, exponentials and sums are 32-bit.
+#include "common.h"
+
+namespace liyab {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr int AD_WAVES = 4;
+constexpr int AD_U = 4;  // keys per lane group and trip
+
+__device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(v[i] << 16);
+        f[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+}
+
+struct Partial {
+    float m, l;
+    float acc[8];
+};
+
+// this <- merge(this, other): both rescaled to the larger maximum; this comes first.
+__device__ __forceinline__ void merge_partial(Partial& a, float mo, float lo, const float* acco) {
+    const float M = fmaxf(a.m, mo);
+    const float wa = a.m == -INFINITY ? 0.0f : __expf(a.m - M);
+    const float wb = mo == -INFINITY ? 0.0f : __expf(mo - M);
+    a.l = wa * a.l + wb * lo;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a.acc[e] = wa * a.acc[e] + wb * acco[e];
+    a.m = M;
+}
+
+template <int LPK>
+__global__ void __launch_bounds__(64 * AD_WAVES)
+attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+                        const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                        const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
+                        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
+                        int n_head, int n_kv_head, int hd, int page_size, int n_splits, float* __restrict__ partials) {
+    constexpr int KPP = 64 / LPK;  // keys per wave and pass
+    __shared__ float lds[AD_WAVES][LPK][10];
+    const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
+    const int h = blockIdx.y, z = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int c = lane % LPK, kg = lane / LPK;
+    const bool active = c * 8 < hd;
+    const int pos = tok_pos[t];
+    const int* bt = block_tables + static_cast<int64_t>(tok_seq[t]) * max_blocks;
+    const int hkv = h / (n_head / n_kv_head);
+    const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_keys = pos - first + 1;
+    const int k_begin = first + static_cast<int>(static_cast<int64_t>(n_keys) * z / n_splits);
+    const int k_end = first + static_cast<int>(static_cast<int64_t>(n_keys) * (z + 1) / n_splits);
+
+    float qf[8];
+    {
+        u32x4 qv = {0, 0, 0, 0};
+        if (active) qv = *reinterpret_cast<const u32x4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * hd + c * 8);
+        unpack8(qv, qf);
+    }
+    Partial st;
+    st.m = -INFINITY;
+    st.l = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) st.acc[e] = 0.0f;
+
+    const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd + c * 8;
+    const int64_t page_stride = static_cast<int64_t>(n_kv_head) * page_size * hd;
+    for (int j0 = k_begin + wave * KPP; j0 < k_end; j0 += AD_WAVES * KPP * AD_U) {
+        u32x4 kv[AD_U], vv[AD_U];
+        bool valid[AD_U];
+#pragma unroll
+        for (int u = 0; u < AD_U; ++u) {
+            const int j = j0 + u * AD_WAVES * KPP + kg;
+            valid[u] = j < k_end;
+            const int jc = valid[u] ? j : pos;  // a mapped position; its values are not used
+            const int64_t at = static_cast<int64_t>(bt[jc / page_size]) * page_stride + head_off +
+                               static_cast<int64_t>(jc % page_size) * hd;
+            kv[u] = u32x4{0, 0, 0, 0};
+            vv[u] = u32x4{0, 0, 0, 0};
+            if (active) {
+                kv[u] = *reinterpret_cast<const u32x4*>(kc + at);
+                vv[u] = *reinterpret_cast<const u32x4*>(vc + at);
+            }
+        }
+        float s[AD_U];
+        float m_new = st.m;
+#pragma unroll
+        for (int u = 0; u < AD_U; ++u) {
+            float kf[8];
+            unpack8(kv[u], kf);
+            float d = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d = fmaf(kf[e], qf[e], d);
+#pragma unroll
+            for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, 64);
+            s[u] = valid[u] ? d * scale : -INFINITY;
+            m_new = fmaxf(m_new, s[u]);
+        }
+        if (m_new == -INFINITY) continue;  // this lane group had no key in this trip (and none before)
+        const float corr = st.m == -INFINITY ? 0.0f : __expf(st.m - m_new);
+        st.l *= corr;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) st.acc[e] *= corr;
+#pragma unroll
+        for (int u = 0; u < AD_U; ++u) {
+            if (!valid[u]) continue;
+            const float p = __expf(s[u] - m_new);
+            st.l += p;
+            float vf[8];
+            unpack8(vv[u], vf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) st.acc[e] = fmaf(p, vf[e], st.acc[e]);
+        }
+        st.m = m_new;
+    }
+    // lane groups of the wave, in a fixed tree
+#pragma unroll
+    for (int off = LPK; off < 64; off <<= 1) {
+        const float mo = __shfl_xor(st.m, off, 64), lo = __shfl_xor(st.l, off, 64);
+        float ao[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ao[e] = __shfl_xor(st.acc[e], off, 64);
+        merge_partial(st, mo, lo, ao);
+    }
+    if (kg == 0) {
+        lds[wave][c][0] = st.m;
+        lds[wave][c][1] = st.l;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) lds[wave][c][2 + e] = st.acc[e];
+    }
+    __syncthreads();
+    if (wave == 0 && kg == 0 && active) {
+#pragma unroll
+        for (int w = 1; w < AD_WAVES; ++w) merge_partial(st, lds[w][c][0], lds[w][c][1], &lds[w][c][2]);
+        if (n_splits == 1) {
+            bf16_t* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
+            const float inv = 1.0f / st.l;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = float_to_bf16(st.acc[e] * inv);
+        } else {
+            // partials [token slot][head][split][hd + 2]: values, then maximum and sum
+            float* p = partials + ((static_cast<int64_t>(blockIdx.x) * n_head + h) * n_splits + z) * (hd + 2);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) p[c * 8 + e] = st.acc[e];
+            if (c == 0) {
+                p[hd] = st.m;
+                p[hd + 1] = st.l;
+            }
+        }
+    }
+}
+
+// Splits of a (token, head) merged in split order.
+__global__ void attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
+                                       const float* __restrict__ partials, int n_head, int hd, int n_splits) {
+    const int slot = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
+    if (e >= hd) return;
+    const int t = tok_list != nullptr ? tok_list[slot] : slot;
+    const float* p = partials + (static_cast<int64_t>(slot) * n_head + h) * n_splits * (hd + 2);
+    float M = -INFINITY;
+    for (int z = 0; z < n_splits; ++z) M = fmaxf(M, p[z * (hd + 2) + hd]);
+    float sum = 0.0f, o = 0.0f;
+    for (int z = 0; z < n_splits; ++z) {
+        const float m = p[z * (hd + 2) + hd];
+        if (m == -INFINITY) continue;
+        const float w = __expf(m - M);
+        sum += w * p[z * (hd + 2) + hd + 1];
+        o += w * p[z * (hd + 2) + e];
+    }
+    out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = float_to_bf16(o / sum);
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+// Tokens tok_list[0..n) (or 0..n-1 when tok_list is null), each on its own. `partials` must hold
+// n * n_head * n_splits * (hd + 2) floats when n_splits > 1.
+extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                      const void* vc, const int* block_tables, int max_blocks, const int* tok_list,
+                                      const int* tok_seq, const int* tok_pos, int n, float scale, int window,
+                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, float* partials,
+                                      hipStream_t stream) {
+    LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
+    LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
+    LIYAB_REQUIRE(hd >= 8 && hd <= 256 && hd % 8 == 0, "attention_decode: head size %d is not a multiple of 8 in 8..256", hd);
+    LIYAB_REQUIRE(q_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(q) & 15) == 0 && (reinterpret_cast<uintptr_t>(kc) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(vc) & 15) == 0,
+                  "attention_decode: queries and caches must be 16-byte aligned with a query stride that is a multiple of 8");
+    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
+                  "attention_decode: row strides are shorter than heads x head size");
+    LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
+    LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
+    if (n == 0) return 0;
+    dim3 grid(n, n_head, n_splits);
+    auto* o = static_cast<bf16_t*>(out);
+    auto* pq = static_cast<const bf16_t*>(q);
+    auto* pk = static_cast<const bf16_t*>(kc);
+    auto* pv = static_cast<const bf16_t*>(vc);
+#define LIYAB_GO(L)                                                                                                   \
+    attention_decode_kernel<L><<<grid, 64 * AD_WAVES, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                   max_blocks, tok_list, tok_seq, tok_pos, scale,    \
+                                                                   window, n_head, n_kv_head, hd, page_size, n_splits, partials)
+    if (hd <= 8) LIYAB_GO(1);
+    else if (hd <= 16) LIYAB_GO(2);
+    else if (hd <= 32) LIYAB_GO(4);
+    else if (hd <= 64) LIYAB_GO(8);
+    else if (hd <= 128) LIYAB_GO(16);
+    else LIYAB_GO(32);
+#undef LIYAB_GO
+    if (int rc = check_launch("attention_decode")) return rc;
+    if (n_splits > 1) {
+        attention_merge_kernel<<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits);
+        return check_launch("attention_merge");
+    }
+    return 0;
+}

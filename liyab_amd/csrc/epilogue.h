@@ -1,0 +1,81 @@
+// What a matrix product does with its accumulators.
+//
+// Every product kernel ends in the same epilogue: add the bias, then one of
+//   none / GELU          -> out[m, n] in the output type
+//   residual             -> residual[m, n] += value (the 32-bit residual stream)
+//   paged QKV            -> columns [0, q_dim) go to out[m, n] (queries);
+//                           columns of keys and values go straight to token
+//                           m's slot of the cache pages, so the projection's
+//                           output is never copied (the reference splits the
+//                           fused output per token and then stores the rows,
+//                           src/core/transformer.cpp:2657-2673, 2875-2890).
+#pragma once
+
+#include "activations.h"
+#include "common.h"
+
+namespace liyab {
+
+enum : int { kEpiQkvPaged = 4 };
+
+struct EpiParams {
+    int mode;
+    int out_dtype;            // of out and of the cache pages
+    const float* bias;        // [N] or null
+    void* out;                // [M, ldo]
+    int64_t ldo;
+    float* residual;          // [M, ldr]
+    int64_t ldr;
+    // paged QKV
+    void* kc;
+    void* vc;
+    const int* slots;         // [M]: page * page_size + offset
+    int q_dim, kv_dim, hd, n_kv_head, page_size;
+    int exact;                // erf in double (32-bit path)
+};
+
+template <typename OutT>
+__device__ __forceinline__ void epilogue_store(const EpiParams& p, int m, int n, float v) {
+    if (p.bias != nullptr) v += p.bias[n];
+    switch (p.mode) {
+        case kEpiGeluTanh: v = gelu_tanh(v); break;
+        case kEpiGeluErf: v = p.exact ? gelu_erf_exact(v) : gelu_erf_fast(v); break;
+        case kEpiResidual:
+            p.residual[static_cast<int64_t>(m) * p.ldr + n] += v;
+            return;
+        case kEpiQkvPaged:
+            if (n >= p.q_dim) {
+                const bool is_v = n >= p.q_dim + p.kv_dim;
+                const int c = n - p.q_dim - (is_v ? p.kv_dim : 0);
+                const int64_t slot = p.slots[m];
+                if (slot < 0) return;
+                const int64_t page = slot / p.page_size;
+                const int off = static_cast<int>(slot % p.page_size);
+                const int64_t dst = ((page * p.n_kv_head + c / p.hd) * p.page_size + off) * p.hd + c % p.hd;
+                static_cast<OutT*>(is_v ? p.vc : p.kc)[dst] = from_float<OutT>(v);
+                return;
+            }
+            break;
+        default: break;
+    }
+    static_cast<OutT*>(p.out)[static_cast<int64_t>(m) * p.ldo + n] = from_float<OutT>(v);
+}
+
+// Host-side check shared by the launchers.
+inline int check_epilogue(const EpiParams& p, int M, int N) {
+    (void)M;
+    if (p.mode == kEpiResidual) {
+        LIYAB_REQUIRE(p.residual != nullptr && p.ldr >= N, "gemm: the residual epilogue needs a residual of row stride >= N");
+    } else if (p.mode == kEpiQkvPaged) {
+        LIYAB_REQUIRE(p.out && p.kc && p.vc && p.slots, "gemm: the paged QKV epilogue needs out, caches and slots");
+        LIYAB_REQUIRE(p.q_dim > 0 && p.kv_dim > 0 && p.hd > 0 && p.page_size > 0 && p.n_kv_head * p.hd == p.kv_dim &&
+                          p.q_dim + 2 * p.kv_dim == N && p.ldo >= p.q_dim,
+                      "gemm: the paged QKV epilogue's sizes do not fit N = %d", N);
+    } else {
+        LIYAB_REQUIRE(p.mode >= kEpiNone && p.mode <= kEpiGeluErf, "gemm: unknown epilogue %d", p.mode);
+        LIYAB_REQUIRE(p.out != nullptr && p.ldo >= N, "gemm: needs an output of row stride >= N");
+    }
+    return 0;
+}
+
+}  // namespace liyab

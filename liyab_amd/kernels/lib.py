@@ -20,6 +20,18 @@ _lib: Optional[ctypes.CDLL] = None
 _path: Optional[str] = None
 
 P = c_void_p
+
+
+class EpiParams(ctypes.Structure):
+    """Mirror of csrc/epilogue.h's EpiParams."""
+
+    _fields_ = [
+        ("mode", c_int), ("out_dtype", c_int), ("bias", P), ("out", P), ("ldo", c_int64), ("residual", P),
+        ("ldr", c_int64), ("kc", P), ("vc", P), ("slots", P), ("q_dim", c_int), ("kv_dim", c_int), ("hd", c_int),
+        ("n_kv_head", c_int), ("page_size", c_int), ("exact", c_int),
+    ]
+
+
 _SIGNATURES = {
     "liyab_check_device": [],
     "liyab_fill": [P, c_int, c_uint32, c_int64, P],
@@ -29,8 +41,12 @@ _SIGNATURES = {
     "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
     "liyab_layernorm": [P, c_int, P, P, P, P, c_int, c_int, c_float, P],
     "liyab_gemm_simple": [P, c_int, c_int64, P, c_int64, P, c_int, P, P, c_int64, c_int, c_int, c_int, c_int, P],
+    "liyab_gemm_mfma": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_skinny": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_generic": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, P],
+    "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
+                               c_int, c_int, c_int, P, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P],
     "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
 }

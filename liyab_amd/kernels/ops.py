@@ -8,6 +8,7 @@ library's own kernel. Nothing here runs without the GPU and the library.
 
 from __future__ import annotations
 
+import ctypes
 import struct
 from typing import Optional
 
@@ -250,16 +251,144 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, t
               top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(), _stream())
 
 
+EPI_QKV_PAGED = 4
+
+
+def _epilogue(a, w, bias, out, residual, epilogue, kv):
+    """Checks the epilogue's operands against [M, N] and fills the launchers' struct."""
+    M, N = a.shape[0], w.shape[0]
+    _f32vec(bias, "bias", N)
+    e = _lib.EpiParams()
+    e.mode = epilogue
+    e.bias = _ptr(bias)
+    e.exact = 1 if a.dtype == torch.float32 else 0
+    e.out_dtype = F32
+    if epilogue == EPI_RESIDUAL:
+        if residual is None or residual.dtype != torch.float32 or tuple(residual.shape) != (M, N):
+            raise KernelError("gemm: the residual epilogue needs a float32 residual [M, N]")
+        e.residual, e.ldr = residual.data_ptr(), _rows(residual, "residual")
+    elif epilogue == EPI_QKV_PAGED:
+        k_cache, v_cache, slots, q_dim = kv
+        if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+            raise KernelError("gemm: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
+        _, hkv, page, hd = k_cache.shape
+        if out is None or tuple(out.shape) != (M, q_dim) or q_dim + 2 * hkv * hd != N:
+            raise KernelError(f"gemm: the paged QKV epilogue needs out [M, {q_dim}] and N = q_dim + 2 * kv_dim")
+        if not (out.dtype == k_cache.dtype == v_cache.dtype):
+            raise KernelError("gemm: queries and caches must share a dtype")
+        _i32(slots, "slots", M)
+        e.out, e.ldo, e.out_dtype = out.data_ptr(), _rows(out, "out"), dtype_code(out.dtype)
+        e.kc, e.vc, e.slots = k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr()
+        e.q_dim, e.kv_dim, e.hd, e.n_kv_head, e.page_size = q_dim, hkv * hd, hd, hkv, page
+    else:
+        if out is None or tuple(out.shape) != (M, N):
+            raise KernelError("gemm: out must be [M, N]")
+        e.out, e.ldo, e.out_dtype = out.data_ptr(), _rows(out, "out"), dtype_code(out.dtype)
+    return e
+
+
+def gemm_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
+              epilogue: int = EPI_NONE, kv=None, tile: int = 0) -> None:
+    """The matrix-core product for bfloat16 operands with K a multiple of 8."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_mfma: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
+    e = _epilogue(a, w, bias, out, residual, epilogue, kv)
+    _lib.call("liyab_gemm_mfma", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, tile, ctypes.byref(e), _stream())
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
+                epilogue: int = EPI_NONE, kv=None, ksplit: int = 0) -> None:
+    """The weight-streaming product for at most 16 bfloat16 rows, K a multiple of 8."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_skinny: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
+    if M > 16:
+        raise KernelError(f"gemm_skinny: {M} rows; it takes at most 16")
+    e = _epilogue(a, w, bias, out, residual, epilogue, kv)
+    _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, ctypes.byref(e), _stream())
+
+
+def mfma_takes(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
-         residual: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE) -> None:
+         residual: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, kv=None) -> None:
     """The product kernel for these operands: matrix cores for bfloat16 shapes they take,
-    the plain tiled kernel for float32 and everything else."""
+    the plain tiled kernel for float32 and everything else. `kv` = (k_cache, v_cache, slots,
+    q_dim) with the paged QKV epilogue."""
+    if mfma_takes(a, w):
+        if a.shape[0] <= 16:
+            gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
+        else:
+            gemm_mfma(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
+        return
+    if epilogue == EPI_QKV_PAGED:
+        # the plain kernel writes the whole projection; a second kernel moves keys and values
+        k_cache, v_cache, slots, q_dim = kv
+        raise KernelError("gemm: the paged QKV epilogue is for the matrix-core kernels; use gemm + kv_write")
     gemm_simple(a, w, bias, out=out, residual=residual, epilogue=epilogue)
+
+
+def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
+                     scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
+                     tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None) -> None:
+    """Each token on its own over its request's bfloat16 cache, its keys cut into `n_splits`.
+    With `tok_list` (int32) only those rows are computed."""
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
+    _, hkv, page, hd = k_cache.shape
+    os_, qs = _rows(out, "out"), _rows(q, "q")
+    rows = out.shape[0]
+    n = rows if n_tokens is None else n_tokens
+    if q.shape[0] != rows or q.shape[1] < n_head * hd or out.shape[1] != n_head * hd:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {n_head} heads of {hd}")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        raise KernelError("attention_decode: q, out and the caches must be bfloat16")
+    _dev(block_tables, "block_tables")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
+    _i32(tok_seq, "tok_seq", rows)
+    _i32(tok_pos, "tok_pos", rows)
+    if tok_list is not None:
+        _i32(tok_list, "tok_list", n)
+    elif n != rows:
+        raise KernelError("attention_decode: n_tokens needs tok_list")
+    if n_splits > 1:
+        need = n * n_head * n_splits * (hd + 2)
+        if partials is None or partials.dtype != torch.float32 or partials.numel() < need or not partials.is_contiguous():
+            raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
+    _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
+              block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
+              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, _ptr(partials), _stream())
+
+
+def decode_splits(n_tokens: int, n_head: int, max_context: int) -> int:
+    """How many splits of the keys give the chip enough workgroups without making them tiny."""
+    groups = max(1, n_tokens * n_head)
+    return max(1, min(-(-1024 // groups), max_context // 128, 32))
 
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0) -> None:
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
     is chosen from the step's shape (`ctx` is the step's StepContext)."""
+    hd = k_cache.shape[3]
+    if q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and ctx.host.max_q_len <= 8:
+        n = out.shape[0]
+        splits = decode_splits(n, n_head, ctx.host.max_context)
+        partials = None
+        if splits > 1:
+            partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 2),), torch.float32)
+        attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
+                         scale=scale, window=window, n_splits=splits, partials=partials)
+        return
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)

@@ -55,12 +55,18 @@ class Attention:
         n = h.shape[0]
         ws = ctx.workspace
         group = ctx.groups[cache.group]
-        qkv = ws.get("qkv", (n, self.q_dim + 2 * self.kv_dim), self.dtype)
-        linear(h, self.qkv_weight, self.qkv_bias, out=qkv)
-        if writes_cache:
-            ops.kv_write(cache.k, cache.v, qkv, self.q_dim, self.q_dim + self.kv_dim, group.slots)
+        if writes_cache and ops.mfma_takes(h, self.qkv_weight):
+            # the projection's epilogue puts keys and values straight into their pages
+            q = ws.get("q", (n, self.q_dim), self.dtype)
+            ops.gemm(h, self.qkv_weight, self.qkv_bias, out=q, epilogue=ops.EPI_QKV_PAGED,
+                     kv=(cache.k, cache.v, group.slots, self.q_dim))
+        else:
+            q = ws.get("qkv", (n, self.q_dim + 2 * self.kv_dim), self.dtype)
+            linear(h, self.qkv_weight, self.qkv_bias, out=q)
+            if writes_cache:
+                ops.kv_write(cache.k, cache.v, q, self.q_dim, self.q_dim + self.kv_dim, group.slots)
         att = ws.get("att", (n, self.q_dim), self.dtype)
-        ops.attention(att, qkv, cache.k, cache.v, group.block_tables, ctx, n_head=self.n_head, scale=self.scale,
+        ops.attention(att, q[:, :self.q_dim] if q.shape[1] != self.q_dim else q, cache.k, cache.v, group.block_tables, ctx, n_head=self.n_head, scale=self.scale,
                       window=self.window)
         linear(att, self.out_weight, self.out_bias, residual=residual)
 

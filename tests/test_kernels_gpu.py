@@ -1,0 +1,288 @@
+"""Each kernel alone against a plain 32-bit PyTorch reference of the same operation, at
+sizes other than the engine's (needs the GPU)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from liyab_amd.kernels import ops as o
+
+    o.check_device()
+    return o
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, tol, what=""):
+    got, want = got.double().cpu(), want.double().cpu()
+    err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30)
+    assert math.isfinite(err) and err <= tol, f"{what}: relative error {err:.3e} > {tol:.1e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,d", [(1, 64), (7, 100), (33, 1600), (5, 4096 + 24)])
+def test_embed_and_add_rows(ops, dtype, n, d):
+    V, P = 321, 77
+    table, pos = rnd(V, d, dtype=dtype), rnd(P, d, dtype=dtype, seed=1)
+    ids = torch.randint(0, V, (n,), dtype=torch.int32, device=DEV)
+    positions = torch.randint(0, P, (n,), dtype=torch.int32, device=DEV)
+    out = torch.empty(n, d, device=DEV)
+    ops.embed(out, table, ids, 1.0, pos_table=pos, positions=positions)
+    want = table.float()[ids.long()] + pos.float()[positions.long()]
+    assert torch.equal(out, want)
+    ops.embed(out, table, ids, 2.5)
+    assert torch.equal(out, table.float()[ids.long()] * 2.5)
+    ops.add_rows_(out, pos, positions)
+    assert torch.equal(out, table.float()[ids.long()] * 2.5 + pos.float()[positions.long()])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,d,eps", [(1, 64, 1e-5), (9, 96, 1e-6), (40, 1600, 1e-5), (3, 777, 1e-3)])
+def test_layernorm(ops, out_dtype, n, d, eps):
+    x = rnd(n + 3, d, scale=3.0) + 1.5
+    w, b = rnd(d, seed=2) + 1.0, rnd(d, seed=3)
+    out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    ops.layernorm(out, x, w, b, eps)
+    want = torch.nn.functional.layer_norm(x[:n].double(), (d,), w.double(), b.double(), eps)
+    close(out, want, 1e-6 if out_dtype == torch.float32 else 5e-3, "layernorm")
+    rows = torch.tensor([(i * 2) % (n + 3) for i in range(n)], dtype=torch.int32, device=DEV)
+    ops.layernorm(out, x, w, None, eps, rows=rows)
+    want = torch.nn.functional.layer_norm(x[rows.long()].double(), (d,), w.double(), None, eps)
+    close(out, want, 1e-6 if out_dtype == torch.float32 else 5e-3, "layernorm gather")
+    # eps is the kernel's argument, not a constant: a low-variance row shows it
+    flat = torch.ones(1, d, device=DEV) + 1e-3 * rnd(1, d, seed=9)
+    o1, o2 = torch.empty(1, d, device=DEV), torch.empty(1, d, device=DEV)
+    ops.layernorm(o1, flat, None, None, 1e-5)
+    ops.layernorm(o2, flat, None, None, 1e-6)
+    assert (o1 - o2).abs().max() > 1e-2
+
+
+def gemm_reference(a, w, bias, epilogue, residual=None):
+    y = a.double() @ w.double().t()
+    if bias is not None:
+        y = y + bias.double()
+    if epilogue == "gelu_tanh":
+        y = torch.nn.functional.gelu(y, approximate="tanh")
+    elif epilogue == "gelu_erf":
+        y = torch.nn.functional.gelu(y)
+    elif epilogue == "residual":
+        y = residual.double() + y
+    return y
+
+
+GEMM_SHAPES = [(1, 64, 64), (7, 200, 96), (33, 777, 144), (130, 50, 320), (64, 1000, 96), (257, 130, 72)]
+
+
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_float32(ops, M, N, K, epilogue):
+    a, w, bias = rnd(M, K), rnd(N, K, seed=1, scale=0.2), rnd(N, seed=2)
+    if epilogue == "residual":
+        res = rnd(M, N, seed=3)
+        want = gemm_reference(a, w, bias, epilogue, res)
+        ops.gemm(a, w, bias, residual=res, epilogue=ops.EPI_RESIDUAL)
+        close(res, want, 2e-6, "gemm f32 residual")
+    else:
+        out = torch.empty(M, N, device=DEV)
+        ops.gemm(a, w, bias, out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue])
+        close(out, gemm_reference(a, w, bias, epilogue), 2e-6, f"gemm f32 {epilogue}")
+    # a row's result does not depend on the rows around it
+    if M > 1:
+        one = torch.empty(1, N, device=DEV)
+        ops.gemm(a[M // 2:M // 2 + 1], w, bias, out=one)
+        full = torch.empty(M, N, device=DEV)
+        ops.gemm(a, w, bias, out=full)
+        assert torch.equal(one[0], full[M // 2])
+
+
+@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16"])
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200)])
+def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
+    a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    tiles = {"mfma128": 1, "mfma64": 2, "mfma128x64": 3}
+
+    if kernel.startswith("skinny") and M > 16:
+        pytest.skip("the skinny kernel takes at most 16 rows")
+
+    def run(**kw):
+        if kernel.startswith("skinny"):
+            ops.gemm_skinny(a, w, bias, ksplit=int(kernel[6:]), **kw)
+        elif kernel == "simple":
+            ops.gemm_simple(a, w, bias, **kw)
+        elif kernel == "auto":
+            ops.gemm(a, w, bias, **kw)
+        else:
+            ops.gemm_mfma(a, w, bias, tile=tiles[kernel], **kw)
+
+    if epilogue == "residual":
+        res = rnd(M, N, seed=3)
+        want = gemm_reference(a, w, bias, epilogue, res)
+        run(residual=res, epilogue=ops.EPI_RESIDUAL)
+        close(res, want, 1e-5, f"gemm bf16 residual {kernel}")
+    else:
+        for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 5e-3)):
+            out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+            run(out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue])
+            close(out, gemm_reference(a, w, bias, epilogue), tol, f"gemm bf16 {epilogue} {kernel} -> {out_dtype}")
+
+
+def test_gemm_strided_rows_and_refusals(ops):
+    from liyab_amd import KernelError
+
+    wide = rnd(20, 256, dtype=torch.bfloat16)
+    a = wide[:, 64:128]  # a view into a wider buffer: rows strided
+    w = rnd(48, 64, dtype=torch.bfloat16, seed=1)
+    out = torch.empty(20, 48, device=DEV)
+    ops.gemm(a, w, None, out=out)
+    close(out, a.double() @ w.double().t(), 1e-5, "strided a")
+    with pytest.raises(KernelError):
+        ops.gemm(a, rnd(48, 63, dtype=torch.bfloat16), None, out=out)  # K mismatch
+    with pytest.raises(KernelError):
+        ops.gemm(a, w, rnd(47), out=out)  # bias length
+    with pytest.raises(KernelError):
+        ops.gemm(a.float(), w, None, out=out)  # mixed dtypes
+    with pytest.raises(KernelError):
+        ops.gemm_mfma(rnd(4, 20, dtype=torch.bfloat16), rnd(8, 20, dtype=torch.bfloat16), None, out=torch.empty(4, 8, device=DEV))  # K % 8
+    with pytest.raises(KernelError):
+        ops.gemm(a, w, None, out=torch.empty(20, 48))  # not on the GPU
+
+
+# ---------------------------------------------------------------------------
+# attention over pages
+# ---------------------------------------------------------------------------
+def paged_case(n_seqs, ctx_lens, q_lens, H, Hkv, hd, page, dtype, seed=0, shuffle=True):
+    """Random requests in a shuffled page pool; returns everything the kernels take and a
+    float64 reference per token."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages_per = [-(-c // page) for c in ctx_lens]
+    total_pages = sum(n_pages_per) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist() if shuffle else list(range(total_pages))
+    kc = torch.full((total_pages, Hkv, page, hd), float("nan"), dtype=dtype)
+    vc = torch.full((total_pages, Hkv, page, hd), float("nan"), dtype=dtype)
+    W = max(n_pages_per) + 1
+    bt = torch.full((n_seqs, W), -1, dtype=torch.int32)
+    ks, vs = [], []
+    nxt = 0
+    for s in range(n_seqs):
+        k = (torch.randn(ctx_lens[s], Hkv, hd, generator=g)).to(dtype)
+        v = (torch.randn(ctx_lens[s], Hkv, hd, generator=g)).to(dtype)
+        ks.append(k)
+        vs.append(v)
+        for lp in range(n_pages_per[s]):
+            pg = perm[nxt]
+            nxt += 1
+            bt[s, lp] = pg
+            a, b = lp * page, min((lp + 1) * page, ctx_lens[s])
+            kc[pg, :, :b - a] = k[a:b].transpose(0, 1)
+            vc[pg, :, :b - a] = v[a:b].transpose(0, 1)
+    tok_seq, tok_pos = [], []
+    for s in range(n_seqs):
+        for i in range(q_lens[s]):
+            tok_seq.append(s)
+            tok_pos.append(ctx_lens[s] - q_lens[s] + i)
+    n = len(tok_seq)
+    q = torch.randn(n, H * hd + 16, generator=g).to(dtype)  # wider than the heads: a strided view
+    return dict(q=q, kc=kc, vc=vc, bt=bt, tok_seq=tok_seq, tok_pos=tok_pos, ks=ks, vs=vs, n=n)
+
+
+def attention_reference(case, H, Hkv, hd, scale, window=0):
+    out = torch.zeros(case["n"], H * hd, dtype=torch.float64)
+    for t, (s, p) in enumerate(zip(case["tok_seq"], case["tok_pos"])):
+        first = max(0, p - window + 1) if window > 0 else 0
+        for h in range(H):
+            hk = h // (H // Hkv)
+            qv = case["q"][t, h * hd:(h + 1) * hd].double()
+            k = case["ks"][s][first:p + 1, hk].double()
+            v = case["vs"][s][first:p + 1, hk].double()
+            w = torch.softmax((k @ qv) * scale, dim=0)
+            out[t, h * hd:(h + 1) * hd] = w @ v
+    return out
+
+
+def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=None):
+    dev = lambda x: x.to(DEV)  # noqa: E731
+    q, kc, vc, bt = dev(case["q"]), dev(case["kc"]), dev(case["vc"]), dev(case["bt"])
+    tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor(case["tok_pos"], dtype=torch.int32, device=DEV)
+    out = torch.zeros(case["n"], H * hd, dtype=q.dtype, device=DEV)
+    qv = q[:, :H * hd]
+    if kernel == "generic":
+        ops.attention_generic(out, qv, kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window)
+    elif kernel == "decode":
+        partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
+        tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
+        ops.attention_decode(out, qv, kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
+                             n_splits=splits, partials=partials, tok_list=tl,
+                             n_tokens=len(tok_list) if tok_list is not None else None)
+    return out
+
+
+ATT_CASES = [
+    # ctx_lens, q_lens, H, Hkv, hd, page
+    ([1, 17, 300], [1, 1, 1], 4, 4, 16, 16),
+    ([40, 129, 5], [7, 1, 5], 3, 3, 32, 16),
+    ([700, 64], [1, 64], 5, 5, 64, 64),
+    ([33, 257], [2, 3], 6, 2, 48, 8),
+    ([100], [100], 2, 1, 128, 16),
+    ([90, 31], [1, 1], 2, 2, 256, 16),
+    ([50, 3], [4, 3], 3, 3, 80, 4),
+]
+
+
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
+def test_attention_generic(ops, case_id, dtype, window):
+    ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, dtype, seed=case_id)
+    scale = 0.7 / math.sqrt(hd)
+    out = run_attention(ops, case, H, hd, scale, window, "generic")
+    close(out, attention_reference(case, H, Hkv, hd, scale, window), 2e-6 if dtype == torch.float32 else 8e-3, "generic")
+
+
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("splits", [1, 2, 5, 32])
+@pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
+def test_attention_decode(ops, case_id, splits, window):
+    ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
+    scale = 0.7 / math.sqrt(hd)
+    out = run_attention(ops, case, H, hd, scale, window, "decode", splits)
+    assert torch.isfinite(out.float()).all()
+    close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, f"decode splits={splits}")
+    # a subset of the rows through tok_list: the others stay untouched
+    if case["n"] > 2:
+        rows = list(range(case["n"]))[::2]
+        part = run_attention(ops, case, H, hd, scale, window, "decode", splits, tok_list=rows)
+        assert torch.equal(part[rows], out[rows]) and (part[1::2] == 0).all()
+
+
+@pytest.mark.parametrize("kernel", ["generic", "decode"])
+def test_attention_finds_one_far_key(ops, kernel):
+    """Random values average a wrong key away; here one key's score stands out, at a page's
+    first and last slot, in the first page and the last, and the output must be its value row."""
+    H = Hkv = 2
+    hd, page, T = 64, 16, 700
+    for target in (0, 15, 16, 17, 255, 256, 511, 512, 687, 688, 698, 699):
+        case = paged_case(1, [T], [1], H, Hkv, hd, page, torch.bfloat16, seed=target)
+        qv = case["q"][0, :hd].float()
+        k = case["ks"][0]
+        k[target, 0] = (qv * 4).to(torch.bfloat16)  # head 0: score ~ 4 |q|^2 ~ 250, all others ~ N(0, 8)
+        lp, off = divmod(target, page)
+        case["kc"][case["bt"][0, lp], 0, off] = k[target, 0]
+        out = run_attention(ops, case, H, hd, 1.0, 0, kernel, splits=3 if kernel == "decode" else 1)
+        want = case["vs"][0][target, 0].float()
+        assert torch.allclose(out[0, :hd].float().cpu(), want, atol=2e-2), f"{kernel}: key {target} was not found"
