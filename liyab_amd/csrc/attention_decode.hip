@@ -2,7 +2,7 @@
 // over paged bfloat16 keys and values, with the keys of a token cut into
 // splits so that few tokens still fill the chip.
 //
-// Grid (token, query head, split). A workgroup of 4 waves walks its split's
+// Grid (token, query head, split). A workgroup of 4 or 16 waves walks its split's
 // keys; LPK lanes share a key (each holds 8 consecutive dimensions, 16
 // bytes), so a wave takes 64 / LPK keys a pass, read straight from the pages
 // through the block table. Each lane group keeps a running maximum, sum and
@@ -19,8 +19,6 @@ namespace liyab {
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-constexpr int AD_WAVES = 4;
-constexpr int AD_U = 4;  // keys per lane group and trip
 
 __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
 #pragma unroll
@@ -46,7 +44,7 @@ __device__ __forceinline__ void merge_partial(Partial& a, float mo, float lo, co
     a.m = M;
 }
 
-template <int LPK>
+template <int LPK, int AD_WAVES, int AD_U>
 __global__ void __launch_bounds__(64 * AD_WAVES)
 attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -196,8 +194,8 @@ using namespace liyab;
 extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                       const void* vc, const int* block_tables, int max_blocks, const int* tok_list,
                                       const int* tok_seq, const int* tok_pos, int n, float scale, int window,
-                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, float* partials,
-                                      hipStream_t stream) {
+                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
+                                      float* partials, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
     LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
     LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
@@ -209,16 +207,24 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
                   "attention_decode: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
     LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
+    LIYAB_REQUIRE(waves == 4 || waves == 16, "attention_decode: %d waves per workgroup is not 4 or 16", waves);
     if (n == 0) return 0;
     dim3 grid(n, n_head, n_splits);
     auto* o = static_cast<bf16_t*>(out);
     auto* pq = static_cast<const bf16_t*>(q);
     auto* pk = static_cast<const bf16_t*>(kc);
     auto* pv = static_cast<const bf16_t*>(vc);
-#define LIYAB_GO(L)                                                                                                   \
-    attention_decode_kernel<L><<<grid, 64 * AD_WAVES, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
-                                                                   max_blocks, tok_list, tok_seq, tok_pos, scale,    \
-                                                                   window, n_head, n_kv_head, hd, page_size, n_splits, partials)
+#define LIYAB_GO(L)                                                                                                  \
+    do {                                                                                                             \
+        if (waves == 4)                                                                                              \
+            attention_decode_kernel<L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                    max_blocks, tok_list, tok_seq, tok_pos, scale,   \
+                                                                    window, n_head, n_kv_head, hd, page_size, n_splits, partials); \
+        else                                                                                                         \
+            attention_decode_kernel<L, 16, 8><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                      max_blocks, tok_list, tok_seq, tok_pos, scale, \
+                                                                      window, n_head, n_kv_head, hd, page_size, n_splits, partials); \
+    } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);
     else if (hd <= 32) LIYAB_GO(4);

@@ -123,11 +123,19 @@ int launch_mfma(const void* a, int64_t lda, const void* w, int M, int N, int K, 
     auto* pw = static_cast<const bf16_t*>(w);
     if (epi.mode == kEpiResidual || epi.out_dtype == kF32) {
         auto kern = gemm_mfma_kernel<BM, BN, float>;
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        static bool ready = false;  // once per instantiation, outside any stream capture's first use
+        if (!ready) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+            ready = true;
+        }
         kern<<<grid, 256, smem, stream>>>(pa, lda, pw, M, N, K, epi);
     } else {
         auto kern = gemm_mfma_kernel<BM, BN, bf16_t>;
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        static bool ready = false;
+        if (!ready) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+            ready = true;
+        }
         kern<<<grid, 256, smem, stream>>>(pa, lda, pw, M, N, K, epi);
     }
     return check_launch("gemm_mfma");

@@ -1,17 +1,24 @@
-// out[M,N] = a[M,K] . w[N,K]^T in bfloat16 for steps of few tokens (M <= 16):
+// out[M,N] = a[M,K] . w[N,K]^T in bfloat16 for steps of few tokens (M <= 64):
 // decoding, where the product is a stream of the weights.
 //
-// A workgroup owns 16 output features (16 rows of `w`) and all M tokens; its
-// waves split K and add their partial sums through LDS in wave order. With
-// v_mfma_f32_16x16x32_bf16 the weights are the first operand (16 rows) and
-// the tokens the second (up to 16), so the accumulator is the transposed
-// output tile. A lane holds 8 consecutive k of its row per instruction; here
-// each lane reads a run of 16 consecutive k (32 bytes) and feeds two
-// instructions, and both operands use the same assignment of k to (lane
-// group, instruction), which a dot product does not mind. Weights are read
-// once, straight from global memory into registers, 16 bytes a lane; the
-// tokens' rows come from L2. K must be a multiple of 8. The order of the sum
-// depends on K and the split only, never on M.
+// A workgroup owns 16 * NT output features (rows of `w`) and all M tokens as
+// MT tiles of 16; its waves split K and add their partial sums through LDS in
+// wave order. With v_mfma_f32_16x16x32_bf16 the weights are the first
+// operand (16 rows) and the tokens the second (16), so an accumulator is a
+// transposed output tile. A lane holds 8 consecutive k of its row per
+// instruction; here each lane reads a run of 16 consecutive k (32 bytes) and
+// feeds two instructions, and both operands use the same assignment of k to
+// (lane group, instruction), which a dot product does not mind. Weights are
+// read once, straight from global memory into registers, 16 bytes a lane,
+// one trip ahead of the multiplies; the tokens' rows come from L2 (every
+// workgroup reads all of them: few, wide tiles of N would starve most CUs).
+// K must be a multiple of 8. The order of the sum depends on K and the split
+// only, never on M.
+//
+// A LayerNorm may be folded into the first operand (M <= 16): the rows are
+// read from the 32-bit residual stream, normalised and written to LDS in
+// bfloat16 by the workgroup itself, a wave per row with its statistics in
+// registers (two passes, 32-bit, as the standalone kernel computes them).
 #include "common.h"
 #include "epilogue.h"
 
@@ -26,83 +33,211 @@ union Frag {
     bf16x8 v;
 };
 
-template <typename OutT, int KSPLIT>
-__global__ void __launch_bounds__(64 * KSPLIT)
+struct LnParams {
+    const float* x;      // [*, K] 32-bit rows; null: no norm, `a` holds bfloat16 rows
+    const float* weight; // [K] or null
+    const float* bias;   // [K] or null
+    const int* rows;     // [M] or null
+    float eps;
+};
+
+template <typename OutT, bool LN, int MT, int NT, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
-                   EpiParams epi) {
-    __shared__ float red[KSPLIT][256];
+                   EpiParams epi, LnParams ln) {
+    constexpr int UPT = (MT * NT == 1) ? 2 : 1;  // units of 64 k per trip
+    constexpr int TILES = MT * NT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int ksplit = blockDim.x / 64;
+    const int ldx = K + 8;
+    bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // LN: [M][K + 8]
+    float* red = reinterpret_cast<float*>(smem + (LN ? ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16 : 0));
+
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int i = lane % 16, g = lane / 16;
-    const int n0 = blockIdx.x * 16;
-    const bf16_t* wrow = w + static_cast<int64_t>(min(n0 + i, N - 1)) * K;
-    const bf16_t* arow = a + static_cast<int64_t>(min(i, M - 1)) * lda;
-    floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int n0 = blockIdx.x * 16 * NT;
     const int units = (K + 63) / 64;
     const u32x4 zero = {0, 0, 0, 0};
-    int u = wave;
-    // two units per trip: eight 16-byte loads in flight per lane
-    for (; u + KSPLIT < units; u += 2 * KSPLIT) {
-        const int k0 = u * 64 + g * 16, k1 = (u + KSPLIT) * 64 + g * 16;
-        Frag w0, w1, w2, w3, x0, x1, x2, x3;
-        w0.u = *reinterpret_cast<const u32x4*>(wrow + k0);
-        w1.u = *reinterpret_cast<const u32x4*>(wrow + k0 + 8);
-        w2.u = k1 < K ? *reinterpret_cast<const u32x4*>(wrow + k1) : zero;
-        w3.u = k1 + 8 < K ? *reinterpret_cast<const u32x4*>(wrow + k1 + 8) : zero;
-        x0.u = *reinterpret_cast<const u32x4*>(arow + k0);
-        x1.u = *reinterpret_cast<const u32x4*>(arow + k0 + 8);
-        x2.u = k1 < K ? *reinterpret_cast<const u32x4*>(arow + k1) : zero;
-        x3.u = k1 + 8 < K ? *reinterpret_cast<const u32x4*>(arow + k1 + 8) : zero;
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, x0.v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, x1.v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2.v, x2.v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w3.v, x3.v, acc, 0, 0, 0);
-    }
-    for (; u < units; u += KSPLIT) {
-        const int k0 = u * 64 + g * 16;
-        Frag w0, w1, x0, x1;
-        w0.u = k0 < K ? *reinterpret_cast<const u32x4*>(wrow + k0) : zero;
-        w1.u = k0 + 8 < K ? *reinterpret_cast<const u32x4*>(wrow + k0 + 8) : zero;
-        x0.u = k0 < K ? *reinterpret_cast<const u32x4*>(arow + k0) : zero;
-        x1.u = k0 + 8 < K ? *reinterpret_cast<const u32x4*>(arow + k0 + 8) : zero;
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, x0.v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, x1.v, acc, 0, 0, 0);
-    }
-    // acc[r] = partial C^T[n = 4 g + r][m = i]
+    const bf16_t* wrow[NT];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][i * 16 + 4 * g + r] = acc[r];  // [m][n]
+    for (int t = 0; t < NT; ++t) wrow[t] = w + static_cast<int64_t>(min(n0 + 16 * t + i, N - 1)) * K;
+
+    // unit u covers k in [64 u, 64 u + 64); this lane's run starts at 64 u + 16 g
+    auto load_w = [&](int u0, Frag (&f)[UPT][NT][2]) {
+#pragma unroll
+        for (int p = 0; p < UPT; ++p) {
+            const int u = u0 + p * ksplit, k = u * 64 + g * 16;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                f[p][t][0].u = (u < units && k < K) ? *reinterpret_cast<const u32x4*>(wrow[t] + k) : zero;
+                f[p][t][1].u = (u < units && k + 8 < K) ? *reinterpret_cast<const u32x4*>(wrow[t] + k + 8) : zero;
+            }
+        }
+    };
+    Frag wc[UPT][NT][2];
+    load_w(wave, wc);  // issued before the norm's prologue, so the two overlap
+
+    const bf16_t* arow[MT];
+    if constexpr (LN) {
+        constexpr int MAXV = 32;  // K <= 64 * MAXV
+        for (int m = wave; m < M; m += ksplit) {
+            const float* xr = ln.x + static_cast<int64_t>(ln.rows != nullptr ? ln.rows[m] : m) * K;
+            float v[MAXV], gw[MAXV], gb[MAXV];
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j) {
+                if (64 * j >= K) break;
+                const int k = lane + 64 * j;
+                const bool in = k < K;
+                v[j] = in ? xr[k] : 0.0f;
+                gw[j] = (in && ln.weight != nullptr) ? ln.weight[k] : 1.0f;
+                gb[j] = (in && ln.bias != nullptr) ? ln.bias[k] : 0.0f;
+                sum += v[j];
+            }
+            const float mean = wave_sum(sum) / static_cast<float>(K);
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j) {
+                if (64 * j >= K) break;
+                const float dev = lane + 64 * j < K ? v[j] - mean : 0.0f;
+                ss += dev * dev;
+            }
+            const float rstd = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(K) + ln.eps);
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j) {
+                if (64 * j >= K) break;
+                const int k = lane + 64 * j;
+                if (k < K) xs[m * ldx + k] = float_to_bf16((v[j] - mean) * rstd * gw[j] + gb[j]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < MT; ++s) arow[s] = xs + min(16 * s + i, M - 1) * ldx;
+    } else {
+#pragma unroll
+        for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(16 * s + i, M - 1)) * lda;
+    }
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int s = 0; s < MT; ++s)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[s][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int u0 = wave; u0 < units; u0 += UPT * ksplit) {
+        Frag wn[UPT][NT][2];
+        load_w(u0 + UPT * ksplit, wn);
+#pragma unroll
+        for (int p = 0; p < UPT; ++p) {
+            const int u = u0 + p * ksplit, k = u * 64 + g * 16;
+            Frag x[MT][2];
+#pragma unroll
+            for (int s = 0; s < MT; ++s) {
+                x[s][0].u = (u < units && k < K) ? *reinterpret_cast<const u32x4*>(arow[s] + k) : zero;
+                x[s][1].u = (u < units && k + 8 < K) ? *reinterpret_cast<const u32x4*>(arow[s] + k + 8) : zero;
+            }
+#pragma unroll
+            for (int s = 0; s < MT; ++s)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, x[s][0].v, acc[s][t], 0, 0, 0);
+                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, x[s][1].v, acc[s][t], 0, 0, 0);
+                }
+        }
+#pragma unroll
+        for (int p = 0; p < UPT; ++p)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                wc[p][t][0] = wn[p][t][0];
+                wc[p][t][1] = wn[p][t][1];
+            }
+    }
+    // acc[s][t][r] = partial C^T[n = 16 t + 4 g + r][m = 16 s + i]; kept [tile][m][n] per wave
+#pragma unroll
+    for (int s = 0; s < MT; ++s)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[(wave * TILES + s * NT + t) * 256 + i * 16 + 4 * g + r] = acc[s][t][r];
     __syncthreads();
-    for (int t = tid; t < 256; t += 64 * KSPLIT) {
-        const int m = t / 16, n = n0 + t % 16;
+    for (int e = tid; e < TILES * 256; e += blockDim.x) {
+        const int tile = e / 256, s = tile / NT, t = tile % NT;
+        const int m = 16 * s + (e % 256) / 16, n = n0 + 16 * t + e % 16;
         float v = 0.0f;
-#pragma unroll
-        for (int s = 0; s < KSPLIT; ++s) v += red[s][t];
+        for (int q = 0; q < ksplit; ++q) v += red[q * TILES * 256 + e];
         if (m < M && n < N) epilogue_store<OutT>(epi, m, n, v);
     }
 }
 
-template <int KSPLIT>
-int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
-    const int grid = (N + 15) / 16;
+template <bool LN, int MT, int NT, int MAXW>
+int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, const EpiParams& epi,
+                  const LnParams& ln, hipStream_t stream) {
+    const int grid = (N + 16 * NT - 1) / (16 * NT);
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
-    if (epi.mode == kEpiResidual || epi.out_dtype == kF32) {
-        gemm_skinny_kernel<float, KSPLIT><<<grid, 64 * KSPLIT, 0, stream>>>(pa, lda, pw, M, N, K, epi);
+    if (ksplit > MAXW) ksplit = MAXW;
+    size_t smem = static_cast<size_t>(ksplit) * MT * NT * 256 * sizeof(float);
+    if (LN) smem += ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16;
+    const bool f32 = epi.mode == kEpiResidual || epi.out_dtype == kF32;
+    if (f32) {
+        auto kern = gemm_skinny_kernel<float, LN, MT, NT, MAXW>;
+        static bool ready = false;
+        if (!ready) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            ready = true;
+        }
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln);
     } else {
-        gemm_skinny_kernel<bf16_t, KSPLIT><<<grid, 64 * KSPLIT, 0, stream>>>(pa, lda, pw, M, N, K, epi);
+        auto kern = gemm_skinny_kernel<bf16_t, LN, MT, NT, MAXW>;
+        static bool ready = false;
+        if (!ready) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            ready = true;
+        }
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln);
     }
     return check_launch("gemm_skinny");
+}
+
+static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide,
+                           const EpiParams& epi, const LnParams& ln, hipStream_t stream) {
+    const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    // wide tiles of N (64 features a workgroup) when N is so large that every workgroup
+    // re-reading the tokens would cost more than the weights
+    if (wide < 0) wide = (mt > 1 && static_cast<long>(N) * M > (1L << 20)) ? 1 : 0;
+    const int nt = wide ? 4 : 1;
+    if (ksplit == 0) {
+        // enough waves to cover the chip several times over, each with at least 128 k
+        const int tiles = (N + 16 * nt - 1) / (16 * nt), units = (K + 63) / 64;
+        ksplit = 1;
+        while (ksplit < 16 && tiles * ksplit < 2048 && units / (ksplit * 2) >= (mt * nt == 1 ? 2 : 1)) ksplit *= 2;
+        // a folded norm takes a wave per row: as many waves as rows, so the rows go side by side
+        if (ln.x != nullptr) ksplit = 8;
+    }
+    LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || ksplit == 4 || ksplit == 8 || ksplit == 16,
+                  "gemm_skinny: ksplit %d is not 1, 2, 4, 8 or 16", ksplit);
+    if (ln.x != nullptr) return launch_skinny<true, 1, 1, 8>(a, lda, w, M, N, K, ksplit, epi, ln, stream);  // 8 waves: registers for a row's values
+    if (nt == 1) {
+        if (mt == 1) return launch_skinny<false, 1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+        if (mt == 2) return launch_skinny<false, 2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+        return launch_skinny<false, 4, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+    }
+    if (mt == 1) return launch_skinny<false, 1, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+    if (mt == 2) return launch_skinny<false, 2, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+    return launch_skinny<false, 4, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
 }
 
 }  // namespace liyab
 
 using namespace liyab;
 
-// a [M <= 16, K] and w [N, K] are bfloat16. ksplit: waves per workgroup sharing K (0 = chosen
-// from the shape; 1, 2, 4, 8 or 16).
-extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit,
+// a [M <= 64, K] and w [N, K] are bfloat16. ksplit: waves per workgroup sharing K (0 = chosen
+// from the shape; 1, 2, 4, 8 or 16). wide: 64 instead of 16 output features a workgroup
+// (-1 = chosen from the shape).
+extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide,
                                  const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
-    LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d (at most 16) N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d (at most 64) N=%d K=%d", M, N, K);
     LIYAB_REQUIRE(K % 8 == 0 && lda % 8 == 0 && lda >= K, "gemm_skinny: K %d and lda %lld must be multiples of 8", K,
                   static_cast<long long>(lda));
     LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0,
@@ -110,18 +245,22 @@ extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int 
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
-    if (ksplit == 0) {
-        // enough waves to cover the chip several times over, each with at least 128 k
-        const int tiles = (N + 15) / 16, units = (K + 63) / 64;
-        ksplit = 1;
-        while (ksplit < 16 && tiles * ksplit < 2048 && units / (ksplit * 2) >= 2) ksplit *= 2;
-    }
-    switch (ksplit) {
-        case 1: return launch_skinny<1>(a, lda, w, M, N, K, epi, stream);
-        case 2: return launch_skinny<2>(a, lda, w, M, N, K, epi, stream);
-        case 4: return launch_skinny<4>(a, lda, w, M, N, K, epi, stream);
-        case 8: return launch_skinny<8>(a, lda, w, M, N, K, epi, stream);
-        case 16: return launch_skinny<16>(a, lda, w, M, N, K, epi, stream);
-        default: return fail(1, "gemm_skinny: ksplit %d is not 1, 2, 4, 8 or 16", ksplit);
-    }
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream);
+}
+
+// The same product with a LayerNorm folded in: the first operand is LayerNorm(x[rows[m] or m])
+// of the 32-bit rows x [*, K]. M <= 16, K <= 2048, and M * (K + 8) * 2 bytes must fit 64 KiB of LDS.
+extern "C" int liyab_gemm_skinny_ln(const float* x, const float* ln_weight, const float* ln_bias, const int* rows,
+                                    float eps, const void* w, int M, int N, int K, int ksplit,
+                                    const EpiParams* epi_in, hipStream_t stream) {
+    LIYAB_REQUIRE(x && w && epi_in, "gemm: null operand");
+    LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 16) N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(K % 8 == 0 && K <= 2048, "gemm_skinny_ln: K %d must be a multiple of 8, at most 2048", K);
+    LIYAB_REQUIRE(static_cast<size_t>(M) * (K + 8) * 2 <= 65536, "gemm_skinny_ln: %d rows of %d do not fit the LDS budget", M, K);
+    LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm_skinny_ln: weights must be 16-byte aligned");
+    LIYAB_REQUIRE(eps >= 0.0f, "gemm_skinny_ln: negative eps");
+    EpiParams epi = *epi_in;
+    if (int rc = check_epilogue(epi, M, N)) return rc;
+    if (M == 0) return 0;
+    return skinny_dispatch(nullptr, K + 8, w, M, N, K, ksplit, 0, epi, LnParams{x, ln_weight, ln_bias, rows, eps}, stream);
 }

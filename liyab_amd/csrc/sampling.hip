@@ -233,26 +233,70 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
     if (tid == 0) out[r] = result < 0 ? imax : result;
 }
 
-__global__ void __launch_bounds__(S_THREADS)
-argmax_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t ld, int V) {
-    __shared__ float redf[S_WAVES];
-    __shared__ int redi[S_WAVES];
-    float v;
-    int i;
-    block_argmax(logits + static_cast<int64_t>(blockIdx.x) * ld, V, v, i, redf, redi);
-    if (threadIdx.x == 0) out[blockIdx.x] = i;
+// Argmax in two stages so that a few rows still use many CUs: chunks of a row give partial
+// (value, id) pairs, then one wave per row picks among them; ties go to the lowest id.
+constexpr int AM_CHUNKS = 64;
+
+__global__ void __launch_bounds__(256)
+argmax_partial_kernel(float* __restrict__ pv, int* __restrict__ pi, const float* __restrict__ logits, int64_t ld, int V) {
+    __shared__ float redv[4];
+    __shared__ int redi[4];
+    const int r = blockIdx.x, c = blockIdx.y;
+    const int per = (V + AM_CHUNKS - 1) / AM_CHUNKS;
+    const int i0 = c * per, i1 = min(V, i0 + per);
+    const float* row = logits + static_cast<int64_t>(r) * ld;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = i0 + threadIdx.x; i < i1; i += 256) {
+        const float v = row[i];
+        if (v > bv) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (threadIdx.x % kWave == 0) { redv[threadIdx.x / kWave] = bv; redi[threadIdx.x / kWave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (redv[w] > bv || (redv[w] == bv && redi[w] < bi)) { bv = redv[w]; bi = redi[w]; }
+        pv[r * AM_CHUNKS + c] = bv;
+        pi[r * AM_CHUNKS + c] = bi;
+    }
+}
+
+__global__ void __launch_bounds__(64)
+argmax_final_kernel(int* __restrict__ out, const float* __restrict__ pv, const int* __restrict__ pi) {
+    const int r = blockIdx.x;
+    float bv = pv[r * AM_CHUNKS + threadIdx.x];
+    int bi = pi[r * AM_CHUNKS + threadIdx.x];
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
 }
 
 }  // namespace liyab
 
 using namespace liyab;
 
-extern "C" int liyab_argmax(int* out, const float* logits, int64_t ld, int rows, int V, hipStream_t stream) {
-    LIYAB_REQUIRE(out && logits, "argmax: null pointer");
+// scratch_v / scratch_i: rows * 64 floats / ints of workspace.
+extern "C" int liyab_argmax(int* out, const float* logits, int64_t ld, int rows, int V, float* scratch_v,
+                            int* scratch_i, hipStream_t stream) {
+    LIYAB_REQUIRE(out && logits && scratch_v && scratch_i, "argmax: null pointer");
     LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d", rows, V);
+    LIYAB_REQUIRE(rows <= 65535 * 16, "argmax: too many rows");
     if (rows == 0) return 0;
-    argmax_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V);
-    return check_launch("argmax");
+    static_assert(AM_CHUNKS == kWave, "the final stage is one wave over the chunks");
+    argmax_partial_kernel<<<dim3(rows, AM_CHUNKS), 256, 0, stream>>>(scratch_v, scratch_i, logits, ld, V);
+    if (int rc = check_launch("argmax_partial")) return rc;
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(out, scratch_v, scratch_i);
+    return check_launch("argmax_final");
 }
 
 // Per-row parameters; a row with temperature <= 0 is greedy. top_k <= 0 and

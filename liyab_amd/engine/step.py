@@ -66,8 +66,25 @@ class _Staging:
         ev.record()
 
 
+DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
+
+
+def _bucket(n: int, least: int = 256) -> int:
+    b = least
+    while b < n:
+        b *= 2
+    return b
+
+
 class StepFunction:
-    def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0"):
+    """`use_graphs`: a step whose shape (tokens, requests, wanted rows, attention mode,
+    context bucket) has been seen before is captured into a HIP graph the second time and
+    replayed from then on; what varies between such steps lives in the metadata block, whose
+    address and layout the shape fixes. Kernels must then depend on the host only through
+    the shape: the ones in this package do."""
+
+    def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0", use_graphs: bool = True,
+                 max_graphs: int = 64):
         self.model = model
         self.manager = manager
         self.storage = storage
@@ -77,6 +94,11 @@ class StepFunction:
         self._meta_dev: Optional[torch.Tensor] = None
         self.steps = 0
         self.tokens = 0
+        self.use_graphs = use_graphs
+        self.max_graphs = max_graphs
+        self._graphs = {}  # shape -> (graph, logits) once captured, or the count of eager runs
+        self.graph_replays = 0
+        self._graph_generation = 0
 
     # -- validation -----------------------------------------------------------
     def _validate(self, items: Sequence[StepItem]) -> None:
@@ -103,6 +125,39 @@ class StepFunction:
             if end > self.model.max_positions:
                 raise ContextFull(
                     f"position {end - 1} is past the model's {self.model.max_positions} learned positions")
+
+    # -- eager or replayed ----------------------------------------------------
+    def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        if not self.use_graphs:
+            return self.model.forward(ctx, self.storage)
+        if self.workspace.generation != self._graph_generation:
+            # a workspace buffer moved since the graphs were captured: they hold its old address
+            self._graphs.clear()
+            self._graph_generation = self.workspace.generation
+        key = (ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows, ctx.host.attention_mode, ctx.host.context_bucket)
+        entry = self._graphs.get(key)
+        if isinstance(entry, tuple):
+            entry[0].replay()
+            self.graph_replays += 1
+            return entry[1]
+        if entry is None:
+            # first sight: run eagerly, which also sizes every workspace buffer for this shape
+            if len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            self._graphs[key] = 1
+            return self.model.forward(ctx, self.storage)
+        before = self.workspace.generation
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx, self.storage)
+        if self.workspace.generation != before:
+            # a buffer grew during capture: its old address is baked into the graph; run eagerly
+            self._graphs[key] = 1
+            return self.model.forward(ctx, self.storage)
+        self._graphs[key] = (graph, logits)
+        graph.replay()
+        self.graph_replays += 1
+        return logits
 
     # -- the step -------------------------------------------------------------
     def run(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
@@ -174,7 +229,10 @@ class StepFunction:
                 sl[a:b] = pages * page + p % page
 
         if self._meta_dev is None or self._meta_dev.numel() < total:
-            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+            # sized for the largest step of this engine's lifetime where possible: a new block
+            # would invalidate captured graphs
+            self._meta_dev = torch.empty(max(2 * total, 1 << 16), dtype=torch.int32, device=self.device)
+            self._graphs.clear()
         dev = self._meta_dev
         dev[:total].copy_(host_t[:total], non_blocking=True)
         self._staging.copied()
@@ -183,6 +241,7 @@ class StepFunction:
             o, size = off[name]
             return dev[o:o + size]
 
+        max_context = max(f + n for f, n in zip(first, q_lens))
         ctx = StepContext(
             n_tokens=N, n_seqs=S,
             token_ids=dview("token_ids"), positions=dview("positions"), tok_seq=dview("tok_seq"),
@@ -190,10 +249,12 @@ class StepFunction:
             logit_rows=dview("logit_rows"), n_logit_rows=R,
             groups=[GroupStep(block_tables=dview(f"bt{g}").view(S, W), slots=dview(f"slots{g}")) for g in range(G)],
             host=StepHost(q_lens=q_lens, starts=[int(s) for s in starts[:-1]], first_pos=first,
-                          max_q_len=max(q_lens), max_context=max(f + n for f, n in zip(first, q_lens))),
+                          max_q_len=max(q_lens), max_context=max_context,
+                          attention_mode="decode" if max(q_lens) <= DECODE_Q_LEN else "prefill",
+                          context_bucket=_bucket(max_context)),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
         )
-        logits = self.model.forward(ctx, self.storage)
+        logits = self._forward(ctx)
         for it, f, n in zip(items, first, q_lens):
             mgr.commit(it.rid, f + n)
         self.steps += 1

@@ -224,13 +224,23 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
               tok_pos.data_ptr(), n, float(scale), int(window), n_head, hkv, hd, page, _stream())
 
 
+_argmax_scratch = {}
+
+
 def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
+    """out[r] = the first maximal element of logits[r] (ties go to the lowest id)."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
     if logits.dtype != torch.float32:
         raise KernelError("argmax: logits must be float32")
     _i32(out, "out", rows)
-    _lib.call("liyab_argmax", out.data_ptr(), logits.data_ptr(), ld, rows, V, _stream())
+    key = logits.device
+    sc = _argmax_scratch.get(key)
+    if sc is None or sc[0].numel() < rows * 64:
+        cap = max(rows, 64) * 64
+        sc = (torch.empty(cap, dtype=torch.float32, device=key), torch.empty(cap, dtype=torch.int32, device=key))
+        _argmax_scratch[key] = sc
+    _lib.call("liyab_argmax", out.data_ptr(), logits.data_ptr(), ld, rows, V, sc[0].data_ptr(), sc[1].data_ptr(), _stream())
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
@@ -300,17 +310,50 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *,
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
-                epilogue: int = EPI_NONE, kv=None, ksplit: int = 0) -> None:
-    """The weight-streaming product for at most 16 bfloat16 rows, K a multiple of 8."""
+                epilogue: int = EPI_NONE, kv=None, ksplit: int = 0, wide: int = -1) -> None:
+    """The weight-streaming product for at most 64 bfloat16 rows, K a multiple of 8."""
     lda = _rows(a, "a")
     M, K = a.shape
     _dev(w, "w")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
         raise KernelError(f"gemm_skinny: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
-    if M > 16:
-        raise KernelError(f"gemm_skinny: {M} rows; it takes at most 16")
+    if M > 64:
+        raise KernelError(f"gemm_skinny: {M} rows; it takes at most 64")
     e = _epilogue(a, w, bias, out, residual, epilogue, kv)
-    _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, ctypes.byref(e), _stream())
+    _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, wide, ctypes.byref(e), _stream())
+
+
+def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,
+                   w: torch.Tensor, bias: Optional[torch.Tensor], *, rows: Optional[torch.Tensor] = None,
+                   n_rows: Optional[int] = None, out=None, residual=None, epilogue: int = EPI_NONE, kv=None,
+                   ksplit: int = 0) -> None:
+    """gemm_skinny over LayerNorm(x[rows[m] or m]) of the float32 rows x [*, K], the norm computed
+    inside the product kernel."""
+    _dev(x, "x")
+    _dev(w, "w")
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("gemm_skinny_ln: x must be contiguous float32 [*, K]")
+    K = x.shape[1]
+    M = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_skinny_ln: needs contiguous bfloat16 w [N, {K}], got {tuple(w.shape)} {w.dtype}")
+    if not skinny_ln_takes(M, K, 0):
+        raise KernelError(f"gemm_skinny_ln: {M} rows of {K} are outside what it takes")
+    _f32vec(ln_weight, "norm weight", K)
+    _f32vec(ln_bias, "norm bias", K)
+    if rows is not None:
+        _i32(rows, "rows", M)
+    fake_a = torch.empty((M, 0), dtype=torch.bfloat16, device="meta")  # shapes only, for the epilogue's checks
+    e = _epilogue(fake_a, w, bias, out, residual, epilogue, kv)
+    e.exact = 0
+    _lib.call("liyab_gemm_skinny_ln", x.data_ptr(), _ptr(ln_weight), _ptr(ln_bias), _ptr(rows), float(eps),
+              w.data_ptr(), M, w.shape[0], K, ksplit, ctypes.byref(e), _stream())
+
+
+def skinny_ln_takes(M: int, K: int, N: int = 0) -> bool:
+    """Every workgroup (16 output features) repeats the norm of all rows, so it pays only while
+    the product has few workgroups."""
+    return 0 < M <= 16 and K % 8 == 0 and K <= 2048 and M * (K + 8) * 2 <= 65536 and N <= 8192
 
 
 def mfma_takes(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -324,8 +367,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
     the plain tiled kernel for float32 and everything else. `kv` = (k_cache, v_cache, slots,
     q_dim) with the paged QKV epilogue."""
     if mfma_takes(a, w):
-        if a.shape[0] <= 16:
-            gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
+        M, N = a.shape[0], w.shape[0]
+        if M <= 16 or (M <= 64 and N <= 8192):
+            # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
+            # kernel's shared loads beat every workgroup re-reading the tokens)
+            gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=0)
         else:
             gemm_mfma(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
         return
@@ -339,7 +385,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
-                     tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None) -> None:
+                     tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4) -> None:
     """Each token on its own over its request's bfloat16 cache, its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
@@ -367,13 +413,18 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
-              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, _ptr(partials), _stream())
+              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, _ptr(partials), _stream())
 
 
-def decode_splits(n_tokens: int, n_head: int, max_context: int) -> int:
-    """How many splits of the keys give the chip enough workgroups without making them tiny."""
-    groups = max(1, n_tokens * n_head)
-    return max(1, min(-(-1024 // groups), max_context // 128, 32))
+def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
+    """(splits of the keys, waves per workgroup), from measurements at 12 heads of 64: with many
+    (token, head) pairs a workgroup of 4 waves per pair is fastest; with few, 16 waves per pair,
+    merged in LDS, beat cutting the keys across workgroups plus a merge kernel up to a few
+    thousand keys; beyond that the keys are also split across workgroups."""
+    pairs = max(1, n_tokens * n_head)
+    if pairs >= 512 or context_bucket <= 256:
+        return 1, 4
+    return max(1, min(context_bucket // 2048, 32)), 16
 
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -381,14 +432,14 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
     is chosen from the step's shape (`ctx` is the step's StepContext)."""
     hd = k_cache.shape[3]
-    if q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and ctx.host.max_q_len <= 8:
+    if q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and ctx.host.attention_mode == "decode":
         n = out.shape[0]
-        splits = decode_splits(n, n_head, ctx.host.max_context)
+        splits, waves = decode_plan(n, n_head, ctx.host.context_bucket)
         partials = None
         if splits > 1:
             partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 2),), torch.float32)
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
-                         scale=scale, window=window, n_splits=splits, partials=partials)
+                         scale=scale, window=window, n_splits=splits, partials=partials, waves=waves)
         return
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)

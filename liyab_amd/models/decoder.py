@@ -81,7 +81,9 @@ class DecoderModel:
         if ctx.n_logit_rows == 0:
             return None
         if self.final_norm is not None:
-            h = self.final_norm.forward(x, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logit_rows, name="head_in")
+            norm = self.final_norm
+            kw = dict(rows=ctx.logit_rows, n_rows=ctx.n_logit_rows, name="head_in")
+            h = norm.lazy(x, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(x, ctx, **kw)
         else:
             raise NotImplementedError("a model without a final norm is not implemented")
         return self.head.forward(h, ctx)

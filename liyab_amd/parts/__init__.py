@@ -12,4 +12,5 @@ from .registry import (  # noqa: F401
     register_norm,
     register_position,
 )
+from .norms import Normed, as_tensor  # noqa: F401
 from . import attention, block, embeddings, feedforward, head, norms  # noqa: F401  (register themselves)

@@ -10,7 +10,7 @@ from ..cache.pages import KVSpec
 from ..cache.storage import LayerCache
 from ..kernels import ops
 from .base import StepContext
-from .linear import linear
+from .linear import linear, paged_qkv_takes
 from .registry import register_mixer
 
 
@@ -55,11 +55,10 @@ class Attention:
         n = h.shape[0]
         ws = ctx.workspace
         group = ctx.groups[cache.group]
-        if writes_cache and ops.mfma_takes(h, self.qkv_weight):
+        if writes_cache and paged_qkv_takes(self.dtype, self.width):
             # the projection's epilogue puts keys and values straight into their pages
             q = ws.get("q", (n, self.q_dim), self.dtype)
-            ops.gemm(h, self.qkv_weight, self.qkv_bias, out=q, epilogue=ops.EPI_QKV_PAGED,
-                     kv=(cache.k, cache.v, group.slots, self.q_dim))
+            linear(h, self.qkv_weight, self.qkv_bias, out=q, kv=(cache.k, cache.v, group.slots, self.q_dim))
         else:
             q = ws.get("qkv", (n, self.q_dim + 2 * self.kv_dim), self.dtype)
             linear(h, self.qkv_weight, self.qkv_bias, out=q)

@@ -36,6 +36,7 @@ class Workspace:
     def __init__(self, device):
         self.device = torch.device(device)
         self._bufs: Dict[str, torch.Tensor] = {}
+        self.generation = 0  # counts reallocations: captured graphs hold the old addresses
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -48,6 +49,7 @@ class Workspace:
             if buf is not None:
                 cap = max(cap, 2 * buf.numel())
             buf = torch.empty(cap, dtype=dtype, device=self.device)
+            self.generation += 1
             self._bufs[key] = buf
         return buf[:n].view(*shape)
 
@@ -72,6 +74,8 @@ class StepHost:
     first_pos: List[int]  # position of each request's first token
     max_q_len: int
     max_context: int  # longest context after this step
+    attention_mode: str = "prefill"  # "decode": every request brings few tokens, each taken on its own
+    context_bucket: int = 256  # max_context rounded up to a power of two: grids follow it, not the exact length
 
 
 @dataclass

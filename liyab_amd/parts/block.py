@@ -17,11 +17,17 @@ class PreNormBlock:
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True) -> None:
-        h = self.norm_mixer.forward(x, ctx)
+        h = self._normed(self.norm_mixer, x, ctx)
         self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
         if self.ffn is not None:
-            h = self.norm_ffn.forward(x, ctx)
+            h = self._normed(self.norm_ffn, x, ctx)
             self.ffn.forward(h, ctx, x)
+
+    @staticmethod
+    def _normed(norm, x, ctx):
+        """The norm's output, left pending when the norm allows it so that the next product
+        may fold it in (parts that need the rows call `as_tensor`)."""
+        return norm.lazy(x, ctx) if hasattr(norm, "lazy") else norm.forward(x, ctx)
 
 
 register_block("pre_norm", PreNormBlock)

@@ -26,7 +26,7 @@ class DenseFFN:
         self.down_weight = store.fetch(t["down_weight"], (self.width, self.inner), "matrix")
         self.down_bias = store.fetch(t["down_bias"], (self.width,), "vector") if "down_bias" in t else None
 
-    def forward(self, h: torch.Tensor, ctx: StepContext, residual: torch.Tensor) -> None:
+    def forward(self, h, ctx: StepContext, residual: torch.Tensor) -> None:
         inner = ctx.workspace.get("ffn_inner", (h.shape[0], self.inner), self.dtype)
         linear(h, self.up_weight, self.up_bias, out=inner, activation=self.activation)
         linear(inner, self.down_weight, self.down_bias, residual=residual)

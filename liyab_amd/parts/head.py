@@ -25,7 +25,7 @@ class LMHead:
         self.weight = store.fetch(t["weight"], (self.vocab_size, self.width), "table")
         self.bias = store.fetch(t["bias"], (self.vocab_size,), "vector") if "bias" in t else None
 
-    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    def forward(self, h, ctx: StepContext) -> torch.Tensor:
         logits = ctx.workspace.get("logits", (h.shape[0], self.vocab_size), torch.float32)
         linear(h, self.weight, self.bias, out=logits)
         return logits

@@ -3,7 +3,9 @@
 W is [out, in], a row per output feature, the layout the reference works in
 (include/liyab/types.h:165-184; y = x . W^T, include/liyab/backend.h:35).
 The kernel is chosen here by dtype and shape; callers only say what they
-want computed.
+want computed. The first operand may be a pending norm (`Normed`): when the
+kernel for this shape can apply the norm itself it does, otherwise the norm
+runs first as its own kernel.
 """
 
 from __future__ import annotations
@@ -13,12 +15,35 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
+from .norms import Normed
 
 
-def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
-           residual: Optional[torch.Tensor] = None, activation: str = "none") -> None:
-    """out = act(a . w^T + bias), or with `residual` given: residual += a . w^T + bias."""
+def _fuses(a, w: torch.Tensor) -> bool:
+    return (isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and w.dtype == torch.bfloat16
+            and a.x.dtype == torch.float32 and a.x.is_contiguous() and ops.skinny_ln_takes(a.n_rows, a.norm.width, w.shape[0]))
+
+
+def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
+           residual: Optional[torch.Tensor] = None, activation: str = "none", kv=None) -> None:
+    """out = act(a . w^T + bias); with `residual`: residual += a . w^T + bias; with `kv` =
+    (k_cache, v_cache, slots, q_dim): queries to `out`, keys and values into their pages."""
     if residual is not None:
-        ops.gemm(a, w, bias, residual=residual, epilogue=ops.EPI_RESIDUAL)
+        epilogue = ops.EPI_RESIDUAL
+    elif kv is not None:
+        epilogue = ops.EPI_QKV_PAGED
     else:
-        ops.gemm(a, w, bias, out=out, epilogue=ops.ACTIVATION_EPILOGUE[activation])
+        epilogue = ops.ACTIVATION_EPILOGUE[activation]
+    if _fuses(a, w):
+        n = a.norm
+        ops.gemm_skinny_ln(a.x, n.weight, n.bias, n.eps, w, bias, rows=a.rows, n_rows=a.n_rows, out=out,
+                           residual=residual, epilogue=epilogue, kv=kv)
+        return
+    if isinstance(a, Normed):
+        a = a.tensor()
+    ops.gemm(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
+
+
+def paged_qkv_takes(dtype: torch.dtype, k: int) -> bool:
+    """Whether the product kernels for this dtype and inner size can write keys and values
+    into cache pages from their epilogue."""
+    return dtype == torch.bfloat16 and k % 8 == 0

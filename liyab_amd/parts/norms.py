@@ -11,6 +11,35 @@ from .base import StepContext
 from .registry import register_norm
 
 
+class Normed:
+    """A norm's output that has not been computed yet: what a block hands to its mixer or
+    feed-forward. A product kernel that can apply the norm to its own first operand takes
+    it as it is (`linear` does); anything else calls `tensor()` and gets the rows."""
+
+    def __init__(self, norm, x: torch.Tensor, ctx: StepContext, rows=None, n_rows=None, name="normed"):
+        self.norm, self.x, self.ctx, self.rows, self.name = norm, x, ctx, rows, name
+        self.n_rows = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        self._tensor = None
+
+    @property
+    def shape(self):
+        return (self.n_rows, self.norm.width)
+
+    @property
+    def dtype(self):
+        return self.norm.dtype
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.norm.forward(self.x, self.ctx, rows=self.rows, n_rows=self.n_rows, name=self.name)
+        return self._tensor
+
+
+def as_tensor(h) -> torch.Tensor:
+    """The rows of a part's input, computing a pending norm if there is one."""
+    return h.tensor() if isinstance(h, Normed) else h
+
+
 class LayerNorm:
     """y = (x - mean) / sqrt(var + eps) * weight + bias over the last axis
     (the reference's layernorm, src/core/transformer.cpp:77-106); weight and
@@ -24,6 +53,12 @@ class LayerNorm:
         b = spec.tensors.get("bias")
         self.weight = store.fetch(w, (self.width,), "vector") if w is not None else None
         self.bias = store.fetch(b, (self.width,), "vector") if b is not None else None
+
+    fusable = "layernorm"  # product kernels know how to fold this norm into their operand
+
+    def lazy(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
+             n_rows: Optional[int] = None, name: str = "normed") -> Normed:
+        return Normed(self, x, ctx, rows, n_rows, name)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
                 n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:

@@ -107,19 +107,19 @@ def test_gemm_float32(ops, M, N, K, epilogue):
         assert torch.equal(one[0], full[M // 2])
 
 
-@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16"])
+@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
-@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600)])
 def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
     a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
     tiles = {"mfma128": 1, "mfma64": 2, "mfma128x64": 3}
 
-    if kernel.startswith("skinny") and M > 16:
-        pytest.skip("the skinny kernel takes at most 16 rows")
+    if kernel.startswith("skinny") and M > 64:
+        pytest.skip("the skinny kernel takes at most 64 rows")
 
     def run(**kw):
         if kernel.startswith("skinny"):
-            ops.gemm_skinny(a, w, bias, ksplit=int(kernel[6:]), **kw)
+            ops.gemm_skinny(a, w, bias, ksplit=int(kernel[6:].rstrip("w")), wide=1 if kernel.endswith("w") else 0, **kw)
         elif kernel == "simple":
             ops.gemm_simple(a, w, bias, **kw)
         elif kernel == "auto":
@@ -137,6 +137,30 @@ def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
             out = torch.empty(M, N, dtype=out_dtype, device=DEV)
             run(out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue])
             close(out, gemm_reference(a, w, bias, epilogue), tol, f"gemm bf16 {epilogue} {kernel} -> {out_dtype}")
+
+
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
+@pytest.mark.parametrize("M,N,K,eps", [(1, 64, 64, 1e-5), (8, 2304, 768, 1e-5), (16, 100, 1600, 1e-6), (5, 777, 144, 1e-5), (3, 50, 2048, 1e-3)])
+def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, epilogue):
+    x = rnd(M + 4, K, scale=2.0) + 0.5
+    lw, lb = rnd(K, seed=5) + 1.0, rnd(K, seed=6)
+    w, bias = rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    rows = torch.tensor([(3 * i + 1) % (M + 4) for i in range(M)], dtype=torch.int32, device=DEV)
+    for use_rows in (False, True):
+        src = x[rows.long()] if use_rows else x[:M]
+        h = torch.nn.functional.layer_norm(src.double(), (K,), lw.double(), lb.double(), eps).to(torch.bfloat16)
+        kw = dict(rows=rows) if use_rows else {}
+        xin = x if use_rows else x[:M].contiguous()
+        if epilogue == "residual":
+            res = rnd(M, N, seed=3)
+            want = gemm_reference(h, w, bias, epilogue, res)
+            ops.gemm_skinny_ln(xin, lw, lb, eps, w, bias, residual=res, epilogue=ops.EPI_RESIDUAL, **kw)
+            close(res, want, 2e-3, "gemm+ln residual")
+        else:
+            out = torch.empty(M, N, device=DEV)
+            ops.gemm_skinny_ln(xin, lw, lb, eps, w, bias, out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue], **kw)
+            # the folded norm rounds to bfloat16 where the standalone kernel does: allow one ulp of the operand
+            close(out, gemm_reference(h, w, bias, epilogue), 4e-3, f"gemm+ln {epilogue}")
 
 
 def test_gemm_strided_rows_and_refusals(ops):
@@ -212,7 +236,7 @@ def attention_reference(case, H, Hkv, hd, scale, window=0):
     return out
 
 
-def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=None):
+def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=None, waves=4):
     dev = lambda x: x.to(DEV)  # noqa: E731
     q, kc, vc, bt = dev(case["q"]), dev(case["kc"]), dev(case["vc"]), dev(case["bt"])
     tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
@@ -225,7 +249,7 @@ def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=No
         partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
         tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
         ops.attention_decode(out, qv, kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
-                             n_splits=splits, partials=partials, tok_list=tl,
+                             n_splits=splits, partials=partials, tok_list=tl, waves=waves,
                              n_tokens=len(tok_list) if tok_list is not None else None)
     return out
 
@@ -254,19 +278,19 @@ def test_attention_generic(ops, case_id, dtype, window):
 
 
 @pytest.mark.parametrize("window", [0, 37])
-@pytest.mark.parametrize("splits", [1, 2, 5, 32])
+@pytest.mark.parametrize("splits,waves", [(1, 4), (1, 16), (2, 4), (5, 16), (32, 4)])
 @pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
-def test_attention_decode(ops, case_id, splits, window):
+def test_attention_decode(ops, case_id, splits, waves, window):
     ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
     case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
     scale = 0.7 / math.sqrt(hd)
-    out = run_attention(ops, case, H, hd, scale, window, "decode", splits)
+    out = run_attention(ops, case, H, hd, scale, window, "decode", splits, waves=waves)
     assert torch.isfinite(out.float()).all()
     close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, f"decode splits={splits}")
     # a subset of the rows through tok_list: the others stay untouched
     if case["n"] > 2:
         rows = list(range(case["n"]))[::2]
-        part = run_attention(ops, case, H, hd, scale, window, "decode", splits, tok_list=rows)
+        part = run_attention(ops, case, H, hd, scale, window, "decode", splits, tok_list=rows, waves=waves)
         assert torch.equal(part[rows], out[rows]) and (part[1::2] == 0).all()
 
 
@@ -286,3 +310,50 @@ def test_attention_finds_one_far_key(ops, kernel):
         out = run_attention(ops, case, H, hd, 1.0, 0, kernel, splits=3 if kernel == "decode" else 1)
         want = case["vs"][0][target, 0].float()
         assert torch.allclose(out[0, :hd].float().cpu(), want, atol=2e-2), f"{kernel}: key {target} was not found"
+
+
+# ---------------------------------------------------------------------------
+# sampling
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,V", [(1, 50257), (9, 1000), (64, 777), (3, 5)])
+def test_argmax_ties_go_to_the_lowest_id(ops, rows, V):
+    logits = rnd(rows, V + 3)[:, :V]  # strided rows
+    logits[:, V // 2] = 50.0
+    logits[:, V - 1] = 50.0  # a tie: the lower id wins
+    if rows > 1:
+        logits[1, 0] = 50.0
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.argmax(out, logits)
+    want = [V // 2] * rows
+    if rows > 1:
+        want[1] = 0
+    assert out.tolist() == want
+    ops.argmax(out, rnd(rows, V, seed=4))
+    assert out.tolist() == rnd(rows, V, seed=4).argmax(dim=1).tolist()
+
+
+def test_sampler_against_the_plain_sampler(ops):
+    """Temperature, top-k and top-p per row against the plain implementation's rules."""
+    import plain_gpt2 as plain
+
+    V = 1000
+    logits = rnd(12, V, scale=2.0, seed=11)
+    logits[5, 100:140] = 3.0  # many ties at the top-k boundary
+    params = [(0.0, 0, 1.0), (1.0, 0, 1.0), (0.8, 0, 1.0), (0.8, 40, 0.95), (1.3, 5, 1.0), (0.7, 20, 1.0), (1.0, 0, 0.5),
+              (1.0, 0, 0.05), (0.5, 1, 1.0), (2.0, 999, 0.9), (1.0, 40, 0.0), (0.8, 0, 0.999)]
+    cpu = logits.cpu().numpy()
+    for trial in range(6):
+        u = [plain.uniform(7 + trial, r) for r in range(12)]
+        out = torch.empty(12, dtype=torch.int32, device=DEV)
+        ops.sample(out, logits,
+                   torch.tensor([p[0] for p in params], dtype=torch.float32, device=DEV),
+                   torch.tensor([p[1] for p in params], dtype=torch.int32, device=DEV),
+                   torch.tensor([p[2] for p in params], dtype=torch.float32, device=DEV),
+                   torch.tensor(u, dtype=torch.float64, device=DEV))
+        got = out.tolist()
+        for r, (T, k, p) in enumerate(params):
+            probs = plain.probabilities(cpu[r], T, k, p)
+            want = plain.sample(probs, u[r])
+            if got[r] != want:
+                cdf = np.cumsum(probs)
+                assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (r, params[r], got[r], want)
