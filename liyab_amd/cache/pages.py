@@ -28,6 +28,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from ..errors import Busy, ContextFull, InvalidArgument, OutOfPages
 
 UNMAPPED = -1
@@ -139,6 +141,8 @@ class CacheManager:
         self._requests: Dict[Hashable, _Request] = {}
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         self.max_blocks = max(1, -(-max_positions // page_size))
+        # the same tables as arrays, a row per state slot: the step function gathers a batch's rows at once
+        self._table_rows = [np.full((max_requests, self.max_blocks), UNMAPPED, dtype=np.int32) for _ in self.groups]
 
     # -- requests -----------------------------------------------------------
     def open(self, rid: Hashable) -> int:
@@ -158,8 +162,9 @@ class CacheManager:
     def close(self, rid: Hashable) -> None:
         """Gives back everything the request holds."""
         r = self._requests.pop(rid)
-        for g, table in zip(self.groups, r.tables):
+        for g, table, rows in zip(self.groups, r.tables, self._table_rows):
             g.pool.release([p for p in table if p != UNMAPPED])
+            rows[r.slot, :] = UNMAPPED
         self._free_slots.append(r.slot)
 
     def length(self, rid: Hashable) -> int:
@@ -213,8 +218,11 @@ class CacheManager:
                 raise OutOfPages(f"group {g.index}: {n} pages wanted, {g.pool.free_pages} free of {g.pool.num_pages}")
         for rid, new_length in wants:
             r = self._requests[rid]
-            for g, table in zip(self.groups, r.tables):
-                table.extend(g.pool.allocate(max(0, self._pages_for(new_length) - len(table))))
+            for g, table, rows in zip(self.groups, r.tables, self._table_rows):
+                new = g.pool.allocate(max(0, self._pages_for(new_length) - len(table)))
+                if new:
+                    rows[r.slot, len(table):len(table) + len(new)] = new
+                    table.extend(new)
             r.reserved = max(r.reserved, new_length)
 
     def commit(self, rid: Hashable, new_length: int) -> None:
@@ -236,6 +244,7 @@ class CacheManager:
                 if table[lp] != UNMAPPED:
                     gone.append(table[lp])
                     table[lp] = UNMAPPED
+                    self._table_rows[gi][r.slot, lp] = UNMAPPED
             r.first_kept[gi] = max(r.first_kept[gi], min(keep_from, len(table)))
             g.pool.release(gone)
 
@@ -253,11 +262,17 @@ class CacheManager:
             table = r.tables[gi]
             g.pool.release([p for p in table[keep:] if p != UNMAPPED])
             del table[keep:]
+            self._table_rows[gi][r.slot, keep:] = UNMAPPED
         r.length = length
         r.reserved = min(r.reserved, keep * self.page_size)
 
     def block_table(self, rid: Hashable, group: int = 0) -> List[int]:
         return self._requests[rid].tables[group]
+
+    def table_rows(self, group: int = 0) -> np.ndarray:
+        """int32 [max_requests, max_blocks]: the block table of the request in each state slot
+        (UNMAPPED where nothing is mapped). Read-only for callers."""
+        return self._table_rows[group]
 
     def slot_of_position(self, rid: Hashable, group: int, position: int) -> int:
         """page * page_size + offset for a mapped position."""

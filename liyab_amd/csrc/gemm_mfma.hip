@@ -160,7 +160,7 @@ extern "C" int liyab_gemm_mfma(const void* a, int64_t lda, const void* w, int M,
     if (M == 0) return 0;
     if (tile == 0) {
         const long big = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-        tile = big >= 200 ? 1 : 2;
+        tile = (big >= 200 && M > 64) ? 1 : 2;
     }
     switch (tile) {
         case 1: return launch_mfma<128, 128>(a, lda, w, M, N, K, epi, stream);

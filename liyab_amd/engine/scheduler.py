@@ -141,16 +141,28 @@ class Scheduler:
         Pages are only counted here; the step function maps them."""
         budget = self.max_batched_tokens
         batch: List[Scheduled] = []
-        wants: List = []
+        groups = self.manager.groups
+        need = [0] * len(groups)  # pages this step's batch takes so far, per group
+
+        def extra(r: Request, count: int) -> List[int]:
+            return self.manager.pages_needed(r.rid, r.computed + count)
 
         def fits(r: Request, count: int) -> bool:
-            return self.manager.can_reserve(wants + [(r.rid, r.computed + count)])
+            return all(n + e <= g.pool.free_pages for n, e, g in zip(need, extra(r, count), groups))
 
         def take(r: Request, count: int) -> None:
             nonlocal budget
+            for gi, e in enumerate(extra(r, count)):
+                need[gi] += e
             batch.append(Scheduled(r, r.computed, count, r.computed + count == r.n_tokens))
-            wants.append((r.rid, r.computed + count))
             budget -= count
+
+        def untake(s: Scheduled) -> None:
+            nonlocal budget
+            for gi, e in enumerate(extra(s.request, s.count)):
+                need[gi] -= e
+            batch.remove(s)
+            budget += s.count
 
         # running requests: decoding ones first, then prompt portions, each in order of admission
         order = [r for r in self.running if r.remaining == 1] + [r for r in self.running if r.remaining > 1]
@@ -168,9 +180,7 @@ class Scheduler:
                         count = 0
                     break
                 for s in [s for s in batch if s.request is victim]:
-                    batch.remove(s)
-                    wants.remove((victim.rid, victim.computed + s.count))
-                    budget += s.count
+                    untake(s)
                 self._preempt(victim)
             if count > 0 and r.state == RUNNING:
                 take(r, count)
@@ -178,7 +188,8 @@ class Scheduler:
         while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
             r = self.waiting[0]
             count = min(r.remaining, self.prefill_chunk, budget)
-            if self.manager.free_slots() == 0 or not self.manager.can_reserve(wants, new_lengths=[count]):
+            pages = -(-count // self.manager.page_size)
+            if self.manager.free_slots() == 0 or any(n + pages > g.pool.free_pages for n, g in zip(need, groups)):
                 break
             self._open(r)
             self.waiting.popleft()

@@ -19,6 +19,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import itertools
+
 import numpy as np
 import torch
 
@@ -115,9 +117,6 @@ class StepFunction:
             n = len(it.tokens)
             if n == 0:
                 raise InvalidArgument(f"request {it.rid!r} brings no tokens")
-            for t in it.tokens:
-                if not (0 <= int(t) < V):
-                    raise InvalidArgument(f"token id {t} of request {it.rid!r} is outside [0, {V})")
             for w in it.want:
                 if not (0 <= int(w) < n):
                     raise InvalidArgument(f"request {it.rid!r} wants logits at place {w} of {n} tokens")
@@ -169,6 +168,11 @@ class StepFunction:
         mgr = self.manager
         first = [mgr.length(it.rid) for it in items]
         q_lens = [len(it.tokens) for it in items]
+        all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64,
+                                 count=sum(q_lens))
+        if all_tokens.min() < 0 or all_tokens.max() >= self.model.vocab_size:
+            bad = int(all_tokens[(all_tokens < 0) | (all_tokens >= self.model.vocab_size)][0])
+            raise InvalidArgument(f"token id {bad} is outside [0, {self.model.vocab_size})")  # src/core/transformer.cpp:6195-6197
         mgr.reserve([(it.rid, f + n) for it, f, n in zip(items, first, q_lens)])
 
         S, N = len(items), sum(q_lens)
@@ -201,32 +205,25 @@ class StepFunction:
 
         tok, pos, seq = view("token_ids"), view("positions"), view("tok_seq")
         rows = view("logit_rows")
+        q_arr = np.asarray(q_lens, dtype=np.int64)
+        first_arr = np.asarray(first, dtype=np.int64)
+        tok[:] = all_tokens
+        seq[:] = np.repeat(np.arange(S, dtype=np.int32), q_arr)
+        pos[:] = np.repeat(first_arr - starts[:-1], q_arr) + np.arange(N, dtype=np.int64)
         rows[:] = 0
-        r = 0
-        for i, it in enumerate(items):
-            a, b = int(starts[i]), int(starts[i + 1])
-            tok[a:b] = np.asarray(it.tokens, dtype=np.int32)
-            pos[a:b] = np.arange(first[i], first[i] + q_lens[i], dtype=np.int32)
-            seq[a:b] = i
-            for w in it.want:
-                rows[r] = a + int(w)
-                r += 1
+        if R:
+            rows[:R] = [int(starts[i]) + int(w) for i, it in enumerate(items) for w in it.want]
         view("seq_starts")[:] = starts
-        view("context_lens")[:] = [f + n for f, n in zip(first, q_lens)]
-        view("state_slots")[:] = [mgr.slot(it.rid) for it in items]
+        view("context_lens")[:] = first_arr + q_arr
+        slot_ids = np.asarray([mgr.slot(it.rid) for it in items], dtype=np.int64)
+        view("state_slots")[:] = slot_ids
         for g in range(G):
-            bt = view(f"bt{g}").reshape(S, W)
-            bt[:] = UNMAPPED
-            sl = view(f"slots{g}")
-            for i, it in enumerate(items):
-                table = np.asarray(mgr.block_table(it.rid, g), dtype=np.int32)
-                bt[i, :len(table)] = table
-                a, b = int(starts[i]), int(starts[i + 1])
-                p = pos[a:b]
-                pages = table[p // page]
-                if (pages < 0).any():
-                    raise AssertionError("a token of this step maps to a released page")
-                sl[a:b] = pages * page + p % page
+            tables = mgr.table_rows(g)[slot_ids]  # [S, W]
+            view(f"bt{g}").reshape(S, W)[:] = tables
+            pages = tables[seq, pos // page]
+            if (pages < 0).any():
+                raise AssertionError("a token of this step maps to a released page")
+            view(f"slots{g}")[:] = pages * page + pos % page
 
         if self._meta_dev is None or self._meta_dev.numel() < total:
             # sized for the largest step of this engine's lifetime where possible: a new block
