@@ -1,0 +1,219 @@
+// Causal attention of prompt portions over paged bfloat16 keys and values, on
+// the matrix cores (the formulas of the reference's attention,
+// src/core/transformer.cpp:2303-2358, blocked as in flash attention: the
+// reference's own remark on flash decoding is at :2146-2153).
+//
+// A work item is (tile of up to 128 consecutive queries of one request, head);
+// each of 4 waves owns 32 queries. Keys are visited in blocks of 32, staged in
+// LDS with their values. Scores are computed transposed, S^T = K Q^T with
+// v_mfma_f32_32x32x16_bf16 (contraction over the head dimension, both operands
+// contiguous along it), so that a lane holds 16 scores of ONE query: the
+// running maximum and sum of a query need one exchange with the lane 32 apart
+// instead of a reduction over 32 lanes. The accumulators then serve, rounded to
+// bfloat16, directly as the second operand of O^T = V^T P^T (contraction over
+// the keys); only V has to be read across its rows, as 2-byte reads of LDS.
+// Maximum, exponentials, sums and outputs are 32-bit. A query's result depends
+// on its position and the block grid (multiples of 32 from the window's start),
+// not on the batch or the pages. Head sizes: multiples of 16 up to 128.
+#include "common.h"
+
+namespace liyab {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+union QFrag {
+    u32x4 u;
+    bf16x8 v;
+    bf16_t h[8];
+};
+
+constexpr int AP_KEYS = 32;     // keys per block
+constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
+
+template <int DB>  // head dimension padded to 32 * DB
+__global__ void __launch_bounds__(256)
+attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+                         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
+                         int window, int n_head, int n_kv_head, int hd, int page_size) {
+    constexpr int HDP = 32 * DB;
+    constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[AP_KEYS * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[AP_KEYS * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t Os[4][32 * LDK];
+
+    const int* wk = work + 4 * blockIdx.x;
+    const int seq = wk[0], row0 = wk[1], pos0 = wk[2], nq = wk[3];
+    const int h = blockIdx.y;
+    const int hkv = h / (n_head / n_kv_head);
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int ql = lane % 32, g2 = lane / 32;
+    const int* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
+
+    const int my_q = 32 * wave + ql;
+    const int qpos = pos0 + min(my_q, nq - 1);  // lanes past the tile's end repeat its last query; never stored
+    const int wave_last = pos0 + min(32 * wave + 31, nq - 1);  // the wave's latest query position
+    const bool wave_has = 32 * wave < nq;
+    const int n_slabs = hd / 16;
+
+    QFrag qf[2 * DB];
+    {
+        const bf16_t* qrow = q + static_cast<int64_t>(row0 + min(my_q, nq - 1)) * q_stride + static_cast<int64_t>(h) * hd;
+#pragma unroll
+        for (int s = 0; s < 2 * DB; ++s) {
+            qf[s].u = u32x4{0, 0, 0, 0};
+            if (s < n_slabs) qf[s].u = *reinterpret_cast<const u32x4*>(qrow + 16 * s + 8 * g2);
+        }
+    }
+    floatx16 o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const int k_hi = pos0 + nq - 1;  // last key any query of the tile sees
+    const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int64_t page_stride = static_cast<int64_t>(n_kv_head) * page_size * hd;
+    const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd;
+    constexpr int CHUNKS = 4 * DB;  // 16-byte pieces per padded row
+
+    for (int kb = (k_lo / AP_KEYS) * AP_KEYS; kb <= k_hi; kb += AP_KEYS) {
+        // stage the block's keys and values (zeros past the head dimension and past the last key)
+        for (int c = tid; c < AP_KEYS * CHUNKS; c += 256) {
+            const int key = c / CHUNKS, col = (c % CHUNKS) * 8;
+            const int kp = kb + key;
+            u32x4 kvv = {0, 0, 0, 0}, vvv = {0, 0, 0, 0};
+            if (kp >= k_lo && kp <= k_hi && col < hd) {
+                const int64_t at = static_cast<int64_t>(bt[kp / page_size]) * page_stride + head_off +
+                                   static_cast<int64_t>(kp % page_size) * hd + col;
+                kvv = *reinterpret_cast<const u32x4*>(kc + at);
+                vvv = *reinterpret_cast<const u32x4*>(vc + at);
+            }
+            *reinterpret_cast<u32x4*>(Ks + key * LDK + col) = kvv;
+            *reinterpret_cast<u32x4*>(Vs + key * LDK + col) = vvv;
+        }
+        __syncthreads();
+        if (wave_has && kb <= wave_last) {
+            // S^T[key][query] = sum_d K[key][d] Q[query][d]
+            floatx16 st;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < 2 * DB; ++s) {
+                if (s < n_slabs) {
+                    QFrag kf;
+                    kf.u = *reinterpret_cast<const u32x4*>(Ks + ql * LDK + 16 * s + 8 * g2);
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[s].v, st, 0, 0, 0);
+                }
+            }
+            // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4
+            float bm = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
+                const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
+                st[r] = ok ? st[r] * scale : -INFINITY;
+                bm = fmaxf(bm, st[r]);
+            }
+            bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+            const float m_new = fmaxf(m_run, bm);
+            float corr = 1.0f, bs = 0.0f;
+            QFrag pf[2];
+            if (m_new == -INFINITY) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[0].h[e] = pf[1].h[e] = 0;
+            } else {
+                corr = m_run == -INFINITY ? 0.0f : __expf(m_run - m_new);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = __expf(st[r] - m_new);  // exp(-inf) = 0 for masked keys
+                    bs += p;
+                    pf[r / 8].h[r % 8] = float_to_bf16(p);
+                }
+            }
+            bs += __shfl_xor(bs, 32, 64);
+            l_run = l_run * corr + bs;
+            m_run = m_new;
+            // O^T[d][query] += sum_key V[key][d] P[key][query]; instruction s2 contracts the keys
+            // of accumulator registers 8 s2 .. 8 s2 + 7: rows 16 s2 + 4 g2 + {0..3} and + 8
+#pragma unroll
+            for (int d = 0; d < DB; ++d) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[d][r] *= corr;
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    QFrag vf;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int key = 16 * s2 + 8 * (e / 4) + 4 * g2 + e % 4;
+                        vf.h[e] = Vs[key * LDK + 32 * d + ql];
+                    }
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[s2].v, o[d], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // o[d][r] = O^T[dim = 32 d + 8 (r / 4) + 4 g2 + r % 4][query ql]: through LDS to rows of 16-byte pieces
+    if (wave_has) {
+        const float inv = 1.0f / l_run;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                Os[wave][ql * LDK + 32 * d + 8 * (r / 4) + 4 * g2 + r % 4] = float_to_bf16(o[d][r] * inv);
+    }
+    __syncthreads();
+    if (wave_has) {
+        const int chunks_row = hd / 8;
+        for (int c = lane; c < 32 * chunks_row; c += 64) {
+            const int qq = c / chunks_row, col = (c % chunks_row) * 8;
+            if (32 * wave + qq < nq) {
+                *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row0 + 32 * wave + qq) * out_stride +
+                                          static_cast<int64_t>(h) * hd + col) =
+                    *reinterpret_cast<const u32x4*>(&Os[wave][qq * LDK + col]);
+            }
+        }
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+// work: n_tiles x (request index, first row, first position, queries <= 128), int32.
+extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                       const void* vc, const int* block_tables, int max_blocks, const int* work,
+                                       int n_tiles, float scale, int window, int n_head, int n_kv_head, int hd,
+                                       int page_size, hipStream_t stream) {
+    LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
+    LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
+    LIYAB_REQUIRE(n_head % n_kv_head == 0 && n_head <= 65535, "attention_prefill: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
+    LIYAB_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0, "attention_prefill: head size %d is not a multiple of 16 in 16..128", hd);
+    LIYAB_REQUIRE(q_stride % 8 == 0 && out_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(q) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(kc) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(vc) & 15) == 0,
+                  "attention_prefill: operands must be 16-byte aligned with strides that are multiples of 8");
+    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
+                  "attention_prefill: row strides are shorter than heads x head size");
+    LIYAB_REQUIRE(window >= 0, "attention_prefill: negative window");
+    if (n_tiles == 0) return 0;
+    dim3 grid(n_tiles, n_head);
+    auto* o = static_cast<bf16_t*>(out);
+    auto* pq = static_cast<const bf16_t*>(q);
+    auto* pk = static_cast<const bf16_t*>(kc);
+    auto* pv = static_cast<const bf16_t*>(vc);
+#define LIYAB_GO(D)                                                                                                \
+    attention_prefill_kernel<D><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables,      \
+                                                          max_blocks, work, scale, window, n_head, n_kv_head, hd, \
+                                                          page_size)
+    if (hd <= 32) LIYAB_GO(1);
+    else if (hd <= 64) LIYAB_GO(2);
+    else if (hd <= 96) LIYAB_GO(3);
+    else LIYAB_GO(4);
+#undef LIYAB_GO
+    return check_launch("attention_prefill");
+}

@@ -68,6 +68,7 @@ class _Staging:
         ev.record()
 
 
+ATTN_TILE = 128  # queries of one request that the prefill attention kernel takes together
 DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
 
 
@@ -133,7 +134,8 @@ class StepFunction:
             # a workspace buffer moved since the graphs were captured: they hold its old address
             self._graphs.clear()
             self._graph_generation = self.workspace.generation
-        key = (ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows, ctx.host.attention_mode, ctx.host.context_bucket)
+        key = (ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows, ctx.host.attention_mode, ctx.host.context_bucket,
+               ctx.host.n_attn_tiles, ctx.host.n_attn_single)
         entry = self._graphs.get(key)
         if isinstance(entry, tuple):
             entry[0].replay()
@@ -183,11 +185,26 @@ class StepFunction:
         starts = np.zeros(S + 1, dtype=np.int64)
         np.cumsum(q_lens, out=starts[1:])
 
+        # attention's work in a step with long portions: tiles of up to 128 queries for them,
+        # single rows for requests that bring few tokens
+        mode = "decode" if max(q_lens) <= DECODE_Q_LEN else "prefill"
+        tiles, singles = [], []
+        if mode == "prefill":
+            for i, (f, n) in enumerate(zip(first, q_lens)):
+                a = int(starts[i])
+                if n <= DECODE_Q_LEN:
+                    singles.extend(range(a, a + n))
+                else:
+                    for t0 in range(0, n, ATTN_TILE):
+                        tiles.extend((i, a + t0, f + t0, min(ATTN_TILE, n - t0)))
+        n_tiles = len(tiles) // 4
+
         # layout of the metadata block (int32 words)
         off = {}
         cur = 0
         for name, size in (("token_ids", N), ("positions", N), ("tok_seq", N), ("seq_starts", S + 1),
-                           ("context_lens", S), ("state_slots", S), ("logit_rows", max(R, 1))):
+                           ("context_lens", S), ("state_slots", S), ("logit_rows", max(R, 1)),
+                           ("attn_work", max(len(tiles), 1)), ("attn_single", max(len(singles), 1))):
             off[name] = (cur, size)
             cur += size
         for g in range(G):
@@ -214,6 +231,10 @@ class StepFunction:
         if R:
             rows[:R] = [int(starts[i]) + int(w) for i, it in enumerate(items) for w in it.want]
         view("seq_starts")[:] = starts
+        if tiles:
+            view("attn_work")[:] = tiles
+        if singles:
+            view("attn_single")[:] = singles
         view("context_lens")[:] = first_arr + q_arr
         slot_ids = np.asarray([mgr.slot(it.rid) for it in items], dtype=np.int64)
         view("state_slots")[:] = slot_ids
@@ -247,9 +268,11 @@ class StepFunction:
             groups=[GroupStep(block_tables=dview(f"bt{g}").view(S, W), slots=dview(f"slots{g}")) for g in range(G)],
             host=StepHost(q_lens=q_lens, starts=[int(s) for s in starts[:-1]], first_pos=first,
                           max_q_len=max(q_lens), max_context=max_context,
-                          attention_mode="decode" if max(q_lens) <= DECODE_Q_LEN else "prefill",
-                          context_bucket=_bucket(max_context)),
+                          attention_mode=mode, context_bucket=_bucket(max_context), n_attn_tiles=n_tiles,
+                          n_attn_single=len(singles)),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
+            attn_work=dview("attn_work") if mode == "prefill" else None,
+            attn_single_rows=dview("attn_single") if mode == "prefill" else None,
         )
         logits = self._forward(ctx)
         for it, f, n in zip(items, first, q_lens):

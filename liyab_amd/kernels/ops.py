@@ -416,6 +416,35 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
               n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, _ptr(partials), _stream())
 
 
+def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_tables: torch.Tensor, work: torch.Tensor, n_tiles: int, *, n_head: int, scale: float,
+                      window: int = 0) -> None:
+    """Tiles of up to 128 consecutive queries of one request over its bfloat16 cache, on the
+    matrix cores. work: int32 [n_tiles, 4] = (request index, first row, first position, queries);
+    the caller has checked rows and positions against out and the block tables."""
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
+    _, hkv, page, hd = k_cache.shape
+    os_, qs = _rows(out, "out"), _rows(q, "q")
+    if q.shape[0] != out.shape[0] or q.shape[1] < n_head * hd or out.shape[1] != n_head * hd:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {n_head} heads of {hd}")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        raise KernelError("attention_prefill: q, out and the caches must be bfloat16")
+    if not prefill_takes(hd):
+        raise KernelError(f"attention_prefill: head size {hd} is not a multiple of 16 in 16..128")
+    _dev(block_tables, "block_tables")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
+    _i32(work, "work", 4 * n_tiles)
+    _lib.call("liyab_attention_prefill", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
+              block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, float(scale), int(window),
+              n_head, hkv, hd, page, _stream())
+
+
+def prefill_takes(hd: int) -> bool:
+    return hd % 16 == 0 and 16 <= hd <= 128
+
+
 def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
     """(splits of the keys, waves per workgroup), from measurements at 12 heads of 64: with many
     (token, head) pairs a workgroup of 4 waves per pair is fastest; with few, 16 waves per pair,
@@ -432,14 +461,28 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
     is chosen from the step's shape (`ctx` is the step's StepContext)."""
     hd = k_cache.shape[3]
-    if q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and ctx.host.attention_mode == "decode":
-        n = out.shape[0]
-        splits, waves = decode_plan(n, n_head, ctx.host.context_bucket)
+    host = ctx.host
+    fast = q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and out.stride(0) % 8 == 0
+
+    def decode(tok_list, n):
+        splits, waves = decode_plan(n, n_head, host.context_bucket)
         partials = None
         if splits > 1:
             partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 2),), torch.float32)
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
-                         scale=scale, window=window, n_splits=splits, partials=partials, waves=waves)
+                         scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
+                         tok_list=tok_list, n_tokens=n if tok_list is not None else None)
+
+    if fast and host.attention_mode == "decode":
+        decode(None, out.shape[0])
+        return
+    if fast and prefill_takes(hd) and ctx.attn_work is not None:
+        # long portions in tiles on the matrix cores, the short ones token by token
+        if host.n_attn_tiles:
+            attention_prefill(out, q, k_cache, v_cache, block_tables, ctx.attn_work, host.n_attn_tiles, n_head=n_head,
+                              scale=scale, window=window)
+        if host.n_attn_single:
+            decode(ctx.attn_single_rows, host.n_attn_single)
         return
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)

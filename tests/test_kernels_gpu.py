@@ -245,6 +245,18 @@ def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=No
     qv = q[:, :H * hd]
     if kernel == "generic":
         ops.attention_generic(out, qv, kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window)
+    elif kernel == "prefill":
+        work, row = [], 0
+        lens = {}
+        for sidx in case["tok_seq"]:
+            lens[sidx] = lens.get(sidx, 0) + 1
+        for sidx, nq in sorted(lens.items()):
+            p0 = case["tok_pos"][row]
+            for t0 in range(0, nq, 128):
+                work.extend((sidx, row + t0, p0 + t0, min(128, nq - t0)))
+            row += nq
+        wk = torch.tensor(work, dtype=torch.int32, device=DEV)
+        ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window)
     elif kernel == "decode":
         partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
         tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
@@ -292,6 +304,51 @@ def test_attention_decode(ops, case_id, splits, waves, window):
         rows = list(range(case["n"]))[::2]
         part = run_attention(ops, case, H, hd, scale, window, "decode", splits, tok_list=rows, waves=waves)
         assert torch.equal(part[rows], out[rows]) and (part[1::2] == 0).all()
+
+
+PREFILL_CASES = [
+    # ctx_lens, q_lens, H, Hkv, hd, page
+    ([1, 17, 300], [1, 17, 300], 4, 4, 16, 16),
+    ([40, 129, 5], [7, 100, 5], 3, 3, 32, 16),
+    ([700, 64], [130, 64], 5, 5, 64, 64),
+    ([33, 257], [20, 129], 6, 2, 48, 8),
+    ([300], [300], 2, 1, 128, 16),
+    ([90, 31], [31, 9], 2, 2, 80, 16),
+    ([1024], [1024], 1, 1, 64, 16),
+]
+
+
+@pytest.mark.parametrize("window", [0, 37, 200])
+@pytest.mark.parametrize("case_id", range(len(PREFILL_CASES)))
+def test_attention_prefill(ops, case_id, window):
+    ctx_lens, q_lens, H, Hkv, hd, page = PREFILL_CASES[case_id]
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
+    scale = 0.7 / math.sqrt(hd)
+    out = run_attention(ops, case, H, hd, scale, window, "prefill")
+    assert torch.isfinite(out.float()).all()
+    close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, "prefill")
+
+
+def test_attention_prefill_finds_one_far_key(ops):
+    """A portion's queries each with one outstanding key, at page and block edges."""
+    H = Hkv = 2
+    hd, page, T, nq = 64, 16, 700, 140
+    targets = [0, 15, 16, 31, 32, 255, 256, 511, 559, 560, 561, 600, 640, 687, 698, 699]
+    case = paged_case(1, [T], [nq], H, Hkv, hd, page, torch.bfloat16, seed=3)
+    k = case["ks"][0]
+    for n, target in enumerate(targets):
+        row = nq - 1 - n * 3  # the query at position T - 1 - 3 n looks for `target` if it may see it
+        qpos = T - nq + row
+        if target > qpos:
+            continue
+        qv = case["q"][row, :hd].float()
+        # orthogonalise against earlier planted keys is not needed: random 64-vectors are nearly orthogonal
+        k[target, 0] = (qv * 4).to(torch.bfloat16)
+        lp, off = divmod(target, page)
+        case["kc"][case["bt"][0, lp], 0, off] = k[target, 0]
+    out = run_attention(ops, case, H, hd, 1.0, 0, "prefill")
+    ref = attention_reference(case, H, Hkv, hd, 1.0, 0)
+    close(out, ref, 8e-3, "prefill far keys")
 
 
 @pytest.mark.parametrize("kernel", ["generic", "decode"])
