@@ -159,8 +159,10 @@ extern "C" int liyab_gemm_mfma(const void* a, int64_t lda, const void* w, int M,
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
     if (tile == 0) {
+        // measured at 2048 x {768, 2304, 3072} x {768, 3072}: 64 x 64 tiles (4 workgroups a CU,
+        // many tiles) beat 128 x 128 (2 a CU, a ragged second round) until there are thousands of tiles
         const long big = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-        tile = (big >= 200 && M > 64) ? 1 : 2;
+        tile = big >= 2048 ? 1 : 2;
     }
     switch (tile) {
         case 1: return launch_mfma<128, 128>(a, lda, w, M, N, K, epi, stream);

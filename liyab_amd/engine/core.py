@@ -21,13 +21,13 @@ from .step import StepFunction, StepItem
 
 
 class EngineCore:
-    def __init__(self, model_dir: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
+    def __init__(self, model_dir: Optional[str] = None, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_requests: int = 64,
-                 context_length: Optional[int] = None):
-        """`num_pages`: pages per cache group; or `max_tokens`: the most tokens
-        live requests hold together (rounded up to whole pages per request by
-        the caller's accounting). With neither, every request slot can reach
-        the full context."""
+                 context_length: Optional[int] = None, use_graphs: bool = True, model=None, config=None):
+        """`model_dir`: a folder with config.json and model.safetensors (or pass a built
+        `model`, see `from_plan`). `num_pages`: pages per cache group; or `max_tokens`: the
+        most tokens live requests hold together (rounded up to whole pages per request by the
+        caller's accounting). With neither, every request slot can reach the full context."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: this engine runs on gfx950 only and has no CPU path")
         from ..kernels import ops
@@ -35,7 +35,12 @@ class EngineCore:
         ops.check_device()
         self.device = torch.device(device)
         self.dtype = resolve_dtype(dtype)
-        self.config, self.model = load_model(model_dir, self.dtype, self.device)
+        if model is None:
+            if model_dir is None:
+                raise InvalidArgument("a model folder or a built model is needed")
+            self.config, self.model = load_model(model_dir, self.dtype, self.device)
+        else:
+            self.config, self.model = config, model
         max_positions = self.model.max_positions
         if context_length is not None:
             if context_length <= 0:
@@ -51,7 +56,21 @@ class EngineCore:
         self.manager = CacheManager(self.model.cache_groups(), page_size=page_size, num_pages=max(1, num_pages),
                                     max_requests=max_requests, max_positions=max_positions)
         self.storage = CacheStorage(self.manager, self.dtype, self.device, self.model.state_specs())
-        self.step_fn = StepFunction(self.model, self.manager, self.storage, self.device)
+        self.step_fn = StepFunction(self.model, self.manager, self.storage, self.device, use_graphs=use_graphs)
+
+    @classmethod
+    def from_plan(cls, plan, tensors, *, dtype="float32", device="cuda:0", **kw) -> "EngineCore":
+        """An engine for a plan and a dict of CPU tensors by name: how a model is built
+        without a folder (tests build toy architectures so)."""
+        from ..models.decoder import DecoderModel
+        from ..weights.loader import WeightStore
+
+        dt = resolve_dtype(dtype)
+        store = WeightStore(dict(tensors), device=device, compute_dtype=dt, name_prefixes=plan.name_prefixes,
+                            ignorable=plan.ignorable)
+        model = DecoderModel(plan, store, dt)
+        store.finish()
+        return cls(None, dtype=dt, device=device, model=model, config=None, **kw)
 
     # -- requests -----------------------------------------------------------
     def open(self, rid: Hashable) -> None:

@@ -166,6 +166,21 @@ class StepFunction:
         Returns float32 logits [wanted, vocab] on the device, rows in the order
         of the items and of each item's `want`, or None when nothing is wanted.
         The tensor is workspace memory: valid until the next step."""
+        ctx, lengths = self.prepare(items)
+        logits = self._forward(ctx)
+        self.commit(items, lengths)
+        return logits
+
+    def commit(self, items: Sequence[StepItem], lengths: Sequence[int]) -> None:
+        """The requests now hold `lengths` positions (after a step's kernels are enqueued)."""
+        for it, n in zip(items, lengths):
+            self.manager.commit(it.rid, n)
+        self.steps += 1
+        self.tokens += sum(len(it.tokens) for it in items)
+
+    def prepare(self, items: Sequence[StepItem]):
+        """Checks the items, maps their pages (all or nothing) and puts the step's metadata on
+        the device. Returns (StepContext, the lengths to commit once the step has run)."""
         self._validate(items)
         mgr = self.manager
         first = [mgr.length(it.rid) for it in items]
@@ -274,9 +289,4 @@ class StepFunction:
             attn_work=dview("attn_work") if mode == "prefill" else None,
             attn_single_rows=dview("attn_single") if mode == "prefill" else None,
         )
-        logits = self._forward(ctx)
-        for it, f, n in zip(items, first, q_lens):
-            mgr.commit(it.rid, f + n)
-        self.steps += 1
-        self.tokens += N
-        return logits
+        return ctx, [f + n for f, n in zip(first, q_lens)]

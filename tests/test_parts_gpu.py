@@ -1,0 +1,395 @@
+"""Each part alone against its plain formula, and the generality of the layer plan: a toy
+mixer with state of its own, defined here, is registered, built and stepped without touching
+the framework's files; a layer reads another layer's cache; the run order names a layer twice
+(needs the GPU)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2 as plain
+import trace_tools as tt
+from conftest import TOL
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def T(name, layout="out_in", required=True):
+    from liyab_amd.config import TensorSource
+
+    return TensorSource(name, layout, required)
+
+
+def norm_spec(prefix, d, eps):
+    from liyab_amd.config import NormSpec
+
+    return NormSpec("layernorm", d, eps, {"weight": T(prefix + ".w"), "bias": T(prefix + ".b")})
+
+
+def attention_spec(prefix, d, H, Hkv, hd, scale, window=0):
+    from liyab_amd.config import AttentionSpec
+
+    return AttentionSpec("attention", d, H, Hkv, hd, scale, window,
+                         {"qkv_weight": T(prefix + ".qkv.w"), "qkv_bias": T(prefix + ".qkv.b"),
+                          "out_weight": T(prefix + ".out.w"), "out_bias": T(prefix + ".out.b")})
+
+
+def ffn_spec(prefix, d, F, act):
+    from liyab_amd.config import DenseFFNSpec
+
+    return DenseFFNSpec("dense_ffn", d, F, act, {"up_weight": T(prefix + ".up.w"), "up_bias": T(prefix + ".up.b"),
+                                                 "down_weight": T(prefix + ".down.w"), "down_bias": T(prefix + ".down.b")})
+
+
+def make_plan(d, V, P, layers, order, eps=1e-5):
+    from liyab_amd.config import HeadSpec, ModelPlan, PositionSpec, TokenEmbeddingSpec
+
+    return ModelPlan(architecture="toy", width=d, vocab_size=V, max_positions=P,
+                     embedding=TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": T("emb")}),
+                     residual_position=PositionSpec("learned_positions", "residual", P, d, {"table": T("pos")}),
+                     layers=layers, order=order, final_norm=norm_spec("nf", d, eps),
+                     head=HeadSpec("lm_head", d, V, 1.0, {"weight": T("emb")}))
+
+
+def rand(rng, *shape, scale=1.0, mean=0.0):
+    return torch.from_numpy((rng.standard_normal(shape) * scale + mean).astype(np.float32))
+
+
+def norm_tensors(rng, prefix, d):
+    return {prefix + ".w": rand(rng, d, scale=0.1, mean=1.0), prefix + ".b": rand(rng, d, scale=0.1)}
+
+
+def attention_tensors(rng, prefix, d, H, Hkv, hd):
+    n = (H + 2 * Hkv) * hd
+    return {prefix + ".qkv.w": rand(rng, n, d, scale=0.15), prefix + ".qkv.b": rand(rng, n, scale=0.1),
+            prefix + ".out.w": rand(rng, d, H * hd, scale=0.1), prefix + ".out.b": rand(rng, d, scale=0.1)}
+
+
+def ffn_tensors(rng, prefix, d, F):
+    return {prefix + ".up.w": rand(rng, F, d, scale=0.15), prefix + ".up.b": rand(rng, F, scale=0.1),
+            prefix + ".down.w": rand(rng, d, F, scale=0.1), prefix + ".down.b": rand(rng, d, scale=0.1)}
+
+
+def f64(t):
+    return t.double().numpy()
+
+
+# ---------------------------------------------------------------------------
+# plain formulas for the toy models (whole sequences, float64)
+# ---------------------------------------------------------------------------
+def plain_attention(h, tw, prefix, H, Hkv, hd, scale, window=0, kv_from=None):
+    """QKV with [out, in] weights, grouped heads, optional window; `kv_from` = (k, v) of another layer."""
+    qkv = h @ f64(tw[prefix + ".qkv.w"]).T + f64(tw[prefix + ".qkv.b"])
+    q, k, v = qkv[:, :H * hd], qkv[:, H * hd:(H + Hkv) * hd], qkv[:, (H + Hkv) * hd:]
+    if kv_from is not None:
+        k, v = kv_from
+    rep = H // Hkv
+    # query head hh reads key/value head hh // rep
+    kk = np.concatenate([k[:, (hh // rep) * hd:(hh // rep + 1) * hd] for hh in range(H)], axis=1)
+    vv = np.concatenate([v[:, (hh // rep) * hd:(hh // rep + 1) * hd] for hh in range(H)], axis=1)
+    att = plain.causal_attention(q, kk, vv, H, scale, window)
+    return att @ f64(tw[prefix + ".out.w"]).T + f64(tw[prefix + ".out.b"]), (k, v)
+
+
+def plain_ffn(h, tw, prefix, act):
+    fn = plain.gelu_tanh if act == "gelu_tanh" else plain.gelu_erf
+    return fn(h @ f64(tw[prefix + ".up.w"]).T + f64(tw[prefix + ".up.b"])) @ f64(tw[prefix + ".down.w"]).T + f64(tw[prefix + ".down.b"])
+
+
+def plain_norm(x, tw, prefix, eps):
+    return plain.layer_norm(x, f64(tw[prefix + ".w"]), f64(tw[prefix + ".b"]), eps)
+
+
+# ---------------------------------------------------------------------------
+# each part alone
+# ---------------------------------------------------------------------------
+class _Parts:
+    """A one-layer engine whose step context and cache the part tests borrow."""
+
+    def __init__(self, dtype, d=80, H=5, Hkv=5, hd=16, F=136, V=300, P=200, window=0, eps=1e-4, act="gelu_erf"):
+        from liyab_amd.config import LayerSpec, OrderEntry
+        from liyab_amd.engine import EngineCore
+
+        rng = np.random.default_rng(7)
+        self.d, self.H, self.Hkv, self.hd, self.F, self.V, self.eps, self.act = d, H, Hkv, hd, F, V, eps, act
+        self.scale = 0.9 / math.sqrt(hd)
+        layer = LayerSpec(attention_spec("a", d, H, Hkv, hd, self.scale, window), ffn_spec("f", d, F, act),
+                          norm_spec("n1", d, eps), norm_spec("n2", d, eps))
+        self.tw = {"emb": rand(rng, V, d, scale=0.5), "pos": rand(rng, P, d, scale=0.3), **norm_tensors(rng, "nf", d),
+                   **norm_tensors(rng, "n1", d), **norm_tensors(rng, "n2", d), **attention_tensors(rng, "a", d, H, Hkv, hd),
+                   **ffn_tensors(rng, "f", d, F)}
+        if dtype == "bfloat16":  # the bfloat16 path holds matrices in bfloat16: compare against those values
+            self.tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in self.tw.items()}
+        self.core = EngineCore.from_plan(make_plan(d, V, P, [layer], [OrderEntry(0)], eps), self.tw, dtype=dtype,
+                                         page_size=8, num_pages=64, max_requests=4, use_graphs=False)
+        self.block = self.core.model.blocks[0]
+
+
+@pytest.fixture(scope="module", params=["float32", "bfloat16"])
+def parts(request):
+    return _Parts(request.param), request.param
+
+
+def test_embedding_and_positions_alone(parts):
+    from liyab_amd.engine import StepItem
+
+    p, dtype = parts
+    core = p.core
+    core.open("e")
+    ids = [5, 299, 0, 17, 5]
+    core.step([StepItem("e", [1, 2, 3], [])])  # so that the next tokens sit at positions 3..7
+    ctx, lengths = core.step_fn.prepare([StepItem("e", ids, [])])
+    x = torch.zeros(5, p.d, device=DEV)
+    core.model.embedding.forward(ctx, x)
+    assert torch.equal(x.cpu(), core.model.embedding.table.float().cpu()[ids])
+    core.model.residual_position.add(ctx, x)
+    want = f64(p.tw["emb"])[ids] + f64(p.tw["pos"])[3:8]
+    assert tt.rel_err(x.cpu().numpy(), want) < 1e-6
+    x2 = torch.zeros(5, p.d, device=DEV)
+    core.model.embedding.forward(ctx, x2, position_table=core.model.residual_position.fused_table())
+    assert torch.equal(x2, x)
+    core.step_fn.commit([StepItem("e", ids, [])], lengths)
+    core.close("e")
+
+
+def test_norm_alone(parts):
+    from liyab_amd.engine import StepItem
+
+    p, dtype = parts
+    core = p.core
+    core.open("n")
+    ctx, _ = core.step_fn.prepare([StepItem("n", [1] * 9, [2, 7])])
+    x = rand(np.random.default_rng(1), 9, p.d, scale=2.0, mean=0.7).to(DEV)
+    tol = 1e-5 if dtype == "float32" else 6e-3
+    got = p.block.norm_mixer.forward(x, ctx)
+    assert tt.rel_err(got.float().cpu().numpy(), plain_norm(f64(x.cpu()), p.tw, "n1", p.eps)) < tol
+    got = core.model.final_norm.forward(x, ctx, rows=ctx.logit_rows, n_rows=2, name="t")
+    assert tt.rel_err(got.float().cpu().numpy(), plain_norm(f64(x.cpu())[[2, 7]], p.tw, "nf", p.eps)) < tol
+    pending = p.block.norm_ffn.lazy(x, ctx)
+    assert pending.shape == (9, p.d)
+    assert tt.rel_err(pending.tensor().float().cpu().numpy(), plain_norm(f64(x.cpu()), p.tw, "n2", p.eps)) < tol
+    core.close("n")
+
+
+@pytest.mark.parametrize("lazy", [False, True])
+def test_feed_forward_alone(parts, lazy):
+    from liyab_amd.engine import StepItem
+
+    p, dtype = parts
+    core = p.core
+    core.open("f")
+    ctx, _ = core.step_fn.prepare([StepItem("f", [1] * 11, [])])
+    rng = np.random.default_rng(2)
+    x = rand(rng, 11, p.d, scale=1.5).to(DEV)
+    residual = rand(rng, 11, p.d).to(DEV)
+    want = f64(residual.cpu()) + plain_ffn(plain_norm(f64(x.cpu()), p.tw, "n2", p.eps), p.tw, "f", p.act)
+    h = p.block.norm_ffn.lazy(x, ctx) if lazy else p.block.norm_ffn.forward(x, ctx)
+    p.block.ffn.forward(h, ctx, residual)
+    assert tt.rel_err(residual.cpu().numpy(), want) < (1e-5 if dtype == "float32" else 1e-2)
+    core.close("f")
+
+
+@pytest.mark.parametrize("geometry", [dict(H=5, Hkv=5, hd=16), dict(H=6, Hkv=2, hd=32, d=96), dict(H=3, Hkv=1, hd=48, d=64, window=13)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_mixer_alone(dtype, geometry):
+    """The mixer over its own cache: a whole portion, then more portions and single tokens,
+    against plain attention over the whole sequence; grouped heads and a window too."""
+    from liyab_amd.engine import StepItem
+
+    p = _Parts(dtype, **geometry)
+    core, att = p.core, p.block.mixer
+    rng = np.random.default_rng(3)
+    n = 60
+    x = rand(rng, n, p.d, scale=1.2)
+    want, _ = plain_attention(plain_norm(f64(x), p.tw, "n1", p.eps), p.tw, "a", p.H, p.Hkv, p.hd, p.scale,
+                              window=geometry.get("window", 0))
+    core.open("m")
+    done = 0
+    for take in (25, 1, 9, 1, 1, 23):
+        item = StepItem("m", [1] * take, [])
+        ctx, lengths = core.step_fn.prepare([item])
+        xs = x[done:done + take].to(DEV)
+        residual = torch.zeros(take, p.d, device=DEV)
+        att.forward(p.block.norm_mixer.forward(xs, ctx), ctx, core.storage.layer(0), None, residual)
+        core.step_fn.commit([item], lengths)
+        err = tt.rel_err(residual.cpu().numpy(), want[done:done + take])
+        assert err < (1e-5 if dtype == "float32" else 1e-2), (take, done, err)
+        done += take
+    core.close("m")
+    core.manager.check()
+
+
+def test_block_and_head_alone(parts):
+    from liyab_amd.engine import StepItem
+
+    p, dtype = parts
+    core = p.core
+    core.open("b")
+    rng = np.random.default_rng(4)
+    n = 21
+    x0 = rand(rng, n, p.d, scale=1.1)
+    item = StepItem("b", [1] * n, [0, n - 1])
+    ctx, lengths = core.step_fn.prepare([item])
+    x = x0.clone().to(DEV)
+    p.block.forward(x, ctx, core.storage.layer(0), None)
+    core.step_fn.commit([item], lengths)
+    a, _ = plain_attention(plain_norm(f64(x0), p.tw, "n1", p.eps), p.tw, "a", p.H, p.Hkv, p.hd, p.scale)
+    want = f64(x0) + a
+    want = want + plain_ffn(plain_norm(want, p.tw, "n2", p.eps), p.tw, "f", p.act)
+    assert tt.rel_err(x.cpu().numpy(), want) < (1e-5 if dtype == "float32" else 1e-2)
+    h = core.model.final_norm.lazy(x, ctx, rows=ctx.logit_rows, n_rows=2, name="head_in")
+    logits = core.model.head.forward(h, ctx)
+    want_logits = plain_norm(want[[0, n - 1]], p.tw, "nf", p.eps) @ f64(p.tw["emb"]).T
+    assert logits.dtype == torch.float32 and logits.shape == (2, p.V)
+    assert tt.rel_err(logits.cpu().numpy(), want_logits) < (1e-5 if dtype == "float32" else 1.5e-2)
+    core.close("b")
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture: a mixer with state of its own, shared caches, a layer named twice
+# ---------------------------------------------------------------------------
+class DecaySpec:
+    """Spec of the toy mixer: any object with a `kind` can stand in a LayerSpec."""
+
+    kind = "toy_decay"
+
+    def __init__(self, width, decay, prefix):
+        self.width, self.decay, self.prefix = width, decay, prefix
+
+
+class DecayMixer:
+    """s_t = decay * s_{t-1} + h_t per request (state of fixed size, no keys), out = s_t . W^T.
+    It keeps its state in the slot the cache manager gives its request, carries it across
+    portions and steps, and uses torch for its arithmetic: it is a test's toy, not a kernel."""
+
+    def __init__(self, spec, store, dtype):
+        from liyab_amd.config import TensorSource
+
+        self.width, self.decay, self.dtype = spec.width, spec.decay, dtype
+        self.weight = store.fetch(TensorSource(spec.prefix + ".w"), (spec.width, spec.width), "matrix")
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        from liyab_amd.cache import StateSpec
+
+        return StateSpec((self.width,), "float32")
+
+    def forward(self, h, ctx, cache, state, residual, writes_cache=True):
+        from liyab_amd.parts import as_tensor
+
+        h = as_tensor(h).float()
+        slots = ctx.state_slots.tolist()
+        out = torch.empty_like(h)
+        for i, (a, n) in enumerate(zip(ctx.host.starts, ctx.host.q_lens)):
+            s = state[slots[i]]
+            for t in range(a, a + n):  # in token order within the request's portion
+                s = self.decay * s + h[t]
+                out[t] = s
+            state[slots[i]] = s
+        residual += out @ self.weight.float().t()
+
+
+def toy_model(dtype="float32"):
+    """Layers: 0 = decay mixer + erf FFN, 1 = attention (5 heads of 16) + tanh FFN, 2 = windowed
+    grouped attention (4 query heads on 2 key/value heads of 32, window 24) + tanh FFN, 3 =
+    attention without a feed-forward that reads layer 1's cache. Run order 0, 1, 2, 3, 1
+    (layer 1 a second time, reading its cache without writing)."""
+    from liyab_amd.config import LayerSpec, OrderEntry
+    from liyab_amd.parts import register_mixer
+
+    register_mixer("toy_decay", DecayMixer)
+    d, V, P, eps = 80, 211, 160, 1e-5
+    rng = np.random.default_rng(11)
+    s1 = 1 / math.sqrt(16)
+    layers = [
+        LayerSpec(DecaySpec(d, 0.8, "m0"), ffn_spec("f0", d, 100, "gelu_erf"), norm_spec("n0a", d, eps), norm_spec("n0b", d, eps)),
+        LayerSpec(attention_spec("a1", d, 5, 5, 16, s1), ffn_spec("f1", d, 160, "gelu_tanh"), norm_spec("n1a", d, eps), norm_spec("n1b", d, eps)),
+        LayerSpec(attention_spec("a2", d, 4, 2, 32, 0.2, window=24), ffn_spec("f2", d, 64, "gelu_tanh"), norm_spec("n2a", d, eps), norm_spec("n2b", d, eps)),
+        LayerSpec(attention_spec("a3", d, 5, 5, 16, s1 / 2), None, norm_spec("n3a", d, eps), None),
+    ]
+    order = [OrderEntry(0), OrderEntry(1), OrderEntry(2), OrderEntry(3, cache_of=1, writes_cache=False),
+             OrderEntry(1, writes_cache=False)]
+    tw = {"emb": rand(rng, V, d, scale=0.5), "pos": rand(rng, P, d, scale=0.3), **norm_tensors(rng, "nf", d),
+          "m0.w": rand(rng, d, d, scale=0.05)}
+    for i, (H, Hkv, hd, F) in enumerate([(0, 0, 0, 100), (5, 5, 16, 160), (4, 2, 32, 64), (5, 5, 16, 0)]):
+        tw.update(norm_tensors(rng, f"n{i}a", d))
+        if F:
+            tw.update(norm_tensors(rng, f"n{i}b", d))
+            tw.update(ffn_tensors(rng, f"f{i}", d, F))
+        if H:
+            tw.update(attention_tensors(rng, f"a{i}", d, H, Hkv, hd))
+    if dtype == "bfloat16":
+        tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tw.items()}
+    return make_plan(d, V, P, layers, order, eps), tw, dict(d=d, V=V, P=P, eps=eps, s1=s1)
+
+
+def toy_plain(tw, info, ids):
+    """The toy model over a whole sequence, float64."""
+    eps, s1 = info["eps"], info["s1"]
+    x = f64(tw["emb"])[ids] + f64(tw["pos"])[:len(ids)]
+    # layer 0: the decay mixer
+    h = plain_norm(x, tw, "n0a", eps)
+    s = np.zeros(info["d"])
+    out = np.zeros_like(h)
+    for t in range(len(ids)):
+        s = 0.8 * s + h[t]
+        out[t] = s
+    x = x + out @ f64(tw["m0.w"]).T
+    x = x + plain_ffn(plain_norm(x, tw, "n0b", eps), tw, "f0", "gelu_erf")
+    # layer 1
+    a, kv1 = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 5, 5, 16, s1)
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_tanh")
+    # layer 2: windowed, grouped
+    a, _ = plain_attention(plain_norm(x, tw, "n2a", eps), tw, "a2", 4, 2, 32, 0.2, window=24)
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n2b", eps), tw, "f2", "gelu_tanh")
+    # layer 3 reads layer 1's keys and values; no feed-forward
+    a, _ = plain_attention(plain_norm(x, tw, "n3a", eps), tw, "a3", 5, 5, 16, s1 / 2, kv_from=kv1)
+    x = x + a
+    # layer 1 again, on its cache as its first run left it
+    a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 5, 5, 16, s1, kv_from=kv1)
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_tanh")
+    return plain_norm(x, tw, "nf", eps) @ f64(tw["emb"]).T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_a_stateful_mixer(dtype):
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = toy_model(dtype)
+    reqs = {f"t{i}": tt.random_tokens(90 + i, n, info["V"]) for i, n in enumerate([37, 90, 5, 128, 61])}
+    ref = {rid: toy_plain(tw, info, toks) for rid, toks in reqs.items()}
+    tol = TOL[dtype]
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=3))):
+        core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4,
+                                    use_graphs=False)  # the toy mixer reads its slots on the host: no capture
+        groups = core.manager.groups
+        assert len(groups) == 2 and sorted(g.spec.window for g in groups) == [0, 24]
+        assert [g.layers for g in groups if g.spec.window == 0] == [[1]]  # layer 3 owns no cache: it reads layer 1's
+        assert set(core.storage.states) == {0}  # only the decay mixer keeps state
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, tol, f"toy {name} {dtype}")
+        core.manager.check()
+        assert all(core.manager.pages_in_use(g.index) == 0 for g in groups)
+
+
+def test_unknown_kinds_are_refused_by_name():
+    from liyab_amd import Unsupported
+    from liyab_amd.config import LayerSpec, OrderEntry
+    from liyab_amd.engine import EngineCore
+
+    class Nameless:
+        kind = "no_such_mixer"
+
+    plan, tw, info = toy_model()
+    bad = LayerSpec(Nameless(), None, norm_spec("n0a", info["d"], 1e-5), None)
+    with pytest.raises(Unsupported, match="mixer kind 'no_such_mixer' is not registered"):
+        EngineCore.from_plan(make_plan(info["d"], info["V"], info["P"], [bad], [OrderEntry(0)]), tw)
