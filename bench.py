@@ -133,6 +133,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="run only the prefill of 2,048 tokens (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -148,6 +149,10 @@ def main():
     with tempfile.TemporaryDirectory() as d:
         write_random_model(d, cfg, 10, dtype="bfloat16" if short == "bf16" else "float32")
         engine = make_engine(d, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), ctx)
+        if args.prefill_only:
+            ptps, pms = prefill_run(engine, cfg, [1024, 1024], repeat=20)
+            print(json.dumps({"prefill": {"value": round(ptps, 1), "tokens": 2048, "ms": round(pms, 4)}}))
+            return 0
         tps, ms, bytes_per_step = decode_run(engine, cfg, args.batch, args.prompt, steps, args.warmup)
         achieved = bytes_per_step / (ms * 1e-3) / 1e9
         out = {
