@@ -283,3 +283,58 @@ def test_command_line_json(model_dirs, plain_models):
     eos = config.get("eos_token_id")
     assert turn["tokens"] == expect[:len(turn["tokens"])] and (len(turn["tokens"]) == 12 or turn["tokens"][-1] == eos)
     assert "decode:" in p.stderr and "prompt: 9 tokens" in p.stderr
+
+
+# ---------------------------------------------------------------------------
+# real widths
+# ---------------------------------------------------------------------------
+SIZES = {
+    # GPT-2 small's sizes, all 12 layers
+    "small": dict(n_layer=12, n_embd=768, n_head=12, n_inner=3072, vocab_size=50257, n_positions=1024, seed=10,
+                  lens=[300, 77, 130]),
+    # GPT-2 XL's layer sizes (width 1600, 25 heads, feed-forward 6400), two layers, a small vocabulary
+    "xl_layers": dict(n_layer=2, n_embd=1600, n_head=25, n_inner=6400, vocab_size=3001, n_positions=512, seed=30,
+                      lens=[200, 33, 90]),
+    # three heads of 48 in a width of 144, a vocabulary that is no multiple of anything
+    "odd": dict(n_layer=2, n_embd=144, n_head=3, n_inner=200, vocab_size=777, n_positions=640, seed=5,
+                lens=[600, 45, 170]),
+}
+
+
+@pytest.fixture(scope="module")
+def sized_models(tmp_path_factory):
+    """{name: (folder, requests, {dtype: plain logits})}, each made on first use."""
+    made = {}
+
+    def get(name):
+        if name not in made:
+            from liyab_amd.weights import write_random_model
+
+            s = SIZES[name]
+            cfg = {"architectures": ["GPT2LMHeadModel"], "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new",
+                   **{k: s[k] for k in ("n_layer", "n_embd", "n_head", "n_inner", "vocab_size", "n_positions")}}
+            d = str(tmp_path_factory.mktemp(f"sized_{name}"))
+            write_random_model(d, cfg, s["seed"])
+            config, tensors = plain.read_model(d)
+            reqs = {f"{name}{i}": tt.random_tokens(s["seed"] + 1 + i, n, s["vocab_size"]) for i, n in enumerate(s["lens"])}
+            refs = {"float32": {rid: plain.forward(config, tensors, t) for rid, t in reqs.items()}}
+            rounded = plain.round_weights_to_bf16(tensors)
+            refs["bfloat16"] = {rid: plain.forward(config, rounded, t) for rid, t in reqs.items()}
+            made[name] = (d, reqs, refs)
+        return made[name]
+
+    return get
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(SIZES))
+def test_real_widths_whole_and_mixed(name, dtype, sized_models):
+    """GPT-2 small's full sizes, XL's layer sizes and an odd geometry: whole prompts and a
+    mixed schedule with pages used again, against the plain implementation."""
+    d, reqs, refs = sized_models(name)
+    for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=1, decode_tail=6))):
+        core = make_core(d, dtype, tt.max_live_tokens(steps))
+        got = tt.run_schedule(core, steps)
+        worst = tt.check_against_plain(got, reqs, refs[dtype], TOL[dtype], f"{name} {label} {dtype}")
+        core.manager.check()
+        del core
