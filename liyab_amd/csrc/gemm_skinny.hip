@@ -41,7 +41,7 @@ struct LnParams {
     float eps;
 };
 
-template <typename OutT, bool LN, int MT, int NT, int MAXW>
+template <typename OutT, bool LN, int MT, int NT, int MAXW, int MAXV = 32>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
                    EpiParams epi, LnParams ln) {
@@ -76,10 +76,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     };
     Frag wc[UPT][NT][2];
     load_w(wave, wc);  // issued before the norm's prologue, so the two overlap
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
 
     const bf16_t* arow[MT];
     if constexpr (LN) {
-        constexpr int MAXV = 32;  // K <= 64 * MAXV
+        // a row's values stay in registers: MAXV per lane, K <= 64 * MAXV
         for (int m = wave; m < M; m += ksplit) {
             const float* xr = ln.x + static_cast<int64_t>(ln.rows != nullptr ? ln.rows[m] : m) * K;
             float v[MAXV], gw[MAXV], gb[MAXV];
@@ -169,7 +170,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     }
 }
 
-template <bool LN, int MT, int NT, int MAXW>
+template <bool LN, int MT, int NT, int MAXW, int MAXV = 32>
 int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, const EpiParams& epi,
                   const LnParams& ln, hipStream_t stream) {
     const int grid = (N + 16 * NT - 1) / (16 * NT);
@@ -180,7 +181,7 @@ int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K
     if (LN) smem += ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16;
     const bool f32 = epi.mode == kEpiResidual || epi.out_dtype == kF32;
     if (f32) {
-        auto kern = gemm_skinny_kernel<float, LN, MT, NT, MAXW>;
+        auto kern = gemm_skinny_kernel<float, LN, MT, NT, MAXW, MAXV>;
         static bool ready = false;
         if (!ready) {
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -188,7 +189,7 @@ int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K
         }
         kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln);
     } else {
-        auto kern = gemm_skinny_kernel<bf16_t, LN, MT, NT, MAXW>;
+        auto kern = gemm_skinny_kernel<bf16_t, LN, MT, NT, MAXW, MAXV>;
         static bool ready = false;
         if (!ready) {
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -216,7 +217,10 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
     }
     LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || ksplit == 4 || ksplit == 8 || ksplit == 16,
                   "gemm_skinny: ksplit %d is not 1, 2, 4, 8 or 16", ksplit);
-    if (ln.x != nullptr) return launch_skinny<true, 1, 1, 8>(a, lda, w, M, N, K, ksplit, epi, ln, stream);  // 8 waves: registers for a row's values
+    if (ln.x != nullptr) {  // 8 waves: registers for a row's values
+        if (K <= 1024) return launch_skinny<true, 1, 1, 8, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+        return launch_skinny<true, 1, 1, 8, 32>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+    }
     if (nt == 1) {
         if (mt == 1) return launch_skinny<false, 1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
         if (mt == 2) return launch_skinny<false, 2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
