@@ -9,11 +9,15 @@
 
 namespace liyab {
 
+// An id below zero is a reference: -1 - id indexes `last_tokens`, where the sampler left the
+// token a request drew in the step before (the host may not have seen it yet).
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ tok, const T* __restrict__ pos,
-                             const int* __restrict__ ids, const int* __restrict__ positions, int d, float scale) {
+                             const int* __restrict__ ids, const int* __restrict__ positions, int d, float scale,
+                             const int* __restrict__ last_tokens) {
     const int t = blockIdx.x;
-    const int64_t id = ids[t];
+    int64_t id = ids[t];
+    if (id < 0) id = last_tokens[-1 - id];
     const T* trow = tok + id * d;
     const T* prow = pos != nullptr ? pos + static_cast<int64_t>(positions[t]) * d : nullptr;
     float* out = x + static_cast<int64_t>(t) * d;
@@ -61,7 +65,7 @@ __global__ void kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc, const T*
 using namespace liyab;
 
 extern "C" int liyab_embed(float* x, const void* tok, const void* pos, int dtype, const int* ids, const int* positions,
-                           int n, int d, float scale, hipStream_t stream) {
+                           int n, int d, float scale, const int* last_tokens, hipStream_t stream) {
     LIYAB_REQUIRE(x && tok && ids, "embed: null pointer");
     LIYAB_REQUIRE(pos == nullptr || positions != nullptr, "embed: a position table needs positions");
     LIYAB_REQUIRE(d > 0 && n >= 0, "embed: bad sizes n=%d d=%d", n, d);
@@ -69,10 +73,10 @@ extern "C" int liyab_embed(float* x, const void* tok, const void* pos, int dtype
     const int threads = d >= 256 ? 256 : 64;
     if (dtype == kF32) {
         embed_kernel<float><<<n, threads, 0, stream>>>(x, static_cast<const float*>(tok), static_cast<const float*>(pos),
-                                                       ids, positions, d, scale);
+                                                       ids, positions, d, scale, last_tokens);
     } else if (dtype == kBF16) {
         embed_kernel<bf16_t><<<n, threads, 0, stream>>>(x, static_cast<const bf16_t*>(tok),
-                                                        static_cast<const bf16_t*>(pos), ids, positions, d, scale);
+                                                        static_cast<const bf16_t*>(pos), ids, positions, d, scale, last_tokens);
     } else {
         return fail(1, "embed: unknown dtype %d", dtype);
     }

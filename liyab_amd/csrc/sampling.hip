@@ -92,7 +92,7 @@ __device__ __forceinline__ void block_argmax(const float* row, int V, float& bes
 __global__ void __launch_bounds__(S_THREADS)
 sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t ld, int V,
               const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
-              const double* __restrict__ uniform) {
+              const double* __restrict__ uniform, const int* __restrict__ scatter_index, int* __restrict__ scatter_out) {
     __shared__ double redd[S_WAVES];
     __shared__ int redi[S_WAVES];
     __shared__ float redf[S_WAVES];
@@ -107,7 +107,10 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
     block_argmax(row, V, lmax, imax, redf, redi);
     const float T = temperature != nullptr ? temperature[r] : 0.0f;
     if (!(T > 0.0f)) {
-        if (tid == 0) out[r] = imax;
+        if (tid == 0) {
+            out[r] = imax;
+            if (scatter_index != nullptr) scatter_out[scatter_index[r]] = imax;
+        }
         return;
     }
     const float inv_t = 1.0f / T;
@@ -230,7 +233,11 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
         if (last >= 0) atomicMax(&result, last);
         __syncthreads();
     }
-    if (tid == 0) out[r] = result < 0 ? imax : result;
+    if (tid == 0) {
+        const int token = result < 0 ? imax : result;
+        out[r] = token;
+        if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
+    }
 }
 
 // Argmax in two stages so that a few rows still use many CUs: chunks of a row give partial
@@ -268,7 +275,8 @@ argmax_partial_kernel(float* __restrict__ pv, int* __restrict__ pi, const float*
 }
 
 __global__ void __launch_bounds__(64)
-argmax_final_kernel(int* __restrict__ out, const float* __restrict__ pv, const int* __restrict__ pi) {
+argmax_final_kernel(int* __restrict__ out, const float* __restrict__ pv, const int* __restrict__ pi,
+                    const int* __restrict__ scatter_index, int* __restrict__ scatter_out) {
     const int r = blockIdx.x;
     float bv = pv[r * AM_CHUNKS + threadIdx.x];
     int bi = pi[r * AM_CHUNKS + threadIdx.x];
@@ -278,16 +286,21 @@ argmax_final_kernel(int* __restrict__ out, const float* __restrict__ pv, const i
         const int oi = __shfl_xor(bi, off, kWave);
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
-    if (threadIdx.x == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+    if (threadIdx.x == 0) {
+        const int token = bi == 0x7fffffff ? 0 : bi;
+        out[r] = token;
+        if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
+    }
 }
 
 }  // namespace liyab
 
 using namespace liyab;
 
-// scratch_v / scratch_i: rows * 64 floats / ints of workspace.
+// scratch_v / scratch_i: rows * 64 floats / ints of workspace. With scatter_index, row r's token
+// also goes to scatter_out[scatter_index[r]] (the requests' last-token table).
 extern "C" int liyab_argmax(int* out, const float* logits, int64_t ld, int rows, int V, float* scratch_v,
-                            int* scratch_i, hipStream_t stream) {
+                            int* scratch_i, const int* scatter_index, int* scatter_out, hipStream_t stream) {
     LIYAB_REQUIRE(out && logits && scratch_v && scratch_i, "argmax: null pointer");
     LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d", rows, V);
     LIYAB_REQUIRE(rows <= 65535 * 16, "argmax: too many rows");
@@ -295,17 +308,19 @@ extern "C" int liyab_argmax(int* out, const float* logits, int64_t ld, int rows,
     static_assert(AM_CHUNKS == kWave, "the final stage is one wave over the chunks");
     argmax_partial_kernel<<<dim3(rows, AM_CHUNKS), 256, 0, stream>>>(scratch_v, scratch_i, logits, ld, V);
     if (int rc = check_launch("argmax_partial")) return rc;
-    argmax_final_kernel<<<rows, 64, 0, stream>>>(out, scratch_v, scratch_i);
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(out, scratch_v, scratch_i, scatter_index, scatter_out);
     return check_launch("argmax_final");
 }
 
 // Per-row parameters; a row with temperature <= 0 is greedy. top_k <= 0 and
 // top_p >= 1 switch those filters off. uniform[r] is in [0, 1).
 extern "C" int liyab_sample(int* out, const float* logits, int64_t ld, int rows, int V, const float* temperature,
-                            const int* top_k, const float* top_p, const double* uniform, hipStream_t stream) {
+                            const int* top_k, const float* top_p, const double* uniform, const int* scatter_index,
+                            int* scatter_out, hipStream_t stream) {
     LIYAB_REQUIRE(out && logits && temperature && uniform, "sample: null pointer");
     LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d", rows, V);
     if (rows == 0) return 0;
-    sample_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform);
+    LIYAB_REQUIRE(scatter_index == nullptr || scatter_out != nullptr, "sample: a scatter index needs a target");
+    sample_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out);
     return check_launch("sample");
 }

@@ -48,12 +48,16 @@ class GenerationResult:
 class Engine:
     def __init__(self, model: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_num_seqs: int = 64,
-                 max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None):
+                 max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None,
+                 overlap: bool = True):
         """`model`: a folder with config.json and model.safetensors. `ctx`: the
         context length (default: the model's). `prefill_chunk`: the longest
         portion of a prompt in one step (the reference's 256,
         src/core/engine.cpp:2863-2864). `num_pages` / `max_tokens` size the
-        page pool."""
+        page pool. `overlap`: schedule and launch the next step before the host has read
+        this step's tokens (decoding requests take their last token from a table on the
+        device); finishing by an end token is then seen one step late and that step's work
+        for the request is dropped. Tokens are the same either way."""
         self.core = EngineCore(model, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
                                max_tokens=max_tokens, max_requests=max_num_seqs, context_length=ctx)
         self.scheduler = Scheduler(self.core.manager, max_num_seqs=max_num_seqs,
@@ -66,6 +70,10 @@ class Engine:
         self._t_end: Dict[Hashable, float] = {}
         self._next_id = 0
         self.stop_at_eos = True
+        self.overlap = overlap
+        self._inflight = None  # (batch, wanting requests, pinned host tokens, event) of the step not yet read
+        self._host_tokens = [None, None]
+        self._turn = 0
 
     # -- plumbing ---------------------------------------------------------------
     def _reset_slot(self, rid: Hashable) -> None:
@@ -97,24 +105,15 @@ class Engine:
         return rid
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.has_unfinished() or self._inflight is not None
 
-    def step(self, on_token: Optional[Callable[[Hashable, int], Optional[bool]]] = None) -> List[Request]:
-        """One scheduler iteration: a batch, a model step, sampling. Returns the
-        requests that finished in it."""
-        batch = self.scheduler.schedule()
-        if not batch:
-            return []
-        items = []
-        for s in batch:
-            toks = s.request.tokens[s.first:s.first + s.count]
-            items.append(StepItem(s.request.rid, toks, [s.count - 1] if s.wants_logits else []))
-        logits = self.core.step(items)
+    def _resolve(self, inflight, on_token) -> List[Request]:
+        """Reads a launched step's tokens and lets the scheduler account for them."""
+        batch, wanting, host, event = inflight
         sampled: Dict[Hashable, int] = {}
-        wanting = [s.request for s in batch if s.wants_logits]
         if wanting:
-            tokens = self.sampler.sample(logits, [r.params for r in wanting], [r.seed for r in wanting],
-                                         [len(r.generated) for r in wanting])
+            event.synchronize()
+            tokens = host[:len(wanting)].tolist()
             now = time.perf_counter()
             for r, t in zip(wanting, tokens):
                 sampled[r.rid] = int(t)
@@ -123,21 +122,71 @@ class Engine:
         cb = None
         if on_token is not None:
             cb = lambda r, t: on_token(r.rid, t)  # noqa: E731
+        saved = self.scheduler.eos_token_id
         if not self.stop_at_eos:
-            saved, self.scheduler.eos_token_id = self.scheduler.eos_token_id, None
-            done = self.scheduler.update(batch, sampled, cb)
+            self.scheduler.eos_token_id = None
+        try:
+            done = self.scheduler.resolve(batch, sampled, cb)
+        finally:
             self.scheduler.eos_token_id = saved
-        else:
-            done = self.scheduler.update(batch, sampled, cb)
         now = time.perf_counter()
         for r in done:
             self._t_end[r.rid] = now
         return done
 
+    def flush(self, on_token=None) -> List[Request]:
+        """Reads the tokens of a step still in flight, if there is one."""
+        if self._inflight is None:
+            return []
+        inflight, self._inflight = self._inflight, None
+        return self._resolve(inflight, on_token)
+
+    def step(self, on_token: Optional[Callable[[Hashable, int], Optional[bool]]] = None) -> List[Request]:
+        """One scheduler iteration: a batch, a model step, sampling. Returns the requests
+        found finished in it (with `overlap`, those of the step before)."""
+        import torch
+
+        done: List[Request] = []
+        if self._inflight is not None and (not self.overlap or self.scheduler.pressure()):
+            done += self.flush(on_token)  # pages are short: no request may carry a pending token into a preemption
+        batch = self.scheduler.schedule()
+        if not batch:
+            return done + self.flush(on_token)
+        items = []
+        for s in batch:
+            r = s.request
+            toks = r.tokens[s.first:s.first + s.count]
+            items.append(StepItem(r.rid, toks, [s.count - 1] if s.wants_logits else [],
+                                  pending_last=r.pending > 0 and s.first + s.count == r.n_tokens))
+        logits = self.core.step(items)
+        wanting = [s.request for s in batch if s.wants_logits]
+        host = event = None
+        if wanting:
+            ctx = self.core.step_fn.last_context
+            out = self.sampler.sample_on_device(
+                logits, [r.params for r in wanting], [r.seed for r in wanting],
+                [len(r.generated) + r.pending for r in wanting],
+                scatter=(ctx.logit_slots, ctx.last_tokens))
+            host = self._host_tokens[self._turn]
+            if host is None or host.numel() < len(wanting):
+                host = self._host_tokens[self._turn] = torch.empty(max(64, 2 * len(wanting)), dtype=torch.int32,
+                                                                   pin_memory=True)
+            self._turn ^= 1
+            host[:len(wanting)].copy_(out, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        self.scheduler.advance(batch)
+        previous, self._inflight = self._inflight, (batch, wanting, host, event)
+        if previous is not None:
+            done += self._resolve(previous, on_token)
+        if not self.overlap:
+            done += self.flush(on_token)
+        return done
+
     def abort(self, rid: Hashable) -> None:
         r = self._requests.get(rid)
         if r is not None and r.state != "finished":
-            self.scheduler.finish(r, "cancelled")
+            self.scheduler.finish(r, "cancelled")  # a step in flight may still hold it: its result is dropped
 
     def result(self, rid: Hashable) -> GenerationResult:
         r = self._requests[rid]
@@ -176,5 +225,6 @@ class Engine:
         rids = [self.add_request(p, sp) for p, sp in zip(plist, params_list)]
         while any(self._requests[r].state != "finished" for r in rids):
             self.step(on_token)
+        self.flush(on_token)
         results = [self.result(r) for r in rids]
         return results[0] if single else results

@@ -49,14 +49,17 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     arrival: int = 0
+    pending: int = 0  # tokens sampled in steps whose result the host has not read yet (at most 1 when scheduling)
 
     @property
     def tokens(self) -> List[int]:
-        return self.prompt + self.generated
+        """Prompt and generated tokens; a pending token stands as 0 at the end (the device
+        knows its value, see StepItem.pending_last)."""
+        return self.prompt + self.generated + [0] * self.pending
 
     @property
     def n_tokens(self) -> int:
-        return len(self.prompt) + len(self.generated)
+        return len(self.prompt) + len(self.generated) + self.pending
 
     @property
     def remaining(self) -> int:
@@ -121,6 +124,24 @@ class Scheduler:
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def draining(self, r: Request) -> bool:
+        """Whether r's pending token is its last whatever it turns out to be: max_tokens
+        reached, or no position left to run it at."""
+        return r.pending > 0 and (len(r.generated) + r.pending >= r.params.max_tokens or
+                                  r.n_tokens > self.manager.max_positions)
+
+    def pressure(self) -> bool:
+        """Whether the running requests' next portions may not all fit the free pages, so that
+        schedule() may have to preempt; the engine then reads pending tokens first."""
+        need = [0] * len(self.manager.groups)
+        for r in self.running:
+            count = min(r.remaining, self.prefill_chunk)
+            if count <= 0:
+                continue
+            for gi, n in enumerate(self.manager.pages_needed(r.rid, r.computed + count)):
+                need[gi] += n
+        return any(n > g.pool.free_pages for n, g in zip(need, self.manager.groups))
+
     # -- one step's decisions ---------------------------------------------------
     def _open(self, r: Request) -> None:
         self.manager.open(r.rid)
@@ -128,6 +149,8 @@ class Scheduler:
             self.on_open(r.rid)
 
     def _preempt(self, r: Request) -> None:
+        if r.pending > 0:
+            raise AssertionError("a request with a pending token cannot be preempted: read the tokens first")
         self.manager.close(r.rid)
         self.running.remove(r)
         r.computed = 0
@@ -165,7 +188,8 @@ class Scheduler:
             budget += s.count
 
         # running requests: decoding ones first, then prompt portions, each in order of admission
-        order = [r for r in self.running if r.remaining == 1] + [r for r in self.running if r.remaining > 1]
+        active = [r for r in self.running if not self.draining(r)]
+        order = [r for r in active if r.remaining == 1] + [r for r in active if r.remaining > 1]
         for r in order:
             if r.state != RUNNING or budget <= 0:
                 continue
@@ -196,7 +220,7 @@ class Scheduler:
             r.state = RUNNING
             self.running.append(r)
             take(r, count)
-        if not batch and self.has_unfinished():
+        if not batch and self.has_unfinished() and not any(r.pending > 0 for r in self.running):
             raise OutOfPages("no request can make progress: the page pool is too small for any of them")
         self.stats.steps += 1
         n = sum(s.count for s in batch)
@@ -206,23 +230,33 @@ class Scheduler:
         return batch
 
     # -- after the step -----------------------------------------------------------
-    def update(self, batch: Sequence[Scheduled], sampled: Dict[Hashable, int],
-               on_token: Optional[Callable[[Request, int], bool]] = None) -> List[Request]:
-        """Records what the step computed and sampled; returns requests that finished."""
+    def advance(self, batch: Sequence[Scheduled]) -> None:
+        """The step has been launched: its tokens are in the cache; requests whose portion
+        reached their last token have a token pending."""
+        for s in batch:
+            s.request.computed += s.count
+            if s.wants_logits:
+                s.request.pending += 1
+
+    def resolve(self, batch: Sequence[Scheduled], sampled: Dict[Hashable, int],
+                on_token: Optional[Callable[[Request, int], bool]] = None) -> List[Request]:
+        """The step's sampled tokens have reached the host; returns requests that finished.
+        A request that finished meanwhile (its earlier token ended it while this step was in
+        flight) is skipped: what this step computed for it is dropped."""
         done = []
         for s in batch:
             r = s.request
-            r.computed += s.count
-            if not s.wants_logits:
+            if not s.wants_logits or r.state == FINISHED:
                 continue
             token = sampled[r.rid]
+            r.pending -= 1
             r.generated.append(token)
             reason = None
             if self.eos_token_id is not None and token == self.eos_token_id:
                 reason = "stop"
             elif len(r.generated) >= r.params.max_tokens:
                 reason = "length"
-            elif r.n_tokens > self.manager.max_positions:
+            elif len(r.prompt) + len(r.generated) > self.manager.max_positions:
                 reason = "context"  # the next token would pass the last position
             if on_token is not None and on_token(r, token) is False and reason is None:
                 reason = "callback"
@@ -233,6 +267,12 @@ class Scheduler:
                                            max((g.pool.peak_in_use for g in self.manager.groups), default=0))
         return done
 
+    def update(self, batch: Sequence[Scheduled], sampled: Dict[Hashable, int],
+               on_token: Optional[Callable[[Request, int], bool]] = None) -> List[Request]:
+        """advance + resolve, for a caller that reads the tokens before the next step."""
+        self.advance(batch)
+        return self.resolve(batch, sampled, on_token)
+
     def finish(self, r: Request, reason: str) -> None:
         if r.state == RUNNING:
             self.manager.close(r.rid)
@@ -240,4 +280,5 @@ class Scheduler:
         elif r.state == WAITING:
             self.waiting.remove(r)
         r.state = FINISHED
+        r.pending = 0
         r.finish_reason = reason

@@ -37,6 +37,9 @@ class StepItem:
     rid: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)
+    # the last of `tokens` is not known on the host yet: the device takes the token this request
+    # drew in the step before (the value given here is ignored)
+    pending_last: bool = False
 
 
 class _Staging:
@@ -102,6 +105,8 @@ class StepFunction:
         self._graphs = {}  # shape -> (graph, logits) once captured, or the count of eager runs
         self.graph_replays = 0
         self._graph_generation = 0
+        self.last_tokens = torch.zeros(manager.max_requests, dtype=torch.int32, device=self.device)
+        self.last_context: Optional[StepContext] = None
 
     # -- validation -----------------------------------------------------------
     def _validate(self, items: Sequence[StepItem]) -> None:
@@ -169,6 +174,7 @@ class StepFunction:
         ctx, lengths = self.prepare(items)
         logits = self._forward(ctx)
         self.commit(items, lengths)
+        self.last_context = ctx
         return logits
 
     def commit(self, items: Sequence[StepItem], lengths: Sequence[int]) -> None:
@@ -187,9 +193,17 @@ class StepFunction:
         q_lens = [len(it.tokens) for it in items]
         all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64,
                                  count=sum(q_lens))
+        if any(it.pending_last for it in items):
+            ends = np.cumsum(q_lens) - 1
+            for i, it in enumerate(items):
+                if it.pending_last:
+                    all_tokens[ends[i]] = 0  # checked as a valid id; replaced by a reference below
         if all_tokens.min() < 0 or all_tokens.max() >= self.model.vocab_size:
             bad = int(all_tokens[(all_tokens < 0) | (all_tokens >= self.model.vocab_size)][0])
             raise InvalidArgument(f"token id {bad} is outside [0, {self.model.vocab_size})")  # src/core/transformer.cpp:6195-6197
+        for i, it in enumerate(items):
+            if it.pending_last:
+                all_tokens[ends[i]] = -1 - mgr.slot(it.rid)
         mgr.reserve([(it.rid, f + n) for it, f, n in zip(items, first, q_lens)])
 
         S, N = len(items), sum(q_lens)
@@ -219,7 +233,7 @@ class StepFunction:
         cur = 0
         for name, size in (("token_ids", N), ("positions", N), ("tok_seq", N), ("seq_starts", S + 1),
                            ("context_lens", S), ("state_slots", S), ("logit_rows", max(R, 1)),
-                           ("attn_work", max(len(tiles), 1)), ("attn_single", max(len(singles), 1))):
+                           ("logit_slots", max(R, 1)), ("attn_work", max(len(tiles), 1)), ("attn_single", max(len(singles), 1))):
             off[name] = (cur, size)
             cur += size
         for g in range(G):
@@ -253,6 +267,8 @@ class StepFunction:
         view("context_lens")[:] = first_arr + q_arr
         slot_ids = np.asarray([mgr.slot(it.rid) for it in items], dtype=np.int64)
         view("state_slots")[:] = slot_ids
+        if R:
+            view("logit_slots")[:R] = [int(slot_ids[i]) for i, it in enumerate(items) for _ in it.want]
         for g in range(G):
             tables = mgr.table_rows(g)[slot_ids]  # [S, W]
             view(f"bt{g}").reshape(S, W)[:] = tables
@@ -286,6 +302,7 @@ class StepFunction:
                           attention_mode=mode, context_bucket=_bucket(max_context), n_attn_tiles=n_tiles,
                           n_attn_single=len(singles)),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
+            logit_slots=dview("logit_slots"), last_tokens=self.last_tokens,
             attn_work=dview("attn_work") if mode == "prefill" else None,
             attn_single_rows=dview("attn_single") if mode == "prefill" else None,
         )

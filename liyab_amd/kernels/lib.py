@@ -36,7 +36,7 @@ _SIGNATURES = {
     "liyab_check_device": [],
     "liyab_fill": [P, c_int, c_uint32, c_int64, P],
     "liyab_add_into": [P, P, c_int, c_int64, P],
-    "liyab_embed": [P, P, P, c_int, P, P, c_int, c_int, c_float, P],
+    "liyab_embed": [P, P, P, c_int, P, P, c_int, c_int, c_float, P, P],
     "liyab_add_rows": [P, P, c_int, P, c_int, c_int, P],
     "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
     "liyab_layernorm": [P, c_int, P, P, P, P, c_int, c_int, c_float, P],
@@ -50,8 +50,8 @@ _SIGNATURES = {
     "liyab_gemm_skinny_ln": [P, P, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_float, c_int, c_int, c_int, c_int,
                                 c_int, P],
-    "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P],
-    "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
+    "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
+    "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P, P, P],
 }
 
 

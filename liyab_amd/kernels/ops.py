@@ -103,9 +103,11 @@ def add_into_(residual: torch.Tensor, x: torch.Tensor) -> None:
 
 
 def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0,
-          pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
+          pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+          last_tokens: Optional[torch.Tensor] = None) -> None:
     """out[t] = scale * table[ids[t]] (+ pos_table[positions[t]]); out is float32 [n, d].
-    The caller has checked ids against the table's rows (and positions against pos_table's)."""
+    An id below zero stands for last_tokens[-1 - id]. The caller has checked ids against the
+    table's rows (and positions against pos_table's)."""
     _dev(out, "out")
     n, d = out.shape
     if out.dtype != torch.float32 or not out.is_contiguous():
@@ -119,8 +121,10 @@ def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: floa
         if positions is None:
             raise KernelError("embed: a position table needs positions")
         _i32(positions, "positions", n)
+    if last_tokens is not None:
+        _i32(last_tokens, "last_tokens")
     _lib.call("liyab_embed", out.data_ptr(), table.data_ptr(), _ptr(pos_table), dtype_code(table.dtype),
-              ids.data_ptr(), _ptr(positions), n, d, float(scale), _stream())
+              ids.data_ptr(), _ptr(positions), n, d, float(scale), _ptr(last_tokens), _stream())
 
 
 def add_rows_(x: torch.Tensor, table: torch.Tensor, rows: torch.Tensor) -> None:
@@ -227,8 +231,19 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
 _argmax_scratch = {}
 
 
-def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
-    """out[r] = the first maximal element of logits[r] (ties go to the lowest id)."""
+def _scatter(scatter, rows):
+    if scatter is None:
+        return None, None
+    index, target = scatter
+    _i32(index, "scatter index", rows)
+    _i32(target, "scatter target")
+    return index.data_ptr(), target.data_ptr()
+
+
+def argmax(out: torch.Tensor, logits: torch.Tensor, scatter=None) -> None:
+    """out[r] = the first maximal element of logits[r] (ties go to the lowest id). With
+    scatter = (index, target), target[index[r]] = out[r] too; the caller has checked the
+    indices against the target."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
     if logits.dtype != torch.float32:
@@ -240,11 +255,13 @@ def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
         cap = max(rows, 64) * 64
         sc = (torch.empty(cap, dtype=torch.float32, device=key), torch.empty(cap, dtype=torch.int32, device=key))
         _argmax_scratch[key] = sc
-    _lib.call("liyab_argmax", out.data_ptr(), logits.data_ptr(), ld, rows, V, sc[0].data_ptr(), sc[1].data_ptr(), _stream())
+    si, so = _scatter(scatter, rows)
+    _lib.call("liyab_argmax", out.data_ptr(), logits.data_ptr(), ld, rows, V, sc[0].data_ptr(), sc[1].data_ptr(), si, so,
+              _stream())
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
-           top_p: torch.Tensor, uniform: torch.Tensor) -> None:
+           top_p: torch.Tensor, uniform: torch.Tensor, scatter=None) -> None:
     """Per-row sampling; temperature/top_p float32 [rows], top_k int32 [rows], uniform float64 [rows] in [0, 1)."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
@@ -257,8 +274,9 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, t
     _dev(uniform, "uniform")
     if uniform.dtype != torch.float64 or uniform.numel() != rows or not uniform.is_contiguous():
         raise KernelError("sample: uniform must be contiguous float64 [rows]")
+    si, so = _scatter(scatter, rows)
     _lib.call("liyab_sample", out.data_ptr(), logits.data_ptr(), ld, rows, V, temperature.data_ptr(),
-              top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(), _stream())
+              top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(), si, so, _stream())
 
 
 EPI_QKV_PAGED = 4

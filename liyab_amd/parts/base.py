@@ -97,5 +97,7 @@ class StepContext:
     workspace: Workspace
     dtype: torch.dtype
     page_size: int
+    logit_slots: Optional[torch.Tensor] = None  # int32 [n_rows]: state slot of each wanted row's request
+    last_tokens: Optional[torch.Tensor] = None  # int32 [slots]: the token each request drew last (on the device)
     attn_work: Optional[torch.Tensor] = None  # int32 [n_attn_tiles, 4]: request index, first row, first position, queries
     attn_single_rows: Optional[torch.Tensor] = None  # int32 [n_attn_single]: rows attended one by one

@@ -21,7 +21,7 @@ class TokenEmbedding:
 
     def forward(self, ctx: StepContext, x: torch.Tensor, position_table: Optional[torch.Tensor] = None) -> None:
         ops.embed(x, self.table, ctx.token_ids, self.scale, pos_table=position_table,
-                  positions=ctx.positions if position_table is not None else None)
+                  positions=ctx.positions if position_table is not None else None, last_tokens=ctx.last_tokens)
 
 
 class LearnedPositions:

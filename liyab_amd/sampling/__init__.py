@@ -73,10 +73,12 @@ class Sampler:
             self._u = torch.empty(cap, dtype=torch.float64, device=self.device)
             self._cap = cap
 
-    def sample(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int]) -> List[int]:
-        """One token per row of `logits` [rows, vocab] (float32, device).
-        `seeds[r]` is row r's resolved seed and `indices[r]` how many tokens
-        its request has generated so far."""
+    def sample_on_device(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int],
+                         scatter=None):
+        """One token per row of `logits` [rows, vocab] (float32, device), left on the device:
+        returns an int32 tensor [rows] that stays valid until the next call. `seeds[r]` is row
+        r's resolved seed and `indices[r]` how many tokens its request has generated so far.
+        With scatter = (index, target), row r's token also goes to target[index[r]]."""
         import torch
 
         from ..kernels import ops
@@ -87,11 +89,16 @@ class Sampler:
         self._buffers(rows)
         out = self._out[:rows]
         if all(p.greedy for p in params):
-            ops.argmax(out, logits)
+            ops.argmax(out, logits, scatter=scatter)
         else:
             self._temp[:rows].copy_(torch.tensor([float(p.temperature) for p in params], dtype=torch.float32))
             self._topk[:rows].copy_(torch.tensor([int(p.top_k) for p in params], dtype=torch.int32))
             self._topp[:rows].copy_(torch.tensor([float(p.top_p) for p in params], dtype=torch.float32))
             self._u[:rows].copy_(torch.tensor([uniform(s, i) for s, i in zip(seeds, indices)], dtype=torch.float64))
-            ops.sample(out, logits, self._temp[:rows], self._topk[:rows], self._topp[:rows], self._u[:rows])
-        return out.tolist()
+            ops.sample(out, logits, self._temp[:rows], self._topk[:rows], self._topp[:rows], self._u[:rows],
+                       scatter=scatter)
+        return out
+
+    def sample(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int]) -> List[int]:
+        """The same, with the tokens brought to the host."""
+        return self.sample_on_device(logits, params, seeds, indices).tolist()

@@ -338,3 +338,34 @@ def test_real_widths_whole_and_mixed(name, dtype, sized_models):
         worst = tt.check_against_plain(got, reqs, refs[dtype], TOL[dtype], f"{name} {label} {dtype}")
         core.manager.check()
         del core
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_overlapped_steps_give_the_same_tokens(dtype, model_dirs):
+    """The engine launches the next step before it has read this step's tokens; with or without
+    that overlap, greedy or sampled, stopping at an end token or not, the tokens are the same."""
+    from liyab_amd import Engine, SamplingParams
+
+    name = "B"
+    V = CONFIGS[name][0]["vocab_size"]
+    prompts = [tt.random_tokens(80 + i, n, V) for i, n in enumerate([1, 13, 64, 100, 5, 30])]
+    for sp in (SamplingParams(temperature=0.0, max_tokens=40), SamplingParams(temperature=0.9, top_k=50, top_p=0.9, seed=9, max_tokens=40)):
+        results = {}
+        for overlap in (False, True):
+            engine = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=24, max_num_seqs=4, max_batched_tokens=48,
+                            prefill_chunk=32, overlap=overlap)
+            engine.stop_at_eos = False
+            free = engine.generate(prompts, sp)
+            # an end token that request 2 draws in the middle: it and others must stop there
+            eos = free[2].tokens[11]
+            engine.scheduler.eos_token_id = eos
+            engine.stop_at_eos = True
+            stopped = engine.generate(prompts, sp)
+            for a, b in zip(free, stopped):
+                cut = a.tokens.index(eos) + 1 if eos in a.tokens else len(a.tokens)
+                assert b.tokens == a.tokens[:cut]
+                assert b.finish_reason == ("stop" if eos in a.tokens else a.finish_reason)
+            results[overlap] = ([r.tokens for r in free], [r.tokens for r in stopped], engine.scheduler.stats.preemptions)
+            assert engine.core.manager.pages_in_use() == 0
+            engine.core.manager.check()
+        assert results[False][:2] == results[True][:2]

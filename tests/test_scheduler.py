@@ -158,3 +158,86 @@ def test_no_request_starves_under_pressure():
     assert steps < 2000
     for r in rs:
         assert r.generated == alone(r.prompt, 30)
+
+
+def run_lagged(m, s, limit=10000):
+    """The engine's overlapped loop: a step's tokens are read only after the next step has been
+    scheduled and launched; a request's last token stands as a placeholder meanwhile."""
+    inflight, steps = None, 0
+    while s.has_unfinished() or inflight is not None:
+        if inflight is not None and s.pressure():
+            s.resolve(*inflight)
+            inflight = None
+        batch = s.schedule()
+        if not batch:
+            assert inflight is not None
+            s.resolve(*inflight)
+            inflight = None
+            continue
+        assert sum(b.count for b in batch) <= s.max_batched_tokens
+        m.reserve([(b.request.rid, b.first + b.count) for b in batch])
+        for b in batch:
+            m.commit(b.request.rid, b.first + b.count)
+            assert b.request.pending <= 1
+        # what the device would sample: a function of the true tokens, which the host learns late
+        truth = {}
+        for b in batch:
+            if b.wants_logits:
+                r = b.request
+                known = Request("x", r.prompt + r.generated + ([r._late] if r.pending else []), r.params)
+                truth[r.rid] = next_token(known)
+                r._late = truth[r.rid]
+        s.advance(batch)
+        previous, inflight = inflight, (batch, truth)
+        if previous is not None:
+            s.resolve(*previous)
+        m.check()
+        steps += 1
+        assert steps < limit
+    return steps
+
+
+def test_overlapped_loop_gives_the_same_tokens_and_sees_eos_a_step_late():
+    prompts = [[3, 4, 5], list(range(40)), [9] * 17, [1]]
+    want = [alone(p, 25) for p in prompts]
+    eos = want[1][6]  # request 1 stops at its 7th token
+    m, s = setup(num_pages=64, budget=32, chunk=16, max_num_seqs=4, eos=eos)
+    rs = [Request(f"r{i}", list(p), SamplingParams(temperature=0, max_tokens=25)) for i, p in enumerate(prompts)]
+    for r in rs:
+        s.add(r)
+    run_lagged(m, s)
+    for r, w in zip(rs, want):
+        cut = w.index(eos) + 1 if eos in w else len(w)
+        assert r.generated == w[:cut], r.rid
+        assert r.finish_reason == ("stop" if eos in w else "length") and r.pending == 0
+    assert m.pages_in_use() == 0 and m.free_slots() == 8
+    m.check()
+
+
+def test_overlapped_loop_under_page_pressure_reads_tokens_before_preempting():
+    m, s = setup(num_pages=8, budget=64, chunk=32, max_num_seqs=3)
+    rs = [Request(f"r{i}", [i + 3] * 30, SamplingParams(temperature=0, max_tokens=45)) for i in range(3)]
+    for r in rs:
+        s.add(r)
+    run_lagged(m, s)
+    assert s.stats.preemptions >= 1
+    for r in rs:
+        assert r.generated == alone(r.prompt, 45), r.rid
+    assert m.pages_in_use() == 0
+
+
+def test_a_request_at_its_last_token_is_not_scheduled_again():
+    m, s = setup(max_positions=32)
+    r = Request("a", list(range(30)), SamplingParams(temperature=0, max_tokens=10))
+    s.add(r)
+    run_lagged(m, s)
+    assert r.finish_reason == "context" and len(r.generated) == 3
+    m2, s2 = setup()
+    r2 = Request("b", [1, 2], SamplingParams(temperature=0, max_tokens=1))
+    s2.add(r2)
+    batch = s2.schedule()
+    m2.reserve([("b", 2)]); m2.commit("b", 2)
+    s2.advance(batch)
+    assert s2.draining(r2) and s2.schedule() == []  # nothing to run while its only token is pending
+    s2.resolve(batch, {"b": 7})
+    assert r2.generated == [7] and r2.finish_reason == "length"
