@@ -21,12 +21,10 @@ typedef uint16_t bf16_t;  // bfloat16 bits
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even; NaN stays NaN. The cast is gfx950's conversion instruction.
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<bf16_t>(u >> 16);
+    const __bf16 b = static_cast<__bf16>(f);
+    return __builtin_bit_cast(bf16_t, b);
 }
 
 template <typename T>

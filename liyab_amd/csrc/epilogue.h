@@ -34,10 +34,25 @@ struct EpiParams {
     int exact;                // erf in double (32-bit path)
 };
 
-template <typename OutT>
+// `MODE` >= 0 fixes the epilogue at compile time (straight-line code in the kernels' store
+// loops); -1 reads it from the parameters.
+// The bias of column n (0 without one). Kernels that store several rows of a column load it
+// once, ahead of their store loop: a load between two stores would have to wait for the first
+// store, since the compiler cannot know that outputs and bias do not overlap.
+__device__ __forceinline__ float epilogue_bias(const EpiParams& p, int n) { return p.bias != nullptr ? p.bias[n] : 0.0f; }
+
+template <typename OutT, int MODE = -1>
+__device__ __forceinline__ void epilogue_store_biased(const EpiParams& p, int m, int n, float v);
+
+template <typename OutT, int MODE = -1>
 __device__ __forceinline__ void epilogue_store(const EpiParams& p, int m, int n, float v) {
-    if (p.bias != nullptr) v += p.bias[n];
-    switch (p.mode) {
+    epilogue_store_biased<OutT, MODE>(p, m, n, v + epilogue_bias(p, n));
+}
+
+// `v` already holds the bias.
+template <typename OutT, int MODE>
+__device__ __forceinline__ void epilogue_store_biased(const EpiParams& p, int m, int n, float v) {
+    switch (MODE >= 0 ? MODE : p.mode) {
         case kEpiGeluTanh: v = gelu_tanh(v); break;
         case kEpiGeluErf: v = p.exact ? gelu_erf_exact(v) : gelu_erf_fast(v); break;
         case kEpiResidual:
@@ -59,6 +74,32 @@ __device__ __forceinline__ void epilogue_store(const EpiParams& p, int m, int n,
         default: break;
     }
     static_cast<OutT*>(p.out)[static_cast<int64_t>(m) * p.ldo + n] = from_float<OutT>(v);
+}
+
+// The paged QKV epilogue for kernels whose lanes hold several rows of one column: what depends
+// on the row (its slot's place in the pages) is computed once per row, ahead of the stores.
+// Element offset of row m's slot for head 0, dimension 0; -1 for a token without a slot.
+__device__ __forceinline__ int64_t qkv_row_base(const EpiParams& p, int m) {
+    const int64_t slot = p.slots[m];
+    if (slot < 0) return -1;
+    return (slot / p.page_size) * (static_cast<int64_t>(p.n_kv_head) * p.page_size * p.hd) + (slot % p.page_size) * p.hd;
+}
+// What depends on the column: -1 for a query column, else the offset of (head, dimension)
+// within a page, with bit 62 set for values.
+__device__ __forceinline__ int64_t qkv_col_offset(const EpiParams& p, int n) {
+    if (n < p.q_dim) return -1;
+    const bool is_v = n >= p.q_dim + p.kv_dim;
+    const int c = n - p.q_dim - (is_v ? p.kv_dim : 0);
+    return (static_cast<int64_t>(c / p.hd) * p.page_size * p.hd + c % p.hd) | (is_v ? (int64_t{1} << 62) : 0);
+}
+template <typename OutT>
+__device__ __forceinline__ void qkv_store(const EpiParams& p, int m, int n, int64_t row_base, int64_t col_offset, float v) {
+    if (col_offset < 0) {
+        static_cast<OutT*>(p.out)[static_cast<int64_t>(m) * p.ldo + n] = from_float<OutT>(v);
+    } else if (row_base >= 0) {
+        const bool is_v = (col_offset >> 62) & 1;
+        static_cast<OutT*>(is_v ? p.vc : p.kc)[row_base + (col_offset & ~(int64_t{1} << 62))] = from_float<OutT>(v);
+    }
 }
 
 // Host-side check shared by the launchers.

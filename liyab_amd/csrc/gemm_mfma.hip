@@ -34,7 +34,13 @@ gemm_mfma_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __rest
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int wm = wave / 2, wn = wave % 2;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // Workgroups go to the 8 XCDs round-robin, each XCD with an L2 of its own. Tile t of the
+    // row-major tile order goes to the XCD that holds the tiles around it, so that an XCD's
+    // tiles share a few row blocks of `a` and its L2 holds them beside all of `w`.
+    const int tiles_n = (N + BN - 1) / BN, n_tiles = tiles_n * ((M + BM - 1) / BM);
+    const int xcd = blockIdx.x % 8, base = n_tiles / 8, rem = n_tiles % 8;
+    const int tile_id = xcd * base + min(xcd, rem) + blockIdx.x / 8;
+    const int m0 = (tile_id / tiles_n) * BM, n0 = (tile_id % tiles_n) * BN;
     const int li = lane % 32, lk = (lane / 32) * 8;
 
     floatx16 acc[TM][TN];
@@ -101,23 +107,55 @@ gemm_mfma_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __rest
         }
     }
     // C block layout: lane holds column li; rows 8 * (r / 4) + 4 * (lane / 32) + r % 4
+    // tiles wholly inside the output skip the per-element bounds checks (a guarded store is a
+    // branch of its own: on an interior tile they cost as much as the whole product)
+    const bool inside = m0 + BM <= M && n0 + BN <= N;
+    if (epi.mode == kEpiQkvPaged) {
+        // keys and values go to their pages: the rows' page places first, then the stores
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * (lane / 32);
+            int64_t row_base[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) row_base[r] = qkv_row_base(epi, min(mb + 8 * (r / 4) + r % 4, M - 1));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = n0 + wn * (BN / 2) + j * 32 + li;
+                if (n >= N) continue;
+                const float bias_n = epilogue_bias(epi, n);
+                const int64_t col = qkv_col_offset(epi, n);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mb + 8 * (r / 4) + r % 4;
+                    if (inside || m < M) qkv_store<OutT>(epi, m, n, row_base[r], col, acc[i][j][r] + bias_n);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int n = n0 + wn * (BN / 2) + j * 32 + li;
-            if (n >= N) continue;
+            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * (lane / 32);
+            const float bias_n = n < N ? epilogue_bias(epi, n) : 0.0f;
+            if (inside) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-                if (m < M) epilogue_store<OutT>(epi, m, n, acc[i][j][r]);
+                for (int r = 0; r < 16; ++r) epilogue_store_biased<OutT, -1>(epi, mb + 8 * (r / 4) + r % 4, n, acc[i][j][r] + bias_n);
+            } else if (n < N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mb + 8 * (r / 4) + r % 4;
+                    if (m < M) epilogue_store_biased<OutT, -1>(epi, m, n, acc[i][j][r] + bias_n);
+                }
             }
         }
 }
 
 template <int BM, int BN>
 int launch_mfma(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
-    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+    dim3 grid(((N + BN - 1) / BN) * ((M + BM - 1) / BM));
     const size_t smem = 2 * static_cast<size_t>(BM + BN) * GLD * sizeof(bf16_t);
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);

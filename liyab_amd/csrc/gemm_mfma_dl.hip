@@ -1,0 +1,225 @@
+// out[M,N] = a[M,K] . w[N,K]^T in bfloat16 on the matrix cores, with tiles
+// brought from global memory straight into LDS (global_load_lds, 16 bytes a
+// lane) in a ring of three stages, so that two tiles of K are in flight
+// while one is multiplied. For steps of many tokens; K must be a multiple of
+// 64 (other shapes go to the register-staged kernel in gemm_mfma.hip).
+//
+// A wave's direct load fills 1 KiB of LDS contiguously, lane after lane: 8
+// rows of 64 k. Rows are therefore unpadded (128 bytes), and bank conflicts
+// of the 16-byte fragment reads are avoided by a swizzle: within a row, the
+// 16-byte piece c sits at position c ^ (row & 7), applied on the
+// global side when loading and again when reading. Rows past M or N are
+// clamped to the last valid row; their results are never stored. MFMA
+// operand layout and the fixed-order sum over k are those of gemm_mfma.hip.
+#include "common.h"
+#include "epilogue.h"
+
+namespace liyab {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+constexpr int DBK = 64;      // k per stage
+
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
+__global__ void __launch_bounds__(256)
+gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
+                    EpiParams epi) {
+    constexpr int TM = BM / 64, TN = BN / 64;
+    constexpr int STAGE = (BM + BN) * DBK;      // elements per stage: the tile of a, then the tile of w
+    constexpr int A_LOADS = BM / 8 / 4, W_LOADS = BN / 8 / 4;  // wave-loads (8 rows each) per wave and stage
+    extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
+
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wm = wave / 2, wn = wave % 2;
+    // Workgroups go to the 8 XCDs round-robin, each XCD with an L2 of its own. Tile t of the
+    // row-major tile order goes to the XCD that holds the tiles around it, so that an XCD's
+    // tiles share a few row blocks of `a` and its L2 holds them beside all of `w`.
+    const int tiles_n = (N + BN - 1) / BN, n_tiles = tiles_n * ((M + BM - 1) / BM);
+    const int xcd = blockIdx.x % 8, base = n_tiles / 8, rem = n_tiles % 8;
+    const int tile_id = xcd * base + min(xcd, rem) + blockIdx.x / 8;
+    const int m0 = (tile_id / tiles_n) * BM, n0 = (tile_id % tiles_n) * BN;
+    const int li = lane % 32, g = lane / 32;
+
+    // this lane's part in a wave-load: row lane / 8 of the 8, LDS piece position lane % 8
+    const int lrow = lane / 8, lpos = lane % 8;
+    auto issue = [&](int kt, int stage) {
+        const int k0 = kt * DBK;
+        bf16_t* sa = lds + stage * STAGE;
+        bf16_t* sw = sa + BM * DBK;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int r0 = (wave * A_LOADS + i) * 8, row = r0 + lrow;
+            const int c = lpos ^ (row & 7);
+            const bf16_t* src = a + static_cast<int64_t>(min(m0 + row, M - 1)) * lda + k0 + c * 8;
+            __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sa + r0 * DBK), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            const int r0 = (wave * W_LOADS + i) * 8, row = r0 + lrow;
+            const int c = lpos ^ (row & 7);
+            const bf16_t* src = w + static_cast<int64_t>(min(n0 + row, N - 1)) * K + k0 + c * 8;
+            __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sw + r0 * DBK), 16, 0, 0);
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const int nk = K / DBK;
+    constexpr int AHEAD = DSTAGES - 1;  // tiles of K in flight or in use beside the one being multiplied
+#pragma unroll
+    for (int p = 0; p < AHEAD; ++p)
+        if (p < nk) issue(p, p);
+    for (int kt = 0; kt < nk; ++kt) {
+        // tile kt must have landed: the loads of the tiles after it may still be in flight (a
+        // wave's loads complete in order, A_LOADS + W_LOADS a tile)
+        const int later = min(nk - 1 - kt, AHEAD - 1);
+        if (later >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (A_LOADS + W_LOADS)) : "memory");
+        else if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (A_LOADS + W_LOADS)) : "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + W_LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // everyone's loads of tile kt are in LDS; everyone is done reading tile kt - 1. A bare
+        // barrier: __syncthreads() would also wait for the loads still meant to be in flight.
+        __builtin_amdgcn_s_barrier();
+        if (kt + AHEAD < nk) issue(kt + AHEAD, (kt + AHEAD) % DSTAGES);  // into the stage tile kt - 1 used
+        const bf16_t* sa = lds + (kt % DSTAGES) * STAGE;
+        const bf16_t* sw = sa + BM * DBK;
+        // fragments of slab ks + 1 are read from LDS while slab ks multiplies
+        bf16x8 fa[2][TM], fw[2][TN];
+        auto read_frags = [&](int ks, int buf) {
+            const int c = ks * 2 + g;  // the 16-byte piece of the row this lane needs
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wm * (BM / 2) + i * 32 + li;
+                fa[buf][i] = *reinterpret_cast<const bf16x8*>(sa + row * DBK + ((c ^ (row & 7)) * 8));
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int row = wn * (BN / 2) + j * 32 + li;
+                fw[buf][j] = *reinterpret_cast<const bf16x8*>(sw + row * DBK + ((c ^ (row & 7)) * 8));
+            }
+        };
+        read_frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < DBK / 16; ++ks) {
+            if (ks + 1 < DBK / 16) read_frags(ks + 1, (ks + 1) & 1);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fw[ks & 1][j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // tiles wholly inside the output skip the per-element bounds checks (a guarded store is a
+    // branch of its own: on an interior tile they cost as much as the whole product)
+    const bool inside = m0 + BM <= M && n0 + BN <= N;
+    if constexpr (EPI == kEpiQkvPaged) {
+        // keys and values go to their pages: the rows' page places first, then the stores
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * g;
+            int64_t row_base[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) row_base[r] = qkv_row_base(epi, min(mb + 8 * (r / 4) + r % 4, M - 1));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = n0 + wn * (BN / 2) + j * 32 + li;
+                if (n >= N) continue;
+                const float bias_n = epilogue_bias(epi, n);
+                const int64_t col = qkv_col_offset(epi, n);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mb + 8 * (r / 4) + r % 4;
+                    if (inside || m < M) qkv_store<OutT>(epi, m, n, row_base[r], col, acc[i][j][r] + bias_n);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * (BN / 2) + j * 32 + li;
+            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * g;
+            const float bias_n = n < N ? epilogue_bias(epi, n) : 0.0f;
+            if (inside) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) epilogue_store_biased<OutT, EPI>(epi, mb + 8 * (r / 4) + r % 4, n, acc[i][j][r] + bias_n);
+            } else if (n < N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = mb + 8 * (r / 4) + r % 4;
+                    if (m < M) epilogue_store_biased<OutT, EPI>(epi, m, n, acc[i][j][r] + bias_n);
+                }
+            }
+        }
+}
+
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
+int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
+    const int grid = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+    const size_t smem = static_cast<size_t>(DSTAGES) * (BM + BN) * DBK * sizeof(bf16_t);
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI>;
+    static bool ready = false;  // once per instantiation, outside any stream capture's first use
+    if (!ready) {
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        ready = true;
+    }
+    kern<<<grid, 256, smem, stream>>>(a, lda, w, M, N, K, epi);
+    return check_launch("gemm_mfma_dl");
+}
+
+template <int BM, int BN, int DSTAGES>
+int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
+    auto* pa = static_cast<const bf16_t*>(a);
+    auto* pw = static_cast<const bf16_t*>(w);
+    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.out_dtype == kF32) {
+        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone>(pa, lda, pw, M, N, K, epi, stream);
+        return launch_dl_as<BM, BN, DSTAGES, float, -1>(pa, lda, pw, M, N, K, epi, stream);
+    }
+    switch (epi.mode) {
+        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged>(pa, lda, pw, M, N, K, epi, stream);
+        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1>(pa, lda, pw, M, N, K, epi, stream);
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+// tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep; 6 = 64x64 with
+// four stages (0 = chosen from the shape).
+extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
+                                  const EpiParams* epi_in, hipStream_t stream) {
+    LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
+    LIYAB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma_dl: bad sizes M=%d N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(K % DBK == 0 && lda % 8 == 0 && lda >= K, "gemm_mfma_dl: K %d must be a multiple of 64 and lda %lld of 8", K,
+                  static_cast<long long>(lda));
+    LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0,
+                  "gemm_mfma_dl: operands must be 16-byte aligned");
+    EpiParams epi = *epi_in;
+    if (int rc = check_epilogue(epi, M, N)) return rc;
+    // measured on {256..2048} x {768, 2304, 3072} x {768, 3072}: 64 x 64 tiles, three workgroups a
+    // CU, win or tie everywhere; a long K likes one more stage in flight
+    if (tile == 0) tile = K >= 2048 ? 6 : 2;
+    switch (tile) {
+        case 1: return launch_dl<128, 128, 3>(a, lda, w, M, N, K, epi, stream);
+        case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
+        case 3: return launch_dl<128, 64, 3>(a, lda, w, M, N, K, epi, stream);
+        case 5: return launch_dl<128, 192, 3>(a, lda, w, M, N, K, epi, stream);
+        case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
+        default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
+    }
+}

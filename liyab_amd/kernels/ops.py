@@ -374,6 +374,21 @@ def skinny_ln_takes(M: int, K: int, N: int = 0) -> bool:
     return 0 < M <= 16 and K % 8 == 0 and K <= 2048 and M * (K + 8) * 2 <= 65536 and N <= 8192
 
 
+def gemm_mfma_dl(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
+                 epilogue: int = EPI_NONE, kv=None, tile: int = 0) -> None:
+    """The matrix-core product with tiles loaded straight into LDS, three stages deep; bfloat16
+    operands, K a multiple of 64."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_mfma_dl: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
+    if K % 64 != 0 or M == 0:
+        raise KernelError(f"gemm_mfma_dl: K = {K} must be a multiple of 64 and M positive")
+    e = _epilogue(a, w, bias, out, residual, epilogue, kv)
+    _lib.call("liyab_gemm_mfma_dl", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, tile, ctypes.byref(e), _stream())
+
+
 def mfma_takes(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
             and w.data_ptr() % 16 == 0)
@@ -390,6 +405,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
             # kernel's shared loads beat every workgroup re-reading the tokens)
             gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=0)
+        elif a.shape[1] % 64 == 0:
+            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
         else:
             gemm_mfma(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
         return

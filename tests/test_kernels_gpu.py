@@ -107,9 +107,11 @@ def test_gemm_float32(ops, M, N, K, epilogue):
         assert torch.equal(one[0], full[M // 2])
 
 
-@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w"])
+@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w",
+                                    "dl1", "dl2", "dl3", "dl5", "dl6"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
-@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
+                                                 (500, 300, 128), (129, 193, 192)])
 def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
     a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
     tiles = {"mfma128": 1, "mfma64": 2, "mfma128x64": 3}
@@ -117,8 +119,13 @@ def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
     if kernel.startswith("skinny") and M > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
 
+    if kernel.startswith("dl") and K % 64 != 0:
+        pytest.skip("the direct-load kernel takes K in multiples of 64")
+
     def run(**kw):
-        if kernel.startswith("skinny"):
+        if kernel.startswith("dl"):
+            ops.gemm_mfma_dl(a, w, bias, tile=int(kernel[2:]), **kw)
+        elif kernel.startswith("skinny"):
             ops.gemm_skinny(a, w, bias, ksplit=int(kernel[6:].rstrip("w")), wide=1 if kernel.endswith("w") else 0, **kw)
         elif kernel == "simple":
             ops.gemm_simple(a, w, bias, **kw)
@@ -414,3 +421,37 @@ def test_sampler_against_the_plain_sampler(ops):
             if got[r] != want:
                 cdf = np.cumsum(probs)
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (r, params[r], got[r], want)
+
+
+@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl5", "auto"])
+@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
+def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
+    """Queries to a dense buffer, keys and values straight into shuffled cache slots, against
+    the plain product followed by the scatter kernel."""
+    if kernel == "skinny" and M > 64:
+        pytest.skip("at most 64 rows")
+    q_dim, kv_dim = H * hd, Hkv * hd
+    N = q_dim + 2 * kv_dim
+    a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    pages = -(-M // page) + 3
+    slots = torch.randperm(pages * page)[:M].to(torch.int32).to(DEV)
+    kc = torch.zeros(pages, Hkv, page, hd, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    q = torch.zeros(M, q_dim, dtype=torch.bfloat16, device=DEV)
+    kw = dict(out=q, epilogue=ops.EPI_QKV_PAGED, kv=(kc, vc, slots, q_dim))
+    if kernel == "skinny":
+        ops.gemm_skinny(a, w, bias, **kw)
+    elif kernel == "auto":
+        ops.gemm(a, w, bias, **kw)
+    elif kernel.startswith("dl"):
+        ops.gemm_mfma_dl(a, w, bias, tile=int(kernel[2:]), **kw)
+    else:
+        ops.gemm_mfma(a, w, bias, tile=1 if kernel == "mfma128" else 2, **kw)
+    full = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_simple(a, w, bias, out=full)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.kv_write(kc2, vc2, full, q_dim, q_dim + kv_dim, slots)
+    close(q, full[:, :q_dim], 1e-2, "queries")
+    close(kc, kc2, 1e-2, "keys")
+    close(vc, vc2, 1e-2, "values")
+    assert (kc == 0).sum() == (kc2 == 0).sum()  # nothing written outside the tokens' slots
