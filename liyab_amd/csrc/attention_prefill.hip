@@ -31,17 +31,19 @@ union QFrag {
 
 constexpr int AP_KEYS = 32;     // keys per block
 constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
+constexpr int AP_DEPTH = 6;     // blocks of keys and values in flight in registers
+constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LDS
 
 template <int DB>  // head dimension padded to 32 * DB
 __global__ void __launch_bounds__(256)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
-                         int window, int n_head, int n_kv_head, int hd, int page_size) {
+                         int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift) {
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[AP_KEYS * LDK];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[AP_KEYS * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t Kb[2][AP_KEYS * LDK];  // two stages: the next block's keys
+    __shared__ __attribute__((aligned(16))) bf16_t Vb[2][AP_KEYS * LDK];  // and values load while this one is used
     __shared__ __attribute__((aligned(16))) bf16_t Os[4][32 * LDK];
 
     const int* wk = work + 4 * blockIdx.x;
@@ -57,6 +59,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     const int wave_last = pos0 + min(32 * wave + 31, nq - 1);  // the wave's latest query position
     const bool wave_has = 32 * wave < nq;
     const int n_slabs = hd / 16;
+    const float scale2 = scale * 1.4426950408889634f;  // log2(e): exp(x) = 2^(x log2 e)
 
     QFrag qf[2 * DB];
     {
@@ -79,23 +82,60 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     const int64_t page_stride = static_cast<int64_t>(n_kv_head) * page_size * hd;
     const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd;
     constexpr int CHUNKS = 4 * DB;  // 16-byte pieces per padded row
-
-    for (int kb = (k_lo / AP_KEYS) * AP_KEYS; kb <= k_hi; kb += AP_KEYS) {
-        // stage the block's keys and values (zeros past the head dimension and past the last key)
-        for (int c = tid; c < AP_KEYS * CHUNKS; c += 256) {
-            const int key = c / CHUNKS, col = (c % CHUNKS) * 8;
-            const int kp = kb + key;
-            u32x4 kvv = {0, 0, 0, 0}, vvv = {0, 0, 0, 0};
-            if (kp >= k_lo && kp <= k_hi && col < hd) {
-                const int64_t at = static_cast<int64_t>(bt[kp / page_size]) * page_stride + head_off +
-                                   static_cast<int64_t>(kp % page_size) * hd + col;
-                kvv = *reinterpret_cast<const u32x4*>(kc + at);
-                vvv = *reinterpret_cast<const u32x4*>(vc + at);
-            }
-            *reinterpret_cast<u32x4*>(Ks + key * LDK + col) = kvv;
-            *reinterpret_cast<u32x4*>(Vs + key * LDK + col) = vvv;
+    // a block's keys and values go global -> registers -> LDS (zeros past the head dimension,
+    // before the window and past the last key). AP_DEPTH register sets form a ring: a block is
+    // fetched AP_DEPTH - 1 blocks before it is multiplied, which covers the latency of the pages.
+    constexpr int PER = (AP_KEYS * CHUNKS + 255) / 256;
+    u32x4 rk[AP_DEPTH][PER], rv[AP_DEPTH][PER];
+    // The request's page ids wait in LDS, so that a fetch is one load deep; and a fetch is
+    // branch-free (a position outside the range reads a valid one and is zeroed when it is
+    // put into LDS): a load under a branch would have to be waited for where the branch ends.
+    __shared__ int sbt[AP_MAX_BLOCKS];
+    const int first_page = k_lo / page_size, n_pages = k_hi / page_size - first_page + 1;
+    for (int i = tid; i < n_pages; i += 256) sbt[i] = bt[first_page + i];  // the host has checked that they fit
+    __syncthreads();
+    auto fetch = [&](int kb, u32x4 (&fk)[PER], u32x4 (&fv)[PER]) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int c = min(tid + 256 * i, AP_KEYS * CHUNKS - 1), key = c / CHUNKS, col = min((c % CHUNKS) * 8, hd - 8);
+            const int kp = min(max(kb + key, k_lo), k_hi);
+            // page_shift >= 0: the page size is a power of two (no integer division)
+            const int lp = page_shift >= 0 ? kp >> page_shift : kp / page_size;
+            const int off = page_shift >= 0 ? kp & (page_size - 1) : kp % page_size;
+            const int64_t page = sbt[lp - first_page];
+            const int64_t at = page * page_stride + head_off + static_cast<int64_t>(off) * hd + col;
+            fk[i] = *reinterpret_cast<const u32x4*>(kc + at);
+            fv[i] = *reinterpret_cast<const u32x4*>(vc + at);
         }
-        __syncthreads();
+    };
+    auto stash = [&](int buf, int kb, const u32x4 (&fk)[PER], const u32x4 (&fv)[PER]) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int c = tid + 256 * i, key = c / CHUNKS, col = (c % CHUNKS) * 8;
+            if (c < AP_KEYS * CHUNKS) {
+                const int kp = kb + key;
+                const bool ok = kp >= k_lo && kp <= k_hi && col < hd;
+                const u32x4 zero = {0, 0, 0, 0};
+                *reinterpret_cast<u32x4*>(&Kb[buf][key * LDK + col]) = ok ? fk[i] : zero;
+                *reinterpret_cast<u32x4*>(&Vb[buf][key * LDK + col]) = ok ? fv[i] : zero;
+            }
+        }
+    };
+    const int kb0 = (k_lo / AP_KEYS) * AP_KEYS;
+#pragma unroll
+    for (int d = 0; d < AP_DEPTH; ++d) fetch(kb0 + d * AP_KEYS, rk[d], rv[d]);
+    stash(0, kb0, rk[0], rv[0]);
+    __syncthreads();
+    int cur = 0;
+    for (int kbase = kb0; kbase <= k_hi; kbase += AP_DEPTH * AP_KEYS) {
+#pragma unroll
+      for (int ring = 0; ring < AP_DEPTH; ++ring) {
+        const int kb = kbase + ring * AP_KEYS;
+        if (kb > k_hi) break;
+        const bool more = kb + AP_KEYS <= k_hi;
+        fetch(kb + AP_DEPTH * AP_KEYS, rk[ring], rv[ring]);  // this set's block is in LDS already
+        const bf16_t* Ks = Kb[cur];
+        const bf16_t* Vs = Vb[cur];
         if (wave_has && kb <= wave_last) {
             // S^T[key][query] = sum_d K[key][d] Q[query][d]
             floatx16 st;
@@ -109,14 +149,25 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                     st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[s].v, st, 0, 0, 0);
                 }
             }
-            // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4
+            // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4. Scores are kept in the
+            // base-2 domain (scale carries log2 e), so that exponentials are bare v_exp_f32.
+            // A block every query of the wave sees whole needs no mask.
+            const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * wave && (window <= 0 || kb > wave_last - window);
             float bm = -INFINITY;
+            if (whole) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
-                const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
-                st[r] = ok ? st[r] * scale : -INFINITY;
-                bm = fmaxf(bm, st[r]);
+                for (int r = 0; r < 16; ++r) {
+                    st[r] *= scale2;
+                    bm = fmaxf(bm, st[r]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
+                    const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
+                    st[r] = ok ? st[r] * scale2 : -INFINITY;
+                    bm = fmaxf(bm, st[r]);
+                }
             }
             bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
             const float m_new = fmaxf(m_run, bm);
@@ -126,10 +177,10 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[0].h[e] = pf[1].h[e] = 0;
             } else {
-                corr = m_run == -INFINITY ? 0.0f : __expf(m_run - m_new);
+                corr = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float p = __expf(st[r] - m_new);  // exp(-inf) = 0 for masked keys
+                    const float p = __builtin_amdgcn_exp2f(st[r] - m_new);  // 2^-inf = 0 for masked keys
                     bs += p;
                     pf[r / 8].h[r % 8] = float_to_bf16(p);
                 }
@@ -137,12 +188,16 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
             bs += __shfl_xor(bs, 32, 64);
             l_run = l_run * corr + bs;
             m_run = m_new;
+            // the running outputs are rescaled only when some query's maximum moved
+            const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.0f) != 0;
             // O^T[d][query] += sum_key V[key][d] P[key][query]; instruction s2 contracts the keys
             // of accumulator registers 8 s2 .. 8 s2 + 7: rows 16 s2 + 4 g2 + {0..3} and + 8
 #pragma unroll
             for (int d = 0; d < DB; ++d) {
+                if (rescale) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[d][r] *= corr;
+                    for (int r = 0; r < 16; ++r) o[d][r] *= corr;
+                }
 #pragma unroll
                 for (int s2 = 0; s2 < 2; ++s2) {
                     QFrag vf;
@@ -155,7 +210,10 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 }
             }
         }
-        __syncthreads();
+        if (more) stash(cur ^ 1, kb + AP_KEYS, rk[(ring + 1) % AP_DEPTH], rv[(ring + 1) % AP_DEPTH]);  // block kb + 32, fetched long ago
+        lds_barrier();  // the blocks still in flight stay in flight
+        cur ^= 1;
+      }
     }
     // o[d][r] = O^T[dim = 32 d + 8 (r / 4) + 4 g2 + r % 4][query ql]: through LDS to rows of 16-byte pieces
     if (wave_has) {
@@ -200,7 +258,11 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
                   "attention_prefill: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(window >= 0, "attention_prefill: negative window");
+    LIYAB_REQUIRE(max_blocks <= AP_MAX_BLOCKS, "attention_prefill: block tables of %d pages; at most %d are taken", max_blocks, AP_MAX_BLOCKS);
     if (n_tiles == 0) return 0;
+    int page_shift = -1;
+    for (int b = 0; b < 31; ++b)
+        if ((1 << b) == page_size) page_shift = b;
     dim3 grid(n_tiles, n_head);
     auto* o = static_cast<bf16_t*>(out);
     auto* pq = static_cast<const bf16_t*>(q);
@@ -209,7 +271,7 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
 #define LIYAB_GO(D)                                                                                                \
     attention_prefill_kernel<D><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables,      \
                                                           max_blocks, work, scale, window, n_head, n_kv_head, hd, \
-                                                          page_size)
+                                                          page_size, page_shift)
     if (hd <= 32) LIYAB_GO(1);
     else if (hd <= 64) LIYAB_GO(2);
     else if (hd <= 96) LIYAB_GO(3);

@@ -48,6 +48,15 @@ int check_launch(const char* what);
 
 constexpr int kWave = 64;
 
+// A workgroup barrier that orders LDS traffic only: this wave's LDS reads and writes are done
+// before it, but global loads may stay in flight across it. __syncthreads() also waits for every
+// outstanding global load, which throws away whatever a kernel prefetched into registers.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

@@ -225,7 +225,11 @@ class StepFunction:
                     singles.extend(range(a, a + n))
                 else:
                     for t0 in range(0, n, ATTN_TILE):
-                        tiles.extend((i, a + t0, f + t0, min(ATTN_TILE, n - t0)))
+                        tiles.append((i, a + t0, f + t0, min(ATTN_TILE, n - t0)))
+            # a tile's work grows with its last position: the longest first, so that the short
+            # ones fill the gaps at the end
+            tiles.sort(key=lambda t: -(t[2] + t[3]))
+            tiles = [v for t in tiles for v in t]
         n_tiles = len(tiles) // 4
 
         # layout of the metadata block (int32 words)

@@ -511,7 +511,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
     if fast and host.attention_mode == "decode":
         decode(None, out.shape[0])
         return
-    if fast and prefill_takes(hd) and ctx.attn_work is not None:
+    if fast and prefill_takes(hd) and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
         # long portions in tiles on the matrix cores, the short ones token by token
         if host.n_attn_tiles:
             attention_prefill(out, q, k_cache, v_cache, block_tables, ctx.attn_work, host.n_attn_tiles, n_head=n_head,
