@@ -34,8 +34,8 @@ constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
 constexpr int AP_DEPTH = 6;     // blocks of keys and values in flight in registers
 constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LDS
 
-template <int DB>  // head dimension padded to 32 * DB
-__global__ void __launch_bounds__(256)
+template <int DB, int WAVES>  // head dimension padded to 32 * DB; 32 * WAVES queries a tile
+__global__ void __launch_bounds__(64 * WAVES)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
@@ -44,7 +44,8 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
     __shared__ __attribute__((aligned(16))) bf16_t Kb[2][AP_KEYS * LDK];  // two stages: the next block's keys
     __shared__ __attribute__((aligned(16))) bf16_t Vb[2][AP_KEYS * LDK];  // and values load while this one is used
-    __shared__ __attribute__((aligned(16))) bf16_t Os[4][32 * LDK];
+    __shared__ __attribute__((aligned(16))) bf16_t Os[WAVES][32 * LDK];
+    constexpr int THREADS = 64 * WAVES;
 
     const int* wk = work + 4 * blockIdx.x;
     const int seq = wk[0], row0 = wk[1], pos0 = wk[2], nq = wk[3];
@@ -85,19 +86,19 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     // a block's keys and values go global -> registers -> LDS (zeros past the head dimension,
     // before the window and past the last key). AP_DEPTH register sets form a ring: a block is
     // fetched AP_DEPTH - 1 blocks before it is multiplied, which covers the latency of the pages.
-    constexpr int PER = (AP_KEYS * CHUNKS + 255) / 256;
+    constexpr int PER = (AP_KEYS * CHUNKS + THREADS - 1) / THREADS;
     u32x4 rk[AP_DEPTH][PER], rv[AP_DEPTH][PER];
     // The request's page ids wait in LDS, so that a fetch is one load deep; and a fetch is
     // branch-free (a position outside the range reads a valid one and is zeroed when it is
     // put into LDS): a load under a branch would have to be waited for where the branch ends.
     __shared__ int sbt[AP_MAX_BLOCKS];
     const int first_page = k_lo / page_size, n_pages = k_hi / page_size - first_page + 1;
-    for (int i = tid; i < n_pages; i += 256) sbt[i] = bt[first_page + i];  // the host has checked that they fit
+    for (int i = tid; i < n_pages; i += THREADS) sbt[i] = bt[first_page + i];  // the host has checked that they fit
     __syncthreads();
     auto fetch = [&](int kb, u32x4 (&fk)[PER], u32x4 (&fv)[PER]) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int c = min(tid + 256 * i, AP_KEYS * CHUNKS - 1), key = c / CHUNKS, col = min((c % CHUNKS) * 8, hd - 8);
+            const int c = min(tid + THREADS * i, AP_KEYS * CHUNKS - 1), key = c / CHUNKS, col = min((c % CHUNKS) * 8, hd - 8);
             const int kp = min(max(kb + key, k_lo), k_hi);
             // page_shift >= 0: the page size is a power of two (no integer division)
             const int lp = page_shift >= 0 ? kp >> page_shift : kp / page_size;
@@ -111,7 +112,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     auto stash = [&](int buf, int kb, const u32x4 (&fk)[PER], const u32x4 (&fv)[PER]) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int c = tid + 256 * i, key = c / CHUNKS, col = (c % CHUNKS) * 8;
+            const int c = tid + THREADS * i, key = c / CHUNKS, col = (c % CHUNKS) * 8;
             if (c < AP_KEYS * CHUNKS) {
                 const int kp = kb + key;
                 const bool ok = kp >= k_lo && kp <= k_hi && col < hd;
@@ -242,10 +243,11 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
 
 using namespace liyab;
 
-// work: n_tiles x (request index, first row, first position, queries <= 128), int32.
+// work: n_tiles x (request index, first row, first position, queries <= tile), int32; tile = 64 or 128
+// queries (2 or 4 waves a workgroup).
 extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                        const void* vc, const int* block_tables, int max_blocks, const int* work,
-                                       int n_tiles, float scale, int window, int n_head, int n_kv_head, int hd,
+                                       int n_tiles, int tile, float scale, int window, int n_head, int n_kv_head, int hd,
                                        int page_size, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
     LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -258,6 +260,7 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
                   "attention_prefill: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(window >= 0, "attention_prefill: negative window");
+    LIYAB_REQUIRE(tile == 64 || tile == 128, "attention_prefill: tiles of %d queries; 64 or 128 are taken", tile);
     LIYAB_REQUIRE(max_blocks <= AP_MAX_BLOCKS, "attention_prefill: block tables of %d pages; at most %d are taken", max_blocks, AP_MAX_BLOCKS);
     if (n_tiles == 0) return 0;
     int page_shift = -1;
@@ -268,10 +271,17 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     auto* pq = static_cast<const bf16_t*>(q);
     auto* pk = static_cast<const bf16_t*>(kc);
     auto* pv = static_cast<const bf16_t*>(vc);
-#define LIYAB_GO(D)                                                                                                \
-    attention_prefill_kernel<D><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables,      \
-                                                          max_blocks, work, scale, window, n_head, n_kv_head, hd, \
-                                                          page_size, page_shift)
+#define LIYAB_GO(D)                                                                                                  \
+    do {                                                                                                             \
+        if (tile == 64)                                                                                              \
+            attention_prefill_kernel<D, 2><<<grid, 128, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                     max_blocks, work, scale, window, n_head, n_kv_head, \
+                                                                     hd, page_size, page_shift);                      \
+        else                                                                                                         \
+            attention_prefill_kernel<D, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                     max_blocks, work, scale, window, n_head, n_kv_head, \
+                                                                     hd, page_size, page_shift);                      \
+    } while (0)
     if (hd <= 32) LIYAB_GO(1);
     else if (hd <= 64) LIYAB_GO(2);
     else if (hd <= 96) LIYAB_GO(3);

@@ -71,7 +71,7 @@ class _Staging:
         ev.record()
 
 
-ATTN_TILE = 128  # queries of one request that the prefill attention kernel takes together
+ATTN_TILE = 128  # queries of one request that the prefill attention kernel takes together (64 or 128)
 DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
 
 
@@ -303,7 +303,7 @@ class StepFunction:
             groups=[GroupStep(block_tables=dview(f"bt{g}").view(S, W), slots=dview(f"slots{g}")) for g in range(G)],
             host=StepHost(q_lens=q_lens, starts=[int(s) for s in starts[:-1]], first_pos=first,
                           max_q_len=max(q_lens), max_context=max_context,
-                          attention_mode=mode, context_bucket=_bucket(max_context), n_attn_tiles=n_tiles,
+                          attention_mode=mode, context_bucket=_bucket(max_context), n_attn_tiles=n_tiles, attn_tile=ATTN_TILE,
                           n_attn_single=len(singles)),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
             logit_slots=dview("logit_slots"), last_tokens=self.last_tokens,

@@ -76,7 +76,8 @@ class StepHost:
     max_context: int  # longest context after this step
     attention_mode: str = "prefill"  # "decode": every request brings few tokens, each taken on its own
     context_bucket: int = 256  # max_context rounded up to a power of two: grids follow it, not the exact length
-    n_attn_tiles: int = 0  # prefill mode: tiles of up to 128 queries of the long portions
+    n_attn_tiles: int = 0  # prefill mode: tiles of up to attn_tile queries of the long portions
+    attn_tile: int = 128
     n_attn_single: int = 0  # prefill mode: tokens of short portions, attended one by one
 
 

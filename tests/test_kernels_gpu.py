@@ -257,13 +257,14 @@ def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=No
         lens = {}
         for sidx in case["tok_seq"]:
             lens[sidx] = lens.get(sidx, 0) + 1
+        tile = splits if splits in (64, 128) else 128
         for sidx, nq in sorted(lens.items()):
             p0 = case["tok_pos"][row]
-            for t0 in range(0, nq, 128):
-                work.extend((sidx, row + t0, p0 + t0, min(128, nq - t0)))
+            for t0 in range(0, nq, tile):
+                work.extend((sidx, row + t0, p0 + t0, min(tile, nq - t0)))
             row += nq
         wk = torch.tensor(work, dtype=torch.int32, device=DEV)
-        ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window)
+        ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window, tile=tile)
     elif kernel == "decode":
         partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
         tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
@@ -325,13 +326,14 @@ PREFILL_CASES = [
 ]
 
 
+@pytest.mark.parametrize("tile", [64, 128])
 @pytest.mark.parametrize("window", [0, 37, 200])
 @pytest.mark.parametrize("case_id", range(len(PREFILL_CASES)))
-def test_attention_prefill(ops, case_id, window):
+def test_attention_prefill(ops, case_id, window, tile):
     ctx_lens, q_lens, H, Hkv, hd, page = PREFILL_CASES[case_id]
     case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
     scale = 0.7 / math.sqrt(hd)
-    out = run_attention(ops, case, H, hd, scale, window, "prefill")
+    out = run_attention(ops, case, H, hd, scale, window, "prefill", splits=tile)
     assert torch.isfinite(out.float()).all()
     close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, "prefill")
 
