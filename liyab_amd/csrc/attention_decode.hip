@@ -19,6 +19,8 @@ namespace liyab {
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
+constexpr int AD_MAX_BLOCKS = 2048;  // page ids of a request kept in LDS
+
 
 __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
 #pragma unroll
@@ -50,7 +52,8 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
                         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
-                        int n_head, int n_kv_head, int hd, int page_size, int n_splits, float* __restrict__ partials) {
+                        int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
+                        int n_splits, float* __restrict__ partials) {
     constexpr int KPP = 64 / LPK;  // keys per wave and pass
     __shared__ float lds[AD_WAVES][LPK][10];
     const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
@@ -58,27 +61,35 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int c = lane % LPK, kg = lane / LPK;
     const bool active = c * 8 < hd;
+    // The request's page ids go to LDS first, so that fetching a key is one load deep; they are
+    // loaded together with the position and the query (when every row is its own request the
+    // block-table row is known without looking the request up).
+    __shared__ int sbt[AD_MAX_BLOCKS];
+    const int seq = rows_are_requests ? t : tok_seq[t];
+    const int* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
+    for (int i = tid; i < max_blocks; i += 64 * AD_WAVES) sbt[i] = bt[i];
     const int pos = tok_pos[t];
-    const int* bt = block_tables + static_cast<int64_t>(tok_seq[t]) * max_blocks;
     const int hkv = h / (n_head / n_kv_head);
+    // lanes past the head dimension read column 0 and multiply it by a zero query
+    const int col = active ? c * 8 : 0;
+    float qf[8];
+    {
+        u32x4 qv = *reinterpret_cast<const u32x4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * hd + col);
+        if (!active) qv = u32x4{0, 0, 0, 0};
+        unpack8(qv, qf);
+    }
+    __syncthreads();
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
     const int n_keys = pos - first + 1;
     const int k_begin = first + static_cast<int>(static_cast<int64_t>(n_keys) * z / n_splits);
     const int k_end = first + static_cast<int>(static_cast<int64_t>(n_keys) * (z + 1) / n_splits);
-
-    float qf[8];
-    {
-        u32x4 qv = {0, 0, 0, 0};
-        if (active) qv = *reinterpret_cast<const u32x4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * hd + c * 8);
-        unpack8(qv, qf);
-    }
     Partial st;
     st.m = -INFINITY;
     st.l = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) st.acc[e] = 0.0f;
 
-    const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd + c * 8;
+    const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd + col;
     const int64_t page_stride = static_cast<int64_t>(n_kv_head) * page_size * hd;
     for (int j0 = k_begin + wave * KPP; j0 < k_end; j0 += AD_WAVES * KPP * AD_U) {
         u32x4 kv[AD_U], vv[AD_U];
@@ -88,14 +99,12 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
             const int j = j0 + u * AD_WAVES * KPP + kg;
             valid[u] = j < k_end;
             const int jc = valid[u] ? j : pos;  // a mapped position; its values are not used
-            const int64_t at = static_cast<int64_t>(bt[jc / page_size]) * page_stride + head_off +
-                               static_cast<int64_t>(jc % page_size) * hd;
-            kv[u] = u32x4{0, 0, 0, 0};
-            vv[u] = u32x4{0, 0, 0, 0};
-            if (active) {
-                kv[u] = *reinterpret_cast<const u32x4*>(kc + at);
-                vv[u] = *reinterpret_cast<const u32x4*>(vc + at);
-            }
+            // no branch around the loads: a load under a branch is waited for where the branch ends
+            const int lp = page_shift >= 0 ? jc >> page_shift : jc / page_size;
+            const int off = page_shift >= 0 ? jc & (page_size - 1) : jc % page_size;
+            const int64_t at = static_cast<int64_t>(sbt[lp]) * page_stride + head_off + static_cast<int64_t>(off) * hd;
+            kv[u] = *reinterpret_cast<const u32x4*>(kc + at);
+            vv[u] = *reinterpret_cast<const u32x4*>(vc + at);
         }
         float s[AD_U];
         float m_new = st.m;
@@ -195,7 +204,7 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
                                       const void* vc, const int* block_tables, int max_blocks, const int* tok_list,
                                       const int* tok_seq, const int* tok_pos, int n, float scale, int window,
                                       int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
-                                      float* partials, hipStream_t stream) {
+                                      int rows_are_requests, float* partials, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
     LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
     LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
@@ -207,8 +216,13 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
                   "attention_decode: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
     LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
+    LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
+    LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
     LIYAB_REQUIRE(waves == 4 || waves == 16, "attention_decode: %d waves per workgroup is not 4 or 16", waves);
     if (n == 0) return 0;
+    int page_shift = -1;
+    for (int b = 0; b < 31; ++b)
+        if ((1 << b) == page_size) page_shift = b;
     dim3 grid(n, n_head, n_splits);
     auto* o = static_cast<bf16_t*>(out);
     auto* pq = static_cast<const bf16_t*>(q);
@@ -219,11 +233,11 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
         if (waves == 4)                                                                                              \
             attention_decode_kernel<L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, n_splits, partials); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
         else                                                                                                         \
             attention_decode_kernel<L, 16, 8><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
-                                                                      window, n_head, n_kv_head, hd, page_size, n_splits, partials); \
+                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
     } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);

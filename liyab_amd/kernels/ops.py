@@ -420,9 +420,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
-                     tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4) -> None:
+                     tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
+                     rows_are_requests: bool = False) -> None:
     """Each token on its own over its request's bfloat16 cache, its keys cut into `n_splits`.
-    With `tok_list` (int32) only those rows are computed."""
+    With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
+    request t (every request brings one token), which saves the kernel a lookup."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
     _, hkv, page, hd = k_cache.shape
@@ -448,7 +450,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
-              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, _ptr(partials), _stream())
+              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, 1 if rows_are_requests else 0,
+              _ptr(partials), _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -506,9 +509,10 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
             partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 2),), torch.float32)
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
                          scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
-                         tok_list=tok_list, n_tokens=n if tok_list is not None else None)
+                         tok_list=tok_list, n_tokens=n if tok_list is not None else None,
+                         rows_are_requests=tok_list is None and host.max_q_len == 1)
 
-    if fast and host.attention_mode == "decode":
+    if fast and host.attention_mode == "decode" and block_tables.shape[1] <= 2048:
         decode(None, out.shape[0])
         return
     if fast and prefill_takes(hd) and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
