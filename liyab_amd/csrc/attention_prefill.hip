@@ -3,9 +3,13 @@
 // src/core/transformer.cpp:2303-2358, blocked as in flash attention: the
 // reference's own remark on flash decoding is at :2146-2153).
 //
-// A work item is (tile of up to 128 consecutive queries of one request, head);
-// each of 4 waves owns 32 queries. Keys are visited in blocks of 32, staged in
-// LDS with their values. Scores are computed transposed, S^T = K Q^T with
+// A work item is (tile of up to 128 consecutive queries of one request, head).
+// A workgroup has QG x KS waves: wave (qg, ks) owns the 32 queries of group qg
+// and, of every KS consecutive blocks of 32 keys, block ks; the KS partial
+// results of a query group are merged at the end in a fixed order. With few
+// tiles in flight KS > 1 puts more waves on the longest tile, whose walk over
+// the keys is the kernel's critical path. Keys are staged in LDS with their
+// values, KS blocks a step. Scores are computed transposed, S^T = K Q^T with
 // v_mfma_f32_32x32x16_bf16 (contraction over the head dimension, both operands
 // contiguous along it), so that a lane holds 16 scores of ONE query: the
 // running maximum and sum of a query need one exchange with the lane 32 apart
@@ -34,31 +38,39 @@ constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
 constexpr int AP_DEPTH = 6;     // blocks of keys and values in flight in registers
 constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LDS
 
-template <int DB, int WAVES>  // head dimension padded to 32 * DB; 32 * WAVES queries a tile
-__global__ void __launch_bounds__(64 * WAVES)
+template <int DB, int QG, int KS>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS blocks of keys a step
+__global__ void __launch_bounds__(64 * QG * KS)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
                          int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift) {
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
-    __shared__ __attribute__((aligned(16))) bf16_t Kb[2][AP_KEYS * LDK];  // two stages: the next block's keys
-    __shared__ __attribute__((aligned(16))) bf16_t Vb[2][AP_KEYS * LDK];  // and values load while this one is used
-    __shared__ __attribute__((aligned(16))) bf16_t Os[WAVES][32 * LDK];
-    constexpr int THREADS = 64 * WAVES;
+    constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
+    constexpr int STEP_KEYS = AP_KEYS * KS;  // keys staged a step
+    constexpr int STAGE = STEP_KEYS * LDK;
+    // two stages of keys and of values (the next step's load while this one is used); after the
+    // walk the same memory carries the partial results of the waves with ks > 0
+    constexpr int PARTIAL = DB * 16 * 64 + 2 * 64;  // floats a wave: outputs, then maximum and sum
+    constexpr int KV_BYTES = 4 * STAGE * 2, MERGE_BYTES = (KS - 1) * QG * PARTIAL * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char kv_raw[KV_BYTES > MERGE_BYTES ? KV_BYTES : MERGE_BYTES];
+    bf16_t* const Kb = reinterpret_cast<bf16_t*>(kv_raw);  // [2][STAGE]
+    bf16_t* const Vb = Kb + 2 * STAGE;                     // [2][STAGE]
+    __shared__ __attribute__((aligned(16))) bf16_t Os[QG][32 * LDK];
 
     const int* wk = work + 4 * blockIdx.x;
     const int seq = wk[0], row0 = wk[1], pos0 = wk[2], nq = wk[3];
     const int h = blockIdx.y;
     const int hkv = h / (n_head / n_kv_head);
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int qg = wave % QG, ks = wave / QG;
     const int ql = lane % 32, g2 = lane / 32;
     const int* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
 
-    const int my_q = 32 * wave + ql;
+    const int my_q = 32 * qg + ql;
     const int qpos = pos0 + min(my_q, nq - 1);  // lanes past the tile's end repeat its last query; never stored
-    const int wave_last = pos0 + min(32 * wave + 31, nq - 1);  // the wave's latest query position
-    const bool wave_has = 32 * wave < nq;
+    const int wave_last = pos0 + min(32 * qg + 31, nq - 1);  // the wave's latest query position
+    const bool wave_has = 32 * qg < nq;
     const int n_slabs = hd / 16;
     const float scale2 = scale * 1.4426950408889634f;  // log2(e): exp(x) = 2^(x log2 e)
 
@@ -86,7 +98,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     // a block's keys and values go global -> registers -> LDS (zeros past the head dimension,
     // before the window and past the last key). AP_DEPTH register sets form a ring: a block is
     // fetched AP_DEPTH - 1 blocks before it is multiplied, which covers the latency of the pages.
-    constexpr int PER = (AP_KEYS * CHUNKS + THREADS - 1) / THREADS;
+    constexpr int PER = (STEP_KEYS * CHUNKS + THREADS - 1) / THREADS;
     u32x4 rk[AP_DEPTH][PER], rv[AP_DEPTH][PER];
     // The request's page ids wait in LDS, so that a fetch is one load deep; and a fetch is
     // branch-free (a position outside the range reads a valid one and is zeroed when it is
@@ -98,7 +110,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     auto fetch = [&](int kb, u32x4 (&fk)[PER], u32x4 (&fv)[PER]) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int c = min(tid + THREADS * i, AP_KEYS * CHUNKS - 1), key = c / CHUNKS, col = min((c % CHUNKS) * 8, hd - 8);
+            const int c = min(tid + THREADS * i, STEP_KEYS * CHUNKS - 1), key = c / CHUNKS, col = min((c % CHUNKS) * 8, hd - 8);
             const int kp = min(max(kb + key, k_lo), k_hi);
             // page_shift >= 0: the page size is a power of two (no integer division)
             const int lp = page_shift >= 0 ? kp >> page_shift : kp / page_size;
@@ -113,47 +125,47 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             const int c = tid + THREADS * i, key = c / CHUNKS, col = (c % CHUNKS) * 8;
-            if (c < AP_KEYS * CHUNKS) {
+            if (c < STEP_KEYS * CHUNKS) {
                 const int kp = kb + key;
                 const bool ok = kp >= k_lo && kp <= k_hi && col < hd;
                 const u32x4 zero = {0, 0, 0, 0};
-                *reinterpret_cast<u32x4*>(&Kb[buf][key * LDK + col]) = ok ? fk[i] : zero;
-                *reinterpret_cast<u32x4*>(&Vb[buf][key * LDK + col]) = ok ? fv[i] : zero;
+                *reinterpret_cast<u32x4*>(&Kb[buf * STAGE + key * LDK + col]) = ok ? fk[i] : zero;
+                *reinterpret_cast<u32x4*>(&Vb[buf * STAGE + key * LDK + col]) = ok ? fv[i] : zero;
             }
         }
     };
     const int kb0 = (k_lo / AP_KEYS) * AP_KEYS;
 #pragma unroll
-    for (int d = 0; d < AP_DEPTH; ++d) fetch(kb0 + d * AP_KEYS, rk[d], rv[d]);
+    for (int d = 0; d < AP_DEPTH; ++d) fetch(kb0 + d * STEP_KEYS, rk[d], rv[d]);
     stash(0, kb0, rk[0], rv[0]);
     __syncthreads();
     int cur = 0;
-    for (int kbase = kb0; kbase <= k_hi; kbase += AP_DEPTH * AP_KEYS) {
+    for (int kbase = kb0; kbase <= k_hi; kbase += AP_DEPTH * STEP_KEYS) {
 #pragma unroll
       for (int ring = 0; ring < AP_DEPTH; ++ring) {
-        const int kb = kbase + ring * AP_KEYS;
-        if (kb > k_hi) break;
-        const bool more = kb + AP_KEYS <= k_hi;
-        fetch(kb + AP_DEPTH * AP_KEYS, rk[ring], rv[ring]);  // this set's block is in LDS already
-        const bf16_t* Ks = Kb[cur];
-        const bf16_t* Vs = Vb[cur];
+        const int kb_step = kbase + ring * STEP_KEYS;
+        if (kb_step > k_hi) break;
+        const bool more = kb_step + STEP_KEYS <= k_hi;
+        fetch(kb_step + AP_DEPTH * STEP_KEYS, rk[ring], rv[ring]);  // this set's keys are in LDS already
+        const int kb = kb_step + ks * AP_KEYS;  // this wave's block of the step
+        const bf16_t* Ks = Kb + cur * STAGE + ks * AP_KEYS * LDK;
+        const bf16_t* Vs = Vb + cur * STAGE + ks * AP_KEYS * LDK;
         if (wave_has && kb <= wave_last) {
             // S^T[key][query] = sum_d K[key][d] Q[query][d]
             floatx16 st;
 #pragma unroll
             for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+            // every slab of the padded head dimension, without a branch (queries and staged keys
+            // are zero past the head dimension): the reads of LDS go out together, ahead of the products
+            QFrag kf[2 * DB];
 #pragma unroll
-            for (int s = 0; s < 2 * DB; ++s) {
-                if (s < n_slabs) {
-                    QFrag kf;
-                    kf.u = *reinterpret_cast<const u32x4*>(Ks + ql * LDK + 16 * s + 8 * g2);
-                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[s].v, st, 0, 0, 0);
-                }
-            }
+            for (int s = 0; s < 2 * DB; ++s) kf[s].u = *reinterpret_cast<const u32x4*>(Ks + ql * LDK + 16 * s + 8 * g2);
+#pragma unroll
+            for (int s = 0; s < 2 * DB; ++s) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s].v, qf[s].v, st, 0, 0, 0);
             // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4. Scores are kept in the
             // base-2 domain (scale carries log2 e), so that exponentials are bare v_exp_f32.
             // A block every query of the wave sees whole needs no mask.
-            const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * wave && (window <= 0 || kb > wave_last - window);
+            const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * qg && (window <= 0 || kb > wave_last - window);
             float bm = -INFINITY;
             if (whole) {
 #pragma unroll
@@ -211,29 +223,61 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 }
             }
         }
-        if (more) stash(cur ^ 1, kb + AP_KEYS, rk[(ring + 1) % AP_DEPTH], rv[(ring + 1) % AP_DEPTH]);  // block kb + 32, fetched long ago
+        if (more) stash(cur ^ 1, kb_step + STEP_KEYS, rk[(ring + 1) % AP_DEPTH], rv[(ring + 1) % AP_DEPTH]);  // the next step's keys, fetched long ago
         lds_barrier();  // the blocks still in flight stay in flight
         cur ^= 1;
       }
     }
+    if constexpr (KS > 1) {
+        // the query group's partial results, merged into wave (qg, 0) in the order of ks (the
+        // walk's last barrier has passed: nobody reads keys or values any more)
+        float* part = reinterpret_cast<float*>(kv_raw);
+        if (ks > 0 && wave_has) {
+            float* mine = part + ((ks - 1) * QG + qg) * PARTIAL;
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mine[(d * 16 + r) * 64 + lane] = o[d][r];
+            mine[DB * 16 * 64 + lane] = m_run;
+            mine[DB * 16 * 64 + 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (ks == 0 && wave_has) {
+#pragma unroll
+            for (int k2 = 1; k2 < KS; ++k2) {
+                const float* other = part + ((k2 - 1) * QG + qg) * PARTIAL;
+                const float mo = other[DB * 16 * 64 + lane], lo = other[DB * 16 * 64 + 64 + lane];
+                const float M = fmaxf(m_run, mo);
+                const float wa = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
+                const float wb = mo == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mo - M);
+                l_run = wa * l_run + wb * lo;
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[d][r] = wa * o[d][r] + wb * other[(d * 16 + r) * 64 + lane];
+                m_run = M;
+            }
+        }
+    }
     // o[d][r] = O^T[dim = 32 d + 8 (r / 4) + 4 g2 + r % 4][query ql]: through LDS to rows of 16-byte pieces
-    if (wave_has) {
+    const bool writes = wave_has && ks == 0;
+    if (writes) {
         const float inv = 1.0f / l_run;
 #pragma unroll
         for (int d = 0; d < DB; ++d)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                Os[wave][ql * LDK + 32 * d + 8 * (r / 4) + 4 * g2 + r % 4] = float_to_bf16(o[d][r] * inv);
+                Os[qg][ql * LDK + 32 * d + 8 * (r / 4) + 4 * g2 + r % 4] = float_to_bf16(o[d][r] * inv);
     }
     __syncthreads();
-    if (wave_has) {
+    if (writes) {
         const int chunks_row = hd / 8;
         for (int c = lane; c < 32 * chunks_row; c += 64) {
             const int qq = c / chunks_row, col = (c % chunks_row) * 8;
-            if (32 * wave + qq < nq) {
-                *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row0 + 32 * wave + qq) * out_stride +
+            if (32 * qg + qq < nq) {
+                *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row0 + 32 * qg + qq) * out_stride +
                                           static_cast<int64_t>(h) * hd + col) =
-                    *reinterpret_cast<const u32x4*>(&Os[wave][qq * LDK + col]);
+                    *reinterpret_cast<const u32x4*>(&Os[qg][qq * LDK + col]);
             }
         }
     }
@@ -244,10 +288,10 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
 using namespace liyab;
 
 // work: n_tiles x (request index, first row, first position, queries <= tile), int32; tile = 64 or 128
-// queries (2 or 4 waves a workgroup).
+// queries (2 or 4 groups of 32); ksplit = 1, 2 or 4 waves share a query group's keys (128-query tiles: 1 or 2).
 extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                        const void* vc, const int* block_tables, int max_blocks, const int* work,
-                                       int n_tiles, int tile, float scale, int window, int n_head, int n_kv_head, int hd,
+                                       int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
                                        int page_size, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
     LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -261,6 +305,8 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
                   "attention_prefill: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(window >= 0, "attention_prefill: negative window");
     LIYAB_REQUIRE(tile == 64 || tile == 128, "attention_prefill: tiles of %d queries; 64 or 128 are taken", tile);
+    LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || (ksplit == 4 && tile == 64), "attention_prefill: %d waves a query group do not go with tiles of %d", ksplit, tile);
+    LIYAB_REQUIRE(ksplit < 4 || hd <= 64, "attention_prefill: 4 waves a query group are taken up to head size 64, not %d", hd);
     LIYAB_REQUIRE(max_blocks <= AP_MAX_BLOCKS, "attention_prefill: block tables of %d pages; at most %d are taken", max_blocks, AP_MAX_BLOCKS);
     if (n_tiles == 0) return 0;
     int page_shift = -1;
@@ -271,21 +317,30 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     auto* pq = static_cast<const bf16_t*>(q);
     auto* pk = static_cast<const bf16_t*>(kc);
     auto* pv = static_cast<const bf16_t*>(vc);
-#define LIYAB_GO(D)                                                                                                  \
-    do {                                                                                                             \
-        if (tile == 64)                                                                                              \
-            attention_prefill_kernel<D, 2><<<grid, 128, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
-                                                                     max_blocks, work, scale, window, n_head, n_kv_head, \
-                                                                     hd, page_size, page_shift);                      \
-        else                                                                                                         \
-            attention_prefill_kernel<D, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
-                                                                     max_blocks, work, scale, window, n_head, n_kv_head, \
-                                                                     hd, page_size, page_shift);                      \
+#define LIYAB_RUN(D, Q, S)                                                                                          \
+    attention_prefill_kernel<D, Q, S><<<grid, 64 * Q * S, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                       max_blocks, work, scale, window, n_head, n_kv_head, \
+                                                                       hd, page_size, page_shift)
+#define LIYAB_RUN4(D) LIYAB_RUN(D, 2, 4)
+#define LIYAB_SKIP4(D) (void)0  // four stages of 128 keys do not fit LDS at these head sizes (refused above)
+#define LIYAB_GO(D, FOUR)                           \
+    do {                                            \
+        if (tile == 64) {                           \
+            if (ksplit == 1) LIYAB_RUN(D, 2, 1);    \
+            else if (ksplit == 2) LIYAB_RUN(D, 2, 2); \
+            else FOUR(D);                           \
+        } else {                                    \
+            if (ksplit == 1) LIYAB_RUN(D, 4, 1);    \
+            else LIYAB_RUN(D, 4, 2);                \
+        }                                           \
     } while (0)
-    if (hd <= 32) LIYAB_GO(1);
-    else if (hd <= 64) LIYAB_GO(2);
-    else if (hd <= 96) LIYAB_GO(3);
-    else LIYAB_GO(4);
+    if (hd <= 32) LIYAB_GO(1, LIYAB_RUN4);
+    else if (hd <= 64) LIYAB_GO(2, LIYAB_RUN4);
+    else if (hd <= 96) LIYAB_GO(3, LIYAB_SKIP4);
+    else LIYAB_GO(4, LIYAB_SKIP4);
 #undef LIYAB_GO
+#undef LIYAB_RUN4
+#undef LIYAB_SKIP4
+#undef LIYAB_RUN
     return check_launch("attention_prefill");
 }

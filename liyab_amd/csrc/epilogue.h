@@ -53,7 +53,7 @@ __device__ __forceinline__ void epilogue_store(const EpiParams& p, int m, int n,
 template <typename OutT, int MODE>
 __device__ __forceinline__ void epilogue_store_biased(const EpiParams& p, int m, int n, float v) {
     switch (MODE >= 0 ? MODE : p.mode) {
-        case kEpiGeluTanh: v = gelu_tanh(v); break;
+        case kEpiGeluTanh: v = p.exact ? gelu_tanh(v) : gelu_tanh_fast(v); break;
         case kEpiGeluErf: v = p.exact ? gelu_erf_exact(v) : gelu_erf_fast(v); break;
         case kEpiResidual:
             p.residual[static_cast<int64_t>(m) * p.ldr + n] += v;

@@ -19,14 +19,28 @@ namespace liyab {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// Four consecutive outputs in one store (16 bytes of float32, 8 of bfloat16).
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* dst, const f32x4& v);
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, const f32x4& v) { *reinterpret_cast<f32x4*>(dst) = v; }
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const f32x4& v) {
+    uint2 packed;
+    packed.x = static_cast<uint32_t>(float_to_bf16(v[0])) | (static_cast<uint32_t>(float_to_bf16(v[1])) << 16);
+    packed.y = static_cast<uint32_t>(float_to_bf16(v[2])) | (static_cast<uint32_t>(float_to_bf16(v[3])) << 16);
+    *reinterpret_cast<uint2*>(dst) = packed;
+}
 
 constexpr int DBK = 64;      // k per stage
 
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
 __global__ void __launch_bounds__(256)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
-                    EpiParams epi) {
+                    EpiParams epi, int vec_ok, int page_shift) {
     constexpr int TM = BM / 64, TN = BN / 64;
     constexpr int STAGE = (BM + BN) * DBK;      // elements per stage: the tile of a, then the tile of w
     constexpr int A_LOADS = BM / 8 / 4, W_LOADS = BN / 8 / 4;  // wave-loads (8 rows each) per wave and stage
@@ -115,53 +129,82 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fw[ks & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0);
         }
     }
-    // tiles wholly inside the output skip the per-element bounds checks (a guarded store is a
-    // branch of its own: on an interior tile they cost as much as the whole product)
+    // The products were taken transposed (w's fragment as the first operand), so a lane holds one
+    // row of each 32 x 32 block, m = li, and of its columns the four groups 8q + 4g + {0..3}: what
+    // depends on the row (a token's place in the pages) is computed once, and every store is four
+    // consecutive columns wide. Tiles wholly inside the output take that path without bounds
+    // checks (a guarded store is a branch of its own: on an interior tile they cost as much as
+    // the whole product); edge tiles, and operands that are not aligned for it, go element by element.
     const bool inside = m0 + BM <= M && n0 + BN <= N;
-    if constexpr (EPI == kEpiQkvPaged) {
-        // keys and values go to their pages: the rows' page places first, then the stores
+    if (EPI >= 0 && inside && vec_ok) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * g;
-            int64_t row_base[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) row_base[r] = qkv_row_base(epi, min(mb + 8 * (r / 4) + r % 4, M - 1));
+            const int m = m0 + wm * (BM / 2) + i * 32 + li;
+            int64_t row_base = -1;
+            if constexpr (EPI == kEpiQkvPaged) {
+                const int slot = epi.slots[m];
+                const int page = page_shift >= 0 ? slot >> page_shift : slot / epi.page_size;
+                const int off = slot - page * epi.page_size;
+                row_base = slot < 0 ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int n = n0 + wn * (BN / 2) + j * 32 + li;
-                if (n >= N) continue;
-                const float bias_n = epilogue_bias(epi, n);
-                const int64_t col = qkv_col_offset(epi, n);
+                const int nb = n0 + wn * (BN / 2) + j * 32 + 4 * g;
+                // loads first, stores after: a load between two stores waits for the first of them
+                f32x4 b4[4], r4[4];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = mb + 8 * (r / 4) + r % 4;
-                    if (inside || m < M) qkv_store<OutT>(epi, m, n, row_base[r], col, acc[i][j][r] + bias_n);
+                for (int q = 0; q < 4; ++q) {
+                    b4[q] = epi.bias != nullptr ? *reinterpret_cast<const f32x4*>(epi.bias + nb + 8 * q) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    if constexpr (EPI == kEpiResidual)
+                        r4[q] = *reinterpret_cast<const f32x4*>(epi.residual + static_cast<int64_t>(m) * epi.ldr + nb + 8 * q);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int n = nb + 8 * q;
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e] + b4[q][e];
+                    if constexpr (EPI == kEpiResidual) {
+                        *reinterpret_cast<f32x4*>(epi.residual + static_cast<int64_t>(m) * epi.ldr + n) = v + r4[q];
+                    } else if constexpr (EPI == kEpiQkvPaged) {
+                        if (n < epi.q_dim) {
+                            store4<OutT>(static_cast<OutT*>(epi.out) + static_cast<int64_t>(m) * epi.ldo + n, v);
+                        } else if (row_base >= 0) {
+                            const bool is_v = n >= epi.q_dim + epi.kv_dim;
+                            const int c = n - epi.q_dim - (is_v ? epi.kv_dim : 0);
+                            const int head = c / epi.hd, dim = c - head * epi.hd;
+                            store4<OutT>(static_cast<OutT*>(is_v ? epi.vc : epi.kc) + row_base + static_cast<int64_t>(head) * epi.page_size * epi.hd + dim, v);
+                        }
+                    } else {
+                        if constexpr (EPI == kEpiGeluTanh) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = gelu_tanh_fast(v[e]);
+                        } else if constexpr (EPI == kEpiGeluErf) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = epi.exact ? gelu_erf_exact(v[e]) : gelu_erf_fast(v[e]);
+                        }
+                        store4<OutT>(static_cast<OutT*>(epi.out) + static_cast<int64_t>(m) * epi.ldo + n, v);
+                    }
                 }
             }
         }
         return;
     }
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wm * (BM / 2) + i * 32 + li;
+        if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + wn * (BN / 2) + j * 32 + li;
-            const int mb = m0 + wm * (BM / 2) + i * 32 + 4 * g;
-            const float bias_n = n < N ? epilogue_bias(epi, n) : 0.0f;
-            if (inside) {
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) epilogue_store_biased<OutT, EPI>(epi, mb + 8 * (r / 4) + r % 4, n, acc[i][j][r] + bias_n);
-            } else if (n < N) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = mb + 8 * (r / 4) + r % 4;
-                    if (m < M) epilogue_store_biased<OutT, EPI>(epi, m, n, acc[i][j][r] + bias_n);
-                }
+            for (int r = 0; r < 16; ++r) {
+                const int n = n0 + wn * (BN / 2) + j * 32 + 8 * (r / 4) + 4 * g + r % 4;
+                if (n < N) epilogue_store<OutT, EPI>(epi, m, n, acc[i][j][r]);
             }
-        }
+    }
 }
 
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
@@ -174,7 +217,20 @@ int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, in
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         ready = true;
     }
-    kern<<<grid, 256, smem, stream>>>(a, lda, w, M, N, K, epi);
+    // four-wide stores need aligned rows; the cache's slots fit 32 bits (checked by the launcher)
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    bool vec = N % 4 == 0 && (epi.bias == nullptr || al16(epi.bias));
+    int page_shift = -1;
+    if (EPI == kEpiResidual) {
+        vec = vec && al16(epi.residual) && epi.ldr % 4 == 0;
+    } else if (EPI == kEpiQkvPaged) {
+        vec = vec && al16(epi.out) && al16(epi.kc) && al16(epi.vc) && epi.ldo % 4 == 0 && epi.hd % 4 == 0 && epi.q_dim % 4 == 0;
+        for (int b = 0; b < 31; ++b)
+            if ((1 << b) == epi.page_size) page_shift = b;
+    } else {
+        vec = vec && al16(epi.out) && epi.ldo % 4 == 0;
+    }
+    kern<<<grid, 256, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, page_shift);
     return check_launch("gemm_mfma_dl");
 }
 
@@ -190,6 +246,7 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
     switch (epi.mode) {
         case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone>(pa, lda, pw, M, N, K, epi, stream);
         case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf>(pa, lda, pw, M, N, K, epi, stream);
         case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged>(pa, lda, pw, M, N, K, epi, stream);
         default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1>(pa, lda, pw, M, N, K, epi, stream);
     }

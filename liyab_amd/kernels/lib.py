@@ -49,8 +49,8 @@ _SIGNATURES = {
     "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_int, c_int, P, P],
     "liyab_gemm_skinny_ln": [P, P, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
-    "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_float, c_int, c_int, c_int,
-                                c_int, c_int, P],
+    "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
+                                c_int, c_int, c_int, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
     "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P, P, P],
 }

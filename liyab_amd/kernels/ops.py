@@ -456,9 +456,10 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, work: torch.Tensor, n_tiles: int, *, n_head: int, scale: float,
-                      window: int = 0, tile: int = 128) -> None:
+                      window: int = 0, tile: int = 128, ksplit: int = 1) -> None:
     """Tiles of up to `tile` (64 or 128) consecutive queries of one request over its bfloat16
-    cache, on the matrix cores. work: int32 [n_tiles, 4] = (request index, first row, first
+    cache, on the matrix cores; `ksplit` waves (1, 2, or 4 with tiles of 64) share the keys of
+    32 queries. work: int32 [n_tiles, 4] = (request index, first row, first
     position, queries); the caller has checked rows and positions against out and the block tables."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
@@ -475,7 +476,7 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
     _i32(work, "work", 4 * n_tiles)
     _lib.call("liyab_attention_prefill", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
-              block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), float(scale), int(window),
+              block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), int(ksplit), float(scale), int(window),
               n_head, hkv, hd, page, _stream())
 
 
@@ -518,8 +519,11 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
     if fast and prefill_takes(hd) and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
         # long portions in tiles on the matrix cores, the short ones token by token
         if host.n_attn_tiles:
+            # with fewer workgroups than compute units, two waves share each query group's keys:
+            # the longest tile's walk over its keys is then the kernel's critical path, and halves
+            ksplit = 2 if host.n_attn_tiles * n_head <= 256 else 1
             attention_prefill(out, q, k_cache, v_cache, block_tables, ctx.attn_work, host.n_attn_tiles, n_head=n_head,
-                              scale=scale, window=window, tile=host.attn_tile)
+                              scale=scale, window=window, tile=host.attn_tile, ksplit=ksplit)
         if host.n_attn_single:
             decode(ctx.attn_single_rows, host.n_attn_single)
         return

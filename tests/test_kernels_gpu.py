@@ -243,7 +243,7 @@ def attention_reference(case, H, Hkv, hd, scale, window=0):
     return out
 
 
-def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=None, waves=4):
+def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=None, waves=4, ksplit=1):
     dev = lambda x: x.to(DEV)  # noqa: E731
     q, kc, vc, bt = dev(case["q"]), dev(case["kc"]), dev(case["vc"]), dev(case["bt"])
     tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
@@ -264,7 +264,8 @@ def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=No
                 work.extend((sidx, row + t0, p0 + t0, min(tile, nq - t0)))
             row += nq
         wk = torch.tensor(work, dtype=torch.int32, device=DEV)
-        ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window, tile=tile)
+        ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window, tile=tile,
+                              ksplit=ksplit)
     elif kernel == "decode":
         partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
         tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
@@ -326,14 +327,16 @@ PREFILL_CASES = [
 ]
 
 
-@pytest.mark.parametrize("tile", [64, 128])
+@pytest.mark.parametrize("tile,ksplit", [(64, 1), (64, 2), (64, 4), (128, 1), (128, 2)])
 @pytest.mark.parametrize("window", [0, 37, 200])
 @pytest.mark.parametrize("case_id", range(len(PREFILL_CASES)))
-def test_attention_prefill(ops, case_id, window, tile):
+def test_attention_prefill(ops, case_id, window, tile, ksplit):
     ctx_lens, q_lens, H, Hkv, hd, page = PREFILL_CASES[case_id]
+    if ksplit == 4 and hd > 64:
+        pytest.skip("4 waves a query group are taken up to head size 64")
     case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
     scale = 0.7 / math.sqrt(hd)
-    out = run_attention(ops, case, H, hd, scale, window, "prefill", splits=tile)
+    out = run_attention(ops, case, H, hd, scale, window, "prefill", splits=tile, ksplit=ksplit)
     assert torch.isfinite(out.float()).all()
     close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, "prefill")
 
