@@ -49,7 +49,8 @@ def test_embed_and_add_rows(ops, dtype, n, d):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,d,eps", [(1, 64, 1e-5), (9, 96, 1e-6), (40, 1600, 1e-5), (3, 777, 1e-3)])
+@pytest.mark.parametrize("n,d,eps", [(1, 64, 1e-5), (9, 96, 1e-6), (40, 1600, 1e-5), (3, 777, 1e-3), (5, 768, 1e-5),
+                                     (70, 260, 1e-5), (6, 1028, 1e-6), (7, 2048, 1e-5), (2, 2052, 1e-5)])
 def test_layernorm(ops, out_dtype, n, d, eps):
     x = rnd(n + 3, d, scale=3.0) + 1.5
     w, b = rnd(d, seed=2) + 1.0, rnd(d, seed=3)
