@@ -56,6 +56,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int i = lane % 16, g = lane / 16;
     const int n0 = blockIdx.x * 16 * NT;
+    const int m0 = blockIdx.y * 16 * MT;  // this workgroup's rows: [m0, m0 + 16 MT) of M
     const int units = (K + 63) / 64;
     const u32x4 zero = {0, 0, 0, 0};
     const bf16_t* wrow[NT];
@@ -116,7 +117,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
         for (int s = 0; s < MT; ++s) arow[s] = xs + min(16 * s + i, M - 1) * ldx;
     } else {
 #pragma unroll
-        for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(16 * s + i, M - 1)) * lda;
+        for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(m0 + 16 * s + i, M - 1)) * lda;
     }
 
     floatx4 acc[MT][NT];
@@ -163,7 +164,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     __syncthreads();
     for (int e = tid; e < TILES * 256; e += blockDim.x) {
         const int tile = e / 256, s = tile / NT, t = tile % NT;
-        const int m = 16 * s + (e % 256) / 16, n = n0 + 16 * t + e % 16;
+        const int m = m0 + 16 * s + (e % 256) / 16, n = n0 + 16 * t + e % 16;
         float v = 0.0f;
         for (int q = 0; q < ksplit; ++q) v += red[q * TILES * 256 + e];
         if (m < M && n < N) epilogue_store<OutT>(epi, m, n, v);
@@ -173,7 +174,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
 template <bool LN, int MT, int NT, int MAXW, int MAXV = 32>
 int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, const EpiParams& epi,
                   const LnParams& ln, hipStream_t stream) {
-    const int grid = (N + 16 * NT - 1) / (16 * NT);
+    const dim3 grid((N + 16 * NT - 1) / (16 * NT), LN ? 1 : (M + 16 * MT - 1) / (16 * MT));
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
     if (ksplit > MAXW) ksplit = MAXW;
@@ -200,16 +201,22 @@ int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K
     return check_launch("gemm_skinny");
 }
 
-static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide,
+static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide, int mtile,
                            const EpiParams& epi, const LnParams& ln, hipStream_t stream) {
-    const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    // tiles of 16 rows a workgroup: all of M in one workgroup reads the weights once; with few
+    // output features that leaves most of the chip idle, and the rows are spread over workgroups
+    // instead (the weights then come from L2 after their first reading)
+    int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    if (mtile > 0) mt = mtile;
+    else if (mt > 1 && N <= 1024) mt = 1;
+    LIYAB_REQUIRE(mt == 1 || mt == 2 || mt == 4, "gemm_skinny: %d tiles of rows a workgroup is not 1, 2 or 4", mt);
     // wide tiles of N (64 features a workgroup) when N is so large that every workgroup
     // re-reading the tokens would cost more than the weights
     if (wide < 0) wide = (mt > 1 && static_cast<long>(N) * M > (1L << 20)) ? 1 : 0;
     const int nt = wide ? 4 : 1;
     if (ksplit == 0) {
         // enough waves to cover the chip several times over, each with at least 128 k
-        const int tiles = (N + 16 * nt - 1) / (16 * nt), units = (K + 63) / 64;
+        const int tiles = ((N + 16 * nt - 1) / (16 * nt)) * ((M + 16 * mt - 1) / (16 * mt)), units = (K + 63) / 64;
         ksplit = 1;
         while (ksplit < 16 && tiles * ksplit < 2048 && units / (ksplit * 2) >= (mt * nt == 1 ? 2 : 1)) ksplit *= 2;
         // a folded norm takes a wave per row: as many waves as rows, so the rows go side by side
@@ -237,9 +244,9 @@ using namespace liyab;
 
 // a [M <= 64, K] and w [N, K] are bfloat16. ksplit: waves per workgroup sharing K (0 = chosen
 // from the shape; 1, 2, 4, 8 or 16). wide: 64 instead of 16 output features a workgroup
-// (-1 = chosen from the shape).
+// (-1 = chosen from the shape). mtile: tiles of 16 rows a workgroup, 1, 2 or 4 (0 = chosen from the shape).
 extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide,
-                                 const EpiParams* epi_in, hipStream_t stream) {
+                                 int mtile, const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
     LIYAB_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d (at most 64) N=%d K=%d", M, N, K);
     LIYAB_REQUIRE(K % 8 == 0 && lda % 8 == 0 && lda >= K, "gemm_skinny: K %d and lda %lld must be multiples of 8", K,
@@ -249,7 +256,7 @@ extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int 
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
-    return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream);
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, mtile, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream);
 }
 
 // The same product with a LayerNorm folded in: the first operand is LayerNorm(x[rows[m] or m])
@@ -266,5 +273,5 @@ extern "C" int liyab_gemm_skinny_ln(const float* x, const float* ln_weight, cons
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
-    return skinny_dispatch(nullptr, K + 8, w, M, N, K, ksplit, 0, epi, LnParams{x, ln_weight, ln_bias, rows, eps}, stream);
+    return skinny_dispatch(nullptr, K + 8, w, M, N, K, ksplit, 0, 0, epi, LnParams{x, ln_weight, ln_bias, rows, eps}, stream);
 }

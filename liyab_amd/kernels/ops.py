@@ -328,8 +328,10 @@ def gemm_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *,
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
-                epilogue: int = EPI_NONE, kv=None, ksplit: int = 0, wide: int = -1) -> None:
-    """The weight-streaming product for at most 64 bfloat16 rows, K a multiple of 8."""
+                epilogue: int = EPI_NONE, kv=None, ksplit: int = 0, wide: int = -1, mtile: int = 0) -> None:
+    """The weight-streaming product for at most 64 bfloat16 rows, K a multiple of 8. ksplit
+    (waves sharing K), wide (64 output features a workgroup) and mtile (tiles of 16 rows a
+    workgroup) are chosen from the shape unless given."""
     lda = _rows(a, "a")
     M, K = a.shape
     _dev(w, "w")
@@ -338,7 +340,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     if M > 64:
         raise KernelError(f"gemm_skinny: {M} rows; it takes at most 64")
     e = _epilogue(a, w, bias, out, residual, epilogue, kv)
-    _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, wide, ctypes.byref(e), _stream())
+    _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, wide, mtile, ctypes.byref(e), _stream())
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,

@@ -108,7 +108,7 @@ def test_gemm_float32(ops, M, N, K, epilogue):
         assert torch.equal(one[0], full[M // 2])
 
 
-@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w",
+@pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
                                     "dl1", "dl2", "dl3", "dl5", "dl6"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
@@ -127,7 +127,9 @@ def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
         if kernel.startswith("dl"):
             ops.gemm_mfma_dl(a, w, bias, tile=int(kernel[2:]), **kw)
         elif kernel.startswith("skinny"):
-            ops.gemm_skinny(a, w, bias, ksplit=int(kernel[6:].rstrip("w")), wide=1 if kernel.endswith("w") else 0, **kw)
+            spec, _, mtile = kernel[6:].partition("m")  # split of K, "w" for wide tiles of N, "m<tiles of rows>"
+            ops.gemm_skinny(a, w, bias, ksplit=int(spec.rstrip("w")), wide=1 if spec.endswith("w") else 0,
+                            mtile=int(mtile or 0), **kw)
         elif kernel == "simple":
             ops.gemm_simple(a, w, bias, **kw)
         elif kernel == "auto":
