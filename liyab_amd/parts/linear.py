@@ -3,9 +3,9 @@
 W is [out, in], a row per output feature, the layout the reference works in
 (include/liyab/types.h:165-184; y = x . W^T, include/liyab/backend.h:35).
 The kernel is chosen here by dtype and shape; callers only say what they
-want computed. The first operand may be a pending norm (`Normed`): when the
-kernel for this shape can apply the norm itself it does, otherwise the norm
-runs first as its own kernel.
+want computed. The first operand may be a pending norm (`Normed`): the norm
+runs first as its own kernel, unless FOLD_NORM asks for the product kernel
+that applies the norm itself where the shape allows it.
 """
 
 from __future__ import annotations
@@ -18,8 +18,15 @@ from ..kernels import ops
 from .norms import Normed
 
 
+# Folding the norm into a decode step's products saves a launch, but every workgroup of the
+# product then repeats the norm ahead of its multiplies. Measured at GPT-2 small's sizes the
+# standalone norm (a wave per row, 2.6 us) plus the plain product is faster: 464 against 506 us
+# a step at batch 1, 526 against 574 at batch 8. Off; the folded kernel stays available.
+FOLD_NORM = False
+
+
 def _fuses(a, w: torch.Tensor) -> bool:
-    return (isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and w.dtype == torch.bfloat16
+    return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and w.dtype == torch.bfloat16
             and a.x.dtype == torch.float32 and a.x.is_contiguous() and ops.skinny_ln_takes(a.n_rows, a.norm.width, w.shape[0]))
 
 

@@ -174,10 +174,13 @@ def test_norm_alone(parts):
     core.close("n")
 
 
-@pytest.mark.parametrize("lazy", [False, True])
-def test_feed_forward_alone(parts, lazy):
+@pytest.mark.parametrize("lazy", [False, True, "folded"])
+def test_feed_forward_alone(parts, lazy, monkeypatch):
     from liyab_amd.engine import StepItem
+    from liyab_amd.parts import linear
 
+    if lazy == "folded":  # the product kernel that applies a pending norm itself (off by default)
+        monkeypatch.setattr(linear, "FOLD_NORM", True)
     p, dtype = parts
     core = p.core
     core.open("f")
