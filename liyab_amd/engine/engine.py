@@ -155,7 +155,7 @@ class Engine:
         items = []
         for s in batch:
             r = s.request
-            toks = r.tokens[s.first:s.first + s.count]
+            toks = r.token_slice(s.first, s.count)
             items.append(StepItem(r.rid, toks, [s.count - 1] if s.wants_logits else [],
                                   pending_last=r.pending > 0 and s.first + s.count == r.n_tokens))
         logits = self.core.step(items)

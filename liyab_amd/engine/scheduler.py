@@ -57,6 +57,17 @@ class Request:
         knows its value, see StepItem.pending_last)."""
         return self.prompt + self.generated + [0] * self.pending
 
+    def token_slice(self, first: int, count: int) -> List[int]:
+        """tokens[first:first + count] without putting the whole list together (a decode step
+        asks for one token of a long request)."""
+        n_prompt, end = len(self.prompt), first + count
+        if end <= n_prompt:
+            return self.prompt[first:end]
+        out = self.prompt[first:] if first < n_prompt else []
+        out += self.generated[max(first - n_prompt, 0):end - n_prompt]
+        missing = count - len(out)
+        return out + [0] * min(missing, self.pending) if missing > 0 else out
+
     @property
     def n_tokens(self) -> int:
         return len(self.prompt) + len(self.generated) + self.pending
@@ -133,14 +144,25 @@ class Scheduler:
     def pressure(self) -> bool:
         """Whether the running requests' next portions may not all fit the free pages, so that
         schedule() may have to preempt; the engine then reads pending tokens first."""
-        need = [0] * len(self.manager.groups)
+        groups = self.manager.groups
+        free = min(g.pool.free_pages for g in groups)
+        page, chunk = self.manager.page_size, self.prefill_chunk
+        # a portion of c tokens takes at most ceil(c / page) + 1 new pages of a group
+        bound = 0
         for r in self.running:
-            count = min(r.remaining, self.prefill_chunk)
+            count = min(r.remaining, chunk)
+            if count > 0:
+                bound += -(-count // page) + 1
+        if bound <= free:
+            return False
+        need = [0] * len(groups)
+        for r in self.running:
+            count = min(r.remaining, chunk)
             if count <= 0:
                 continue
             for gi, n in enumerate(self.manager.pages_needed(r.rid, r.computed + count)):
                 need[gi] += n
-        return any(n > g.pool.free_pages for n, g in zip(need, self.manager.groups))
+        return any(n > g.pool.free_pages for n, g in zip(need, groups))
 
     # -- one step's decisions ---------------------------------------------------
     def _open(self, r: Request) -> None:
@@ -170,12 +192,12 @@ class Scheduler:
         def extra(r: Request, count: int) -> List[int]:
             return self.manager.pages_needed(r.rid, r.computed + count)
 
-        def fits(r: Request, count: int) -> bool:
-            return all(n + e <= g.pool.free_pages for n, e, g in zip(need, extra(r, count), groups))
+        def fits(r: Request, count: int, pages: Optional[List[int]] = None) -> bool:
+            return all(n + e <= g.pool.free_pages for n, e, g in zip(need, pages or extra(r, count), groups))
 
-        def take(r: Request, count: int) -> None:
+        def take(r: Request, count: int, pages: Optional[List[int]] = None) -> None:
             nonlocal budget
-            for gi, e in enumerate(extra(r, count)):
+            for gi, e in enumerate(pages or extra(r, count)):
                 need[gi] += e
             batch.append(Scheduled(r, r.computed, count, r.computed + count == r.n_tokens))
             budget -= count
@@ -194,6 +216,10 @@ class Scheduler:
             if r.state != RUNNING or budget <= 0:
                 continue
             count = min(r.remaining, self.prefill_chunk, budget)
+            pages = extra(r, count)  # counted once on the common path, where everything fits
+            if fits(r, count, pages):
+                take(r, count, pages)
+                continue
             while not fits(r, count):
                 victim = self.running[-1]
                 if victim is r:

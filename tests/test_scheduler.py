@@ -241,3 +241,20 @@ def test_a_request_at_its_last_token_is_not_scheduled_again():
     assert s2.draining(r2) and s2.schedule() == []  # nothing to run while its only token is pending
     s2.resolve(batch, {"b": 7})
     assert r2.generated == [7] and r2.finish_reason == "length"
+
+
+def test_token_slice_equals_a_slice_of_tokens():
+    import random
+
+    from liyab_amd.engine.scheduler import Request
+    from liyab_amd.sampling import SamplingParams
+
+    rng = random.Random(0)
+    for _ in range(500):
+        r = Request(rid=0, prompt=[rng.randrange(100) for _ in range(rng.randrange(1, 8))], params=SamplingParams())
+        r.generated = [rng.randrange(100) for _ in range(rng.randrange(0, 6))]
+        r.pending = rng.randrange(0, 3)
+        first = rng.randrange(0, r.n_tokens + 1)
+        count = rng.randrange(0, r.n_tokens - first + 1)
+        assert r.token_slice(first, count) == r.tokens[first:first + count]
+        assert len(r.prompt) + len(r.generated) + r.pending == r.n_tokens
