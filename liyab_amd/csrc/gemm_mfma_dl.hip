@@ -37,17 +37,19 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const f32x4& v) {
 
 constexpr int DBK = 64;      // k per stage
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
-__global__ void __launch_bounds__(256)
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
+__global__ void __launch_bounds__(64 * WM * WN)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
                     EpiParams epi, int vec_ok, int page_shift) {
-    constexpr int TM = BM / 64, TN = BN / 64;
+    // WM x WN waves, each with (BM / WM) x (BN / WN) of the tile in blocks of 32 x 32
+    constexpr int WAVES = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int STAGE = (BM + BN) * DBK;      // elements per stage: the tile of a, then the tile of w
-    constexpr int A_LOADS = BM / 8 / 4, W_LOADS = BN / 8 / 4;  // wave-loads (8 rows each) per wave and stage
+    constexpr int A_LOADS = BM / 8 / WAVES, W_LOADS = BN / 8 / WAVES;  // wave-loads (8 rows each) per wave and stage
+    static_assert(TM >= 1 && TN >= 1 && A_LOADS >= 1 && W_LOADS >= 1, "tile too small for its waves");
     extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int wm = wave / 2, wn = wave % 2;
+    const int wm = wave / WN, wn = wave % WN;
     // Workgroups go to the 8 XCDs round-robin, each XCD with an L2 of its own. Tile t of the
     // row-major tile order goes to the XCD that holds the tiles around it, so that an XCD's
     // tiles share a few row blocks of `a` and its L2 holds them beside all of `w`.
@@ -112,12 +114,12 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
             const int c = ks * 2 + g;  // the 16-byte piece of the row this lane needs
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const int row = wm * (BM / 2) + i * 32 + li;
+                const int row = wm * (BM / WM) + i * 32 + li;
                 fa[buf][i] = *reinterpret_cast<const bf16x8*>(sa + row * DBK + ((c ^ (row & 7)) * 8));
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int row = wn * (BN / 2) + j * 32 + li;
+                const int row = wn * (BN / WN) + j * 32 + li;
                 fw[buf][j] = *reinterpret_cast<const bf16x8*>(sw + row * DBK + ((c ^ (row & 7)) * 8));
             }
         };
@@ -142,7 +144,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     if (EPI >= 0 && inside && vec_ok) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int m = m0 + wm * (BM / 2) + i * 32 + li;
+            const int m = m0 + wm * (BM / WM) + i * 32 + li;
             int64_t row_base = -1;
             if constexpr (EPI == kEpiQkvPaged) {
                 const int slot = epi.slots[m];
@@ -152,7 +154,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int nb = n0 + wn * (BN / 2) + j * 32 + 4 * g;
+                const int nb = n0 + wn * (BN / WN) + j * 32 + 4 * g;
                 // loads first, stores after: a load between two stores waits for the first of them
                 f32x4 b4[4], r4[4];
 #pragma unroll
@@ -195,23 +197,23 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm * (BM / 2) + i * 32 + li;
+        const int m = m0 + wm * (BM / WM) + i * 32 + li;
         if (m >= M) continue;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int n = n0 + wn * (BN / 2) + j * 32 + 8 * (r / 4) + 4 * g + r % 4;
+                const int n = n0 + wn * (BN / WN) + j * 32 + 8 * (r / 4) + 4 * g + r % 4;
                 if (n < N) epilogue_store<OutT, EPI>(epi, m, n, acc[i][j][r]);
             }
     }
 }
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI>
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
 int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     const int grid = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
     const size_t smem = static_cast<size_t>(DSTAGES) * (BM + BN) * DBK * sizeof(bf16_t);
-    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI>;
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN>;
     static bool ready = false;  // once per instantiation, outside any stream capture's first use
     if (!ready) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
@@ -230,25 +232,25 @@ int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, in
     } else {
         vec = vec && al16(epi.out) && epi.ldo % 4 == 0;
     }
-    kern<<<grid, 256, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, page_shift);
+    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, page_shift);
     return check_launch("gemm_mfma_dl");
 }
 
-template <int BM, int BN, int DSTAGES>
+template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2>
 int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
-    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
     if (epi.out_dtype == kF32) {
-        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone>(pa, lda, pw, M, N, K, epi, stream);
-        return launch_dl_as<BM, BN, DSTAGES, float, -1>(pa, lda, pw, M, N, K, epi, stream);
+        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        return launch_dl_as<BM, BN, DSTAGES, float, -1, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
     }
     switch (epi.mode) {
-        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged>(pa, lda, pw, M, N, K, epi, stream);
-        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
     }
 }
 
@@ -256,8 +258,9 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
 
 using namespace liyab;
 
-// tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep; 6 = 64x64 with
-// four stages (0 = chosen from the shape).
+// tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep and four waves; 6 = 64x64
+// with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages, 9 = 128x64
+// (0 = chosen from the shape).
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
@@ -269,14 +272,18 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
     // measured on {256..2048} x {768, 2304, 3072} x {768, 3072}: 64 x 64 tiles, three workgroups a
-    // CU, win or tie everywhere; a long K likes one more stage in flight
-    if (tile == 0) tile = K >= 2048 ? 6 : 2;
+    // CU, win or tie nearly everywhere; a long K likes one more stage in flight; a large output
+    // (2,048 x 2,304 and up) likes 128 x 128 tiles on eight waves, two stages deep
+    if (tile == 0) tile = K >= 2048 ? 6 : (static_cast<long>(M) * N >= 2048L * 2048L ? 8 : 2);
     switch (tile) {
         case 1: return launch_dl<128, 128, 3>(a, lda, w, M, N, K, epi, stream);
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
         case 3: return launch_dl<128, 64, 3>(a, lda, w, M, N, K, epi, stream);
         case 5: return launch_dl<128, 192, 3>(a, lda, w, M, N, K, epi, stream);
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
+        case 7: return launch_dl<128, 128, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
+        case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
+        case 9: return launch_dl<128, 64, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }
