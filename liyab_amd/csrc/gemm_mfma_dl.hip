@@ -7,7 +7,7 @@
 // A wave's direct load fills 1 KiB of LDS contiguously, lane after lane: 8
 // rows of 64 k. Rows are therefore unpadded (128 bytes), and bank conflicts
 // of the 16-byte fragment reads are avoided by a swizzle: within a row, the
-// 16-byte piece c sits at position c ^ (row & 7), applied on the
+// 16-byte piece c sits at position c ^ swizzle(row), applied on the
 // global side when loading and again when reading. Rows past M or N are
 // clamped to the last valid row; their results are never stored. MFMA
 // operand layout and the fixed-order sum over k are those of gemm_mfma.hip.
@@ -36,6 +36,12 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const f32x4& v) {
 }
 
 constexpr int DBK = 64;      // k per stage
+
+// Where a row's 16-byte pieces sit within the row. LDS has 64 banks of 4 bytes: a 16-byte read
+// serves 16 lanes a cycle, which read 16 consecutive rows at one piece index. Rows are 128 bytes,
+// so even and odd rows start in different halves of the banks; within a half, 8 rows must land on
+// 8 different pieces: the piece index is XORed with (row / 2) % 8.
+__device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
 __global__ void __launch_bounds__(64 * WM * WN)
@@ -68,14 +74,14 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) {
             const int r0 = (wave * A_LOADS + i) * 8, row = r0 + lrow;
-            const int c = lpos ^ (row & 7);
+            const int c = lpos ^ swizzle(row);
             const bf16_t* src = a + static_cast<int64_t>(min(m0 + row, M - 1)) * lda + k0 + c * 8;
             __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sa + r0 * DBK), 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) {
             const int r0 = (wave * W_LOADS + i) * 8, row = r0 + lrow;
-            const int c = lpos ^ (row & 7);
+            const int c = lpos ^ swizzle(row);
             const bf16_t* src = w + static_cast<int64_t>(min(n0 + row, N - 1)) * K + k0 + c * 8;
             __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sw + r0 * DBK), 16, 0, 0);
         }
@@ -115,12 +121,12 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int row = wm * (BM / WM) + i * 32 + li;
-                fa[buf][i] = *reinterpret_cast<const bf16x8*>(sa + row * DBK + ((c ^ (row & 7)) * 8));
+                fa[buf][i] = *reinterpret_cast<const bf16x8*>(sa + row * DBK + ((c ^ swizzle(row)) * 8));
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const int row = wn * (BN / WN) + j * 32 + li;
-                fw[buf][j] = *reinterpret_cast<const bf16x8*>(sw + row * DBK + ((c ^ (row & 7)) * 8));
+                fw[buf][j] = *reinterpret_cast<const bf16x8*>(sw + row * DBK + ((c ^ swizzle(row)) * 8));
             }
         };
         read_frags(0, 0);
@@ -259,7 +265,8 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
 using namespace liyab;
 
 // tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep and four waves; 6 = 64x64
-// with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages, 9 = 128x64
+// with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages (deeper rings
+// measured slower: their LDS leaves one workgroup a compute unit, and 288 tiles then take two rounds), 9 = 128x64
 // (0 = chosen from the shape).
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
