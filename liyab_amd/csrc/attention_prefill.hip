@@ -15,7 +15,11 @@
 // running maximum and sum of a query need one exchange with the lane 32 apart
 // instead of a reduction over 32 lanes. The accumulators then serve, rounded to
 // bfloat16, directly as the second operand of O^T = V^T P^T (contraction over
-// the keys); only V has to be read across its rows, as 2-byte reads of LDS.
+// the keys); V is transposed once on its way into LDS (2-byte writes by the
+// staging threads), so that every wave reads its operand as 8-byte pieces.
+// Exponentials are taken against a reference value that follows the running
+// maximum from below by at most 2^8: the outputs are rescaled only when a
+// query's maximum jumps past that, which is rare, instead of at every block.
 // Maximum, exponentials, sums and outputs are 32-bit. A query's result depends
 // on its position and the block grid (multiples of 32 from the window's start),
 // not on the batch or the pages. Head sizes: multiples of 16 up to 128.
@@ -49,13 +53,16 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
     constexpr int STEP_KEYS = AP_KEYS * KS;  // keys staged a step
     constexpr int STAGE = STEP_KEYS * LDK;
+    // values are kept transposed, [dimension][key of the step], rows padded by 4 keys: the 8-byte
+    // reads of 32 lanes (32 dimensions, one group of 4 keys) then fall in 64 different banks
+    constexpr int LDV = STEP_KEYS + 4, VSTAGE = HDP * LDV;
     // two stages of keys and of values (the next step's load while this one is used); after the
     // walk the same memory carries the partial results of the waves with ks > 0
     constexpr int PARTIAL = DB * 16 * 64 + 2 * 64;  // floats a wave: outputs, then maximum and sum
-    constexpr int KV_BYTES = 4 * STAGE * 2, MERGE_BYTES = (KS - 1) * QG * PARTIAL * 4;
+    constexpr int KV_BYTES = 2 * (STAGE + VSTAGE) * 2, MERGE_BYTES = (KS - 1) * QG * PARTIAL * 4;
     __shared__ __attribute__((aligned(16))) unsigned char kv_raw[KV_BYTES > MERGE_BYTES ? KV_BYTES : MERGE_BYTES];
     bf16_t* const Kb = reinterpret_cast<bf16_t*>(kv_raw);  // [2][STAGE]
-    bf16_t* const Vb = Kb + 2 * STAGE;                     // [2][STAGE]
+    bf16_t* const Vb = Kb + 2 * STAGE;                     // [2][VSTAGE]
     __shared__ __attribute__((aligned(16))) bf16_t Os[QG][32 * LDK];
 
     const int* wk = work + 4 * blockIdx.x;
@@ -130,7 +137,10 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 const bool ok = kp >= k_lo && kp <= k_hi && col < hd;
                 const u32x4 zero = {0, 0, 0, 0};
                 *reinterpret_cast<u32x4*>(&Kb[buf * STAGE + key * LDK + col]) = ok ? fk[i] : zero;
-                *reinterpret_cast<u32x4*>(&Vb[buf * STAGE + key * LDK + col]) = ok ? fv[i] : zero;
+                QFrag vt;
+                vt.u = ok ? fv[i] : zero;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) Vb[buf * VSTAGE + (col + e) * LDV + key] = vt.h[e];
             }
         }
     };
@@ -149,7 +159,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
         fetch(kb_step + AP_DEPTH * STEP_KEYS, rk[ring], rv[ring]);  // this set's keys are in LDS already
         const int kb = kb_step + ks * AP_KEYS;  // this wave's block of the step
         const bf16_t* Ks = Kb + cur * STAGE + ks * AP_KEYS * LDK;
-        const bf16_t* Vs = Vb + cur * STAGE + ks * AP_KEYS * LDK;
+        const bf16_t* Vs = Vb + cur * VSTAGE + ks * AP_KEYS;
         if (wave_has && kb <= wave_last) {
             // S^T[key][query] = sum_d K[key][d] Q[query][d]
             floatx16 st;
@@ -162,46 +172,45 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
             for (int s = 0; s < 2 * DB; ++s) kf[s].u = *reinterpret_cast<const u32x4*>(Ks + ql * LDK + 16 * s + 8 * g2);
 #pragma unroll
             for (int s = 0; s < 2 * DB; ++s) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s].v, qf[s].v, st, 0, 0, 0);
-            // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4. Scores are kept in the
-            // base-2 domain (scale carries log2 e), so that exponentials are bare v_exp_f32.
-            // A block every query of the wave sees whole needs no mask.
+            // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4. A block every query of the
+            // wave sees whole needs no mask. The maximum is taken over the raw scores (the scale is
+            // positive); exponentials are 2^(score * scale2 - reference), one fused multiply-add and
+            // one v_exp_f32 a score.
             const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * qg && (window <= 0 || kb > wave_last - window);
             float bm = -INFINITY;
             if (whole) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    st[r] *= scale2;
-                    bm = fmaxf(bm, st[r]);
-                }
+                for (int r = 0; r < 16; ++r) bm = fmaxf(bm, st[r]);
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
                     const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
-                    st[r] = ok ? st[r] * scale2 : -INFINITY;
+                    st[r] = ok ? st[r] : -INFINITY;
                     bm = fmaxf(bm, st[r]);
                 }
             }
-            bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-            const float m_new = fmaxf(m_run, bm);
-            float corr = 1.0f, bs = 0.0f;
+            bm = fmaxf(bm, __shfl_xor(bm, 32, 64)) * scale2;
+            // the reference m_run is raised only when the block's maximum passes it by more than
+            // kLag: until then exponentials may reach 2^kLag, which 32-bit sums and bfloat16
+            // products hold as well as values below 1
+            constexpr float kLag = 8.0f;
+            float corr = 1.0f;
+            if (bm > m_run + kLag) {  // also the first block with a visible key (m_run = -inf)
+                corr = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - bm);
+                m_run = bm;
+            }
+            const float ref = m_run == -INFINITY ? 0.0f : m_run;  // nothing visible yet: every score is -inf, 2^-inf = 0
+            float bs = 0.0f;
             QFrag pf[2];
-            if (m_new == -INFINITY) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pf[0].h[e] = pf[1].h[e] = 0;
-            } else {
-                corr = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float p = __builtin_amdgcn_exp2f(st[r] - m_new);  // 2^-inf = 0 for masked keys
-                    bs += p;
-                    pf[r / 8].h[r % 8] = float_to_bf16(p);
-                }
+            for (int r = 0; r < 16; ++r) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(st[r], scale2, -ref));  // 0 for masked keys
+                bs += p;
+                pf[r / 8].h[r % 8] = float_to_bf16(p);
             }
             bs += __shfl_xor(bs, 32, 64);
             l_run = l_run * corr + bs;
-            m_run = m_new;
-            // the running outputs are rescaled only when some query's maximum moved
             const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.0f) != 0;
             // O^T[d][query] += sum_key V[key][d] P[key][query]; instruction s2 contracts the keys
             // of accumulator registers 8 s2 .. 8 s2 + 7: rows 16 s2 + 4 g2 + {0..3} and + 8
@@ -213,12 +222,11 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 }
 #pragma unroll
                 for (int s2 = 0; s2 < 2; ++s2) {
-                    QFrag vf;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int key = 16 * s2 + 8 * (e / 4) + 4 * g2 + e % 4;
-                        vf.h[e] = Vs[key * LDK + 32 * d + ql];
-                    }
+                    // this lane: dimension 32 d + ql, keys 16 s2 + 4 g2 + {0..3} and the same + 8
+                    union { uint2 u[2]; bf16x8 v; } vf;
+                    const bf16_t* vrow = Vs + (32 * d + ql) * LDV + 16 * s2 + 4 * g2;
+                    vf.u[0] = *reinterpret_cast<const uint2*>(vrow);
+                    vf.u[1] = *reinterpret_cast<const uint2*>(vrow + 8);
                     o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[s2].v, o[d], 0, 0, 0);
                 }
             }
@@ -304,6 +312,7 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
                   "attention_prefill: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(window >= 0, "attention_prefill: negative window");
+    LIYAB_REQUIRE(scale > 0.0f, "attention_prefill: the scale must be positive (the maximum is taken before scaling), not %g", scale);
     LIYAB_REQUIRE(tile == 64 || tile == 128, "attention_prefill: tiles of %d queries; 64 or 128 are taken", tile);
     LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || (ksplit == 4 && tile == 64), "attention_prefill: %d waves a query group do not go with tiles of %d", ksplit, tile);
     LIYAB_REQUIRE(ksplit < 4 || hd <= 64, "attention_prefill: 4 waves a query group are taken up to head size 64, not %d", hd);

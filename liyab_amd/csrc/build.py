@@ -34,6 +34,13 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# Matrix-instruction results in ordinary vector registers for kernels that work on them with
+# vector instructions between the products (softmax on the scores, rescaling of the outputs):
+# by default they land in accumulation registers and every such use costs a move each way.
+VGPR_MFMA = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+FILE_FLAGS = {
+    "attention_prefill.hip": VGPR_MFMA,
+}
 
 
 def sources() -> List[str]:
@@ -51,6 +58,7 @@ def source_hash() -> str:
         with open(p, "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -121,7 +129,8 @@ def build(quiet: bool = False, jobs: Optional[int] = None) -> str:
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
         t = time.time()
-        r = subprocess.run([hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj], env=env, capture_output=True, text=True)
+        extra = FILE_FLAGS.get(os.path.basename(src), [])
+        r = subprocess.run([hipcc, *FLAGS, *extra, "-I", CSRC, "-c", src, "-o", obj], env=env, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {os.path.basename(src)}:\n{r.stdout}\n{r.stderr}")
         _say(f"  {os.path.basename(src)} done in {time.time() - t:.0f} s", quiet)

@@ -518,7 +518,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
     if fast and host.attention_mode == "decode" and block_tables.shape[1] <= 2048:
         decode(None, out.shape[0])
         return
-    if fast and prefill_takes(hd) and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
+    if fast and prefill_takes(hd) and scale > 0 and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
         # long portions in tiles on the matrix cores, the short ones token by token
         if host.n_attn_tiles:
             # with fewer workgroups than compute units, two waves share each query group's keys:
