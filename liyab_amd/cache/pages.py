@@ -1,38 +1,42 @@
 """The cache manager: pages of keys and values, block tables, state slots.
 
-What the reference's KvCache does for one context (`include/liyab/kv_cache.h`,
-`src/core/kv_cache.cpp`): fixed pages of `page_size` positions mapped on
-demand (`reserve`, kv_cache.cpp:249-265), a table from logical page to pool
-page per layer group (kv_cache.h:358-365), groups of layers by what they keep
--- every position, or a window that gives older pages back as the context
-advances (kv_cache.h:10-23, kv_cache.cpp:474-487) -- and counters
-(kv_cache.h:347-352). Differences, all deliberate: one pool per group is
-shared by every live request (the reference gives each context a pool of its
-own, src/core/transformer.cpp:6529-6545), so pages a finished request gives
-back are used again by the next; pages are not zeroed when mapped, readers
-mask by position instead; a request that cannot get its pages changes
-nothing and the caller decides (`OutOfPages`), where the reference fails the
-pass (kv_cache.cpp:192-197).
+The bookkeeping itself is native (`csrc/host/cache_manager.{h,cpp}`, where the rules and
+their sources in the reference are written down); this module is its Python face: it maps
+the callers' request ids to the state slots the native side knows requests by, turns
+status codes into exceptions, and describes the groups of layers. One pool per group is
+shared by every live request, so pages a finished request gives back are used again by
+the next; a request that cannot get its pages changes nothing (`OutOfPages`).
 
-Beside the pages, each request holds one slot of fixed-size state for
-mixers that keep state instead of keys (the reference's `Context::states_`,
-src/core/transformer.h:853-865, 1296-1303); a model without such mixers
-has slots of zero bytes.
+Beside the pages, each request holds one slot of fixed-size state for mixers that keep
+state instead of keys (the reference's `Context::states_`, src/core/transformer.h:853-865,
+1296-1303); a model without such mixers has slots of zero bytes.
 
-This module is bookkeeping on the host only; the device memory the page ids
-and slots index lives in `CacheStorage`.
+This is bookkeeping on the host only; the device memory that page ids and slots index
+lives in `CacheStorage`.
 """
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+import ctypes
+from dataclasses import dataclass
+from typing import Dict, Hashable, List, Sequence, Tuple
 
 import numpy as np
 
-from ..errors import Busy, ContextFull, InvalidArgument, OutOfPages
+from .. import host
+from ..errors import InvalidArgument
 
 UNMAPPED = -1
+_I32P = ctypes.POINTER(ctypes.c_int32)
+_IP = ctypes.POINTER(ctypes.c_int)
+
+
+def _ints(values) -> np.ndarray:
+    return np.ascontiguousarray(values, dtype=np.intc)
+
+
+def _ip(a: np.ndarray):
+    return a.ctypes.data_as(_IP)
 
 
 @dataclass(frozen=True)
@@ -57,47 +61,63 @@ class StateSpec:
 
 
 class PagePool:
-    """Page ids 0..n-1 with a free stack; a page is held by at most one owner."""
+    """Page ids 0..n-1 with a free stack; a page is held by at most one owner. (A pool on its
+    own; a manager's pools are reached through `CacheManager.groups[i].pool`.)"""
 
     def __init__(self, num_pages: int):
         if num_pages <= 0:
             raise InvalidArgument("a page pool needs at least one page")
         self.num_pages = num_pages
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))  # pop() gives page 0 first
-        self._held = [False] * num_pages
-        self.peak_in_use = 0
+        self._lib = host.lib()
+        self._h = self._lib.liyab_pool_create(num_pages)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.liyab_pool_destroy(self._h)
+            self._h = None
 
     @property
     def free_pages(self) -> int:
-        return len(self._free)
+        return self._lib.liyab_pool_free_pages(self._h)
 
     @property
     def pages_in_use(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.free_pages
+
+    @property
+    def peak_in_use(self) -> int:
+        return self._lib.liyab_pool_peak(self._h)
 
     def allocate(self, n: int) -> List[int]:
-        if n > len(self._free):
-            raise OutOfPages(f"{n} pages wanted, {len(self._free)} free of {self.num_pages}")
-        out = [self._free.pop() for _ in range(n)]
-        for p in out:
-            assert not self._held[p], f"page {p} handed out twice"
-            self._held[p] = True
-        self.peak_in_use = max(self.peak_in_use, self.pages_in_use)
-        return out
+        out = np.empty(max(n, 1), dtype=np.int32)
+        host.check(self._lib.liyab_pool_allocate(self._h, n, out.ctypes.data_as(_I32P)))
+        return out[:n].tolist()
 
     def release(self, pages: Sequence[int]) -> None:
-        for p in pages:
-            if not (0 <= p < self.num_pages) or not self._held[p]:
-                raise AssertionError(f"page {p} freed but not held")
-            self._held[p] = False
-            self._free.append(p)  # most recently freed is used first
+        a = np.ascontiguousarray(pages, dtype=np.int32)
+        host.check(self._lib.liyab_pool_release(self._h, a.ctypes.data_as(_I32P), len(a)))
 
     def check(self) -> None:
-        """Invariants: every page is free or held, none both, none twice."""
-        assert len(set(self._free)) == len(self._free), "a page is on the free list twice"
-        for p in self._free:
-            assert not self._held[p], f"page {p} is free and held"
-        assert sum(self._held) + len(self._free) == self.num_pages, "a page was lost"
+        host.check(self._lib.liyab_pool_check(self._h))
+
+
+class _GroupPool:
+    """The counters of one of a manager's pools."""
+
+    def __init__(self, manager: "CacheManager", group: int, num_pages: int):
+        self._m, self._g, self.num_pages = manager, group, num_pages
+
+    @property
+    def free_pages(self) -> int:
+        return self._m._lib.liyab_cm_free_pages(self._m._h, self._g)
+
+    @property
+    def pages_in_use(self) -> int:
+        return self.num_pages - self.free_pages
+
+    @property
+    def peak_in_use(self) -> int:
+        return self._m._lib.liyab_cm_peak_in_use(self._m._h, self._g)
 
 
 @dataclass
@@ -107,16 +127,7 @@ class CacheGroup:
     index: int
     spec: KVSpec
     layers: List[int]
-    pool: PagePool
-
-
-@dataclass
-class _Request:
-    length: int = 0  # positions committed
-    reserved: int = 0  # positions whose pages are mapped (>= length)
-    tables: List[List[int]] = field(default_factory=list)  # per group: logical page -> pool page
-    first_kept: List[int] = field(default_factory=list)  # per group: first logical page still mapped
-    slot: int = UNMAPPED
+    pool: _GroupPool
 
 
 class CacheManager:
@@ -129,52 +140,69 @@ class CacheManager:
             raise InvalidArgument("page_size must be positive")
         if max_requests <= 0:
             raise InvalidArgument("max_requests must be positive")
+        if max_positions <= 0:
+            raise InvalidArgument("max_positions must be positive")
         self.page_size = page_size
         self.max_positions = max_positions
         self.max_requests = max_requests
         counts = [num_pages] * len(group_specs) if isinstance(num_pages, int) else list(num_pages)
         if len(counts) != len(group_specs):
             raise InvalidArgument("one page count per group is needed")
-        self.groups = [CacheGroup(i, spec, list(layers), PagePool(n))
+        if any(n <= 0 for n in counts):
+            raise InvalidArgument("a page pool needs at least one page")
+        if len(group_specs) > host.MAX_GROUPS:
+            raise InvalidArgument(f"{len(group_specs)} cache groups; at most {host.MAX_GROUPS} are taken")
+        self._lib = host.lib()
+        windows = _ints([spec.window for spec, _ in group_specs])
+        self._h = self._lib.liyab_cm_create(len(group_specs), _ip(windows), _ip(_ints(counts)), page_size, max_requests,
+                                            max_positions)
+        if not self._h:
+            raise InvalidArgument(self._lib.liyab_host_last_error().decode())
+        self.groups = [CacheGroup(i, spec, list(layers), _GroupPool(self, i, n))
                        for i, ((spec, layers), n) in enumerate(zip(group_specs, counts))]
         self.group_of_layer: Dict[int, int] = {l: g.index for g in self.groups for l in g.layers}
-        self._requests: Dict[Hashable, _Request] = {}
-        self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
-        self.max_blocks = max(1, -(-max_positions // page_size))
-        # the same tables as arrays, a row per state slot: the step function gathers a batch's rows at once
-        self._table_rows = [np.full((max_requests, self.max_blocks), UNMAPPED, dtype=np.int32) for _ in self.groups]
+        self.max_blocks = self._lib.liyab_cm_max_blocks(self._h)
+        self._slots: Dict[Hashable, int] = {}
+        # the native tables, a row per state slot (the memory never moves)
+        self._table_rows = [np.ctypeslib.as_array(self._lib.liyab_cm_table_rows(self._h, g),
+                                                  shape=(max_requests, self.max_blocks)) for g in range(len(self.groups))]
+        self._need = np.zeros(max(len(self.groups), 1), dtype=np.intc)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.liyab_cm_destroy(self._h)
+            self._h = None
+
+    @property
+    def handle(self):
+        """The native manager, for the native calls that take one (a step's metadata)."""
+        return self._h
 
     # -- requests -----------------------------------------------------------
     def open(self, rid: Hashable) -> int:
         """Registers a request and gives it a state slot; returns the slot."""
-        if rid in self._requests:
+        if rid in self._slots:
             raise InvalidArgument(f"request {rid!r} is already open")
-        if not self._free_slots:
-            raise Busy(f"all {self.max_requests} request slots are in use")
-        r = _Request(tables=[[] for _ in self.groups], first_kept=[0 for _ in self.groups],
-                     slot=self._free_slots.pop())
-        self._requests[rid] = r
-        return r.slot
+        slot = ctypes.c_int(-1)
+        host.check(self._lib.liyab_cm_open(self._h, ctypes.byref(slot)))
+        self._slots[rid] = slot.value
+        return slot.value
 
     def is_open(self, rid: Hashable) -> bool:
-        return rid in self._requests
+        return rid in self._slots
 
     def close(self, rid: Hashable) -> None:
         """Gives back everything the request holds."""
-        r = self._requests.pop(rid)
-        for g, table, rows in zip(self.groups, r.tables, self._table_rows):
-            g.pool.release([p for p in table if p != UNMAPPED])
-            rows[r.slot, :] = UNMAPPED
-        self._free_slots.append(r.slot)
+        host.check(self._lib.liyab_cm_close(self._h, self._slots.pop(rid)))
 
     def length(self, rid: Hashable) -> int:
-        return self._requests[rid].length
+        return self._lib.liyab_cm_length(self._h, self._slots[rid])
 
     def slot(self, rid: Hashable) -> int:
-        return self._requests[rid].slot
+        return self._slots[rid]
 
     def live_requests(self) -> List[Hashable]:
-        return list(self._requests)
+        return list(self._slots)
 
     # -- pages --------------------------------------------------------------
     def _pages_for(self, n_positions: int) -> int:
@@ -182,8 +210,8 @@ class CacheManager:
 
     def pages_needed(self, rid: Hashable, new_length: int) -> List[int]:
         """New pages per group that `reserve(rid, new_length)` would take."""
-        r = self._requests[rid]
-        return [max(0, self._pages_for(new_length) - len(t)) for t in r.tables]
+        self._lib.liyab_cm_pages_needed(self._h, self._slots[rid], new_length, _ip(self._need))
+        return self._need[:len(self.groups)].tolist()
 
     def can_reserve(self, wants: Sequence[Tuple[Hashable, int]], new_lengths: Sequence[int] = ()) -> bool:
         """Whether `reserve(wants)` would succeed, with requests that are not
@@ -198,76 +226,43 @@ class CacheManager:
         return all(n <= g.pool.free_pages for n, g in zip(need, self.groups))
 
     def free_slots(self) -> int:
-        return len(self._free_slots)
+        return self._lib.liyab_cm_free_slots(self._h)
 
     def reserve(self, wants: Sequence[Tuple[Hashable, int]]) -> None:
         """Maps pages so that each request can hold `new_length` positions.
         All or nothing: raises OutOfPages (or ContextFull) before anything
         changed."""
-        need = [0] * len(self.groups)
-        for rid, new_length in wants:
-            r = self._requests[rid]
-            if new_length > self.max_positions:
-                raise ContextFull(f"request {rid!r} would reach {new_length} positions; the context holds {self.max_positions}")
-            if new_length < r.length:
-                raise InvalidArgument("reserve cannot shrink a request; use truncate")
-            for gi, n in enumerate(self.pages_needed(rid, new_length)):
-                need[gi] += n
-        for n, g in zip(need, self.groups):
-            if n > g.pool.free_pages:
-                raise OutOfPages(f"group {g.index}: {n} pages wanted, {g.pool.free_pages} free of {g.pool.num_pages}")
-        for rid, new_length in wants:
-            r = self._requests[rid]
-            for g, table, rows in zip(self.groups, r.tables, self._table_rows):
-                new = g.pool.allocate(max(0, self._pages_for(new_length) - len(table)))
-                if new:
-                    rows[r.slot, len(table):len(table) + len(new)] = new
-                    table.extend(new)
-            r.reserved = max(r.reserved, new_length)
+        slots = _ints([self._slots[rid] for rid, _ in wants])
+        lengths = _ints([n for _, n in wants])
+        host.check(self._lib.liyab_cm_reserve(self._h, _ip(slots), _ip(lengths), len(slots)))
+
+    def reserve_more(self, slots: np.ndarray, extra: np.ndarray) -> np.ndarray:
+        """`reserve` for requests named by slot that each bring `extra[i]` more positions than
+        they hold (intc arrays); returns the lengths they will have."""
+        out = np.empty(len(slots), dtype=np.intc)
+        host.check(self._lib.liyab_cm_reserve_more(self._h, _ip(slots), _ip(extra), len(slots), _ip(out)))
+        return out
 
     def commit(self, rid: Hashable, new_length: int) -> None:
         """The request now holds `new_length` positions. Windowed groups give
         back the pages no later query can see: a query at position p >= length
         reads [p - W + 1, p], so pages wholly below length - W + 1 go."""
-        r = self._requests[rid]
-        if self.groups and new_length > len(r.tables[0]) * self.page_size:
-            raise InvalidArgument("commit past the reserved pages")
-        r.length = new_length
-        for gi, g in enumerate(self.groups):
-            if g.spec.window <= 0:
-                continue
-            first_needed = max(0, new_length - g.spec.window + 1)
-            keep_from = first_needed // self.page_size
-            table = r.tables[gi]
-            gone = []
-            for lp in range(r.first_kept[gi], min(keep_from, len(table))):
-                if table[lp] != UNMAPPED:
-                    gone.append(table[lp])
-                    table[lp] = UNMAPPED
-                    self._table_rows[gi][r.slot, lp] = UNMAPPED
-            r.first_kept[gi] = max(r.first_kept[gi], min(keep_from, len(table)))
-            g.pool.release(gone)
+        host.check(self._lib.liyab_cm_commit(self._h, self._slots[rid], new_length))
+
+    def commit_slots(self, slots: np.ndarray, new_lengths: np.ndarray) -> None:
+        """`commit` for several requests named by slot (intc arrays), in one call."""
+        host.check(self._lib.liyab_cm_commit_many(self._h, _ip(slots), _ip(new_lengths), len(slots)))
 
     def truncate(self, rid: Hashable, length: int) -> None:
         """Forgets positions >= length; pages wholly past it are given back
         (the reference's truncate, kv_cache.cpp:418-439). A windowed group
         cannot go back below what it has already released."""
-        r = self._requests[rid]
-        if length > r.length:
-            raise InvalidArgument("truncate cannot grow a request")
-        keep = self._pages_for(length)
-        for gi, g in enumerate(self.groups):
-            if g.spec.window > 0 and r.first_kept[gi] * self.page_size > max(0, length - g.spec.window + 1):
-                raise InvalidArgument("a windowed group has already released what this truncate needs")
-            table = r.tables[gi]
-            g.pool.release([p for p in table[keep:] if p != UNMAPPED])
-            del table[keep:]
-            self._table_rows[gi][r.slot, keep:] = UNMAPPED
-        r.length = length
-        r.reserved = min(r.reserved, keep * self.page_size)
+        host.check(self._lib.liyab_cm_truncate(self._h, self._slots[rid], length))
 
     def block_table(self, rid: Hashable, group: int = 0) -> List[int]:
-        return self._requests[rid].tables[group]
+        slot = self._slots[rid]
+        n = self._lib.liyab_cm_table_length(self._h, slot, group)
+        return self._table_rows[group][slot, :n].tolist()
 
     def table_rows(self, group: int = 0) -> np.ndarray:
         """int32 [max_requests, max_blocks]: the block table of the request in each state slot
@@ -276,10 +271,11 @@ class CacheManager:
 
     def slot_of_position(self, rid: Hashable, group: int, position: int) -> int:
         """page * page_size + offset for a mapped position."""
-        page = self._requests[rid].tables[group][position // self.page_size]
-        if page == UNMAPPED:
+        table = self.block_table(rid, group)
+        lp = position // self.page_size
+        if lp >= len(table) or table[lp] == UNMAPPED:
             raise InvalidArgument(f"position {position} of request {rid!r} is not mapped in group {group}")
-        return page * self.page_size + position % self.page_size
+        return table[lp] * self.page_size + position % self.page_size
 
     # -- accounting -----------------------------------------------------------
     def pages_in_use(self, group: int = 0) -> int:
@@ -290,13 +286,7 @@ class CacheManager:
 
     def check(self) -> None:
         """Invariants over pools, tables and slots (used by the tests)."""
-        for gi, g in enumerate(self.groups):
-            g.pool.check()
-            held = [p for r in self._requests.values() for p in r.tables[gi] if p != UNMAPPED]
-            assert len(held) == len(set(held)), f"group {gi}: a page is in two tables"
-            assert len(held) == g.pool.pages_in_use, f"group {gi}: {g.pool.pages_in_use} pages held, tables name {len(held)}"
-        slots = [r.slot for r in self._requests.values()]
+        host.check(self._lib.liyab_cm_check(self._h))
+        slots = list(self._slots.values())
         assert len(set(slots)) == len(slots), "a state slot is held twice"
-        assert len(set(self._free_slots)) == len(self._free_slots)
-        assert not set(slots) & set(self._free_slots), "a state slot is free and held"
-        assert len(slots) + len(self._free_slots) == self.max_requests, "a state slot was lost"
+        assert len(slots) + self.free_slots() == self.max_requests, "a state slot was lost"

@@ -5,7 +5,10 @@ parallel, and links `liyab_amd/_lib/libliyab_hip.so`; it prints a line per
 file so that a first call in a fresh checkout shows progress. When the
 package folder cannot be written to, the library goes to a per-user folder
 under the system's temporary directory instead. Nothing here needs a GPU:
-hipcc cross-compiles.
+hipcc cross-compiles. `build_host()` does the same for the host-side C++
+under `host/` (the cache manager's bookkeeping and a step's metadata), with
+the system's C++ compiler, into `libliyab_host.so`; that library has nothing
+to do with HIP and loads on a machine without a GPU.
 """
 
 from __future__ import annotations
@@ -152,5 +155,71 @@ def build(quiet: bool = False, jobs: Optional[int] = None) -> str:
     return lib
 
 
+# -- the host library ------------------------------------------------------------------
+HOST_DIR = os.path.join(CSRC, "host")
+HOST_LIB_NAME = "libliyab_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra"]
+
+
+def host_sources() -> List[str]:
+    return sorted(os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+
+
+def host_hash() -> str:
+    h = hashlib.sha256()
+    for f in sorted(os.listdir(HOST_DIR)):
+        if f.endswith((".cpp", ".h")):
+            h.update(f.encode())
+            with open(os.path.join(HOST_DIR, f), "rb") as fh:
+                h.update(fh.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def host_lib_dirs() -> List[str]:
+    return [os.path.join(PKG, "_lib"), os.path.join(tempfile.gettempdir(), f"liyab_amd_{os.getuid()}_host_{host_hash()}")]
+
+
+def find_host_library() -> Optional[str]:
+    """The host library built from the current sources, if there is one."""
+    for d in host_lib_dirs():
+        p = os.path.join(d, HOST_LIB_NAME)
+        try:
+            with open(p + ".hash") as f:
+                if f.read().strip() == host_hash() and os.path.isfile(p):
+                    return p
+        except OSError:
+            pass
+    return None
+
+
+def cxx_path() -> Optional[str]:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"), hipcc_path()):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def build_host(quiet: bool = False) -> str:
+    cxx = cxx_path()
+    if cxx is None:
+        raise RuntimeError("no C++ compiler was found (looked at $CXX, g++, c++, clang++, hipcc): the host library cannot be built")
+    out_dir = next((d for d in host_lib_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError("no writable folder for the host library: tried " + ", ".join(host_lib_dirs()))
+    t0 = time.time()
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    r = subprocess.run([cxx, *HOST_FLAGS, "-I", HOST_DIR, "-o", tmp, *host_sources()], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building {HOST_LIB_NAME} failed:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, lib)
+    with open(lib + ".hash", "w") as f:
+        f.write(host_hash())
+    _say(f"built {lib} in {time.time() - t0:.0f} s", quiet)
+    return lib
+
+
 if __name__ == "__main__":
+    print(build_host())
     print(build())

@@ -1,0 +1,142 @@
+#include "step_meta.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace liyab_host {
+
+static Status fail(std::string* err, Status s, const std::string& msg) {
+    if (err != nullptr) *err = msg;
+    return s;
+}
+
+Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int* q_lens, const int* want_counts,
+                  int decode_q_len, int attn_tile, StepShape* out, std::string* err) {
+    if (n_seqs <= 0) return fail(err, kInvalidArgument, "a step needs at least one item");
+    if (m.n_groups() > kMaxGroups) return fail(err, kInvalidArgument, "more cache groups than a step's metadata holds");
+    StepShape s{};
+    s.n_seqs = n_seqs;
+    s.n_groups = m.n_groups();
+    s.max_blocks = m.max_blocks();
+    for (int i = 0; i < n_seqs; ++i) {
+        if (!m.is_open(slots[i])) return fail(err, kInvalidArgument, "slot " + std::to_string(slots[i]) + " is not open");
+        if (q_lens[i] <= 0) return fail(err, kInvalidArgument, "an item brings no tokens");
+        s.n_tokens += q_lens[i];
+        s.n_logit_rows += want_counts[i];
+        s.max_q_len = std::max(s.max_q_len, q_lens[i]);
+        s.max_context = std::max(s.max_context, m.length(slots[i]) + q_lens[i]);
+    }
+    s.mode = s.max_q_len <= decode_q_len ? 0 : 1;
+    if (s.mode == 1) {
+        for (int i = 0; i < n_seqs; ++i) {
+            if (q_lens[i] <= decode_q_len) s.n_single += q_lens[i];
+            else s.n_tiles += (q_lens[i] + attn_tile - 1) / attn_tile;
+        }
+    }
+    int cur = 0;
+    auto place = [&cur](int size) {
+        const int at = cur;
+        cur += size;
+        return at;
+    };
+    const int N = s.n_tokens, S = n_seqs, R = s.n_logit_rows;
+    s.off_token_ids = place(N);
+    s.off_positions = place(N);
+    s.off_tok_seq = place(N);
+    s.off_seq_starts = place(S + 1);
+    s.off_context_lens = place(S);
+    s.off_state_slots = place(S);
+    s.off_logit_rows = place(std::max(R, 1));
+    s.off_logit_slots = place(std::max(R, 1));
+    s.off_attn_work = place(std::max(4 * s.n_tiles, 1));
+    s.off_attn_single = place(std::max(s.n_single, 1));
+    for (int g = 0; g < s.n_groups; ++g) {
+        s.off_block_tables[g] = place(S * s.max_blocks);
+        s.off_slots[g] = place(N);
+    }
+    s.total = cur;
+    *out = s;
+    return kOk;
+}
+
+Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, const int* q_lens, const int64_t* tokens,
+                 const int* want_counts, const int* wants, int vocab_size, int decode_q_len, int attn_tile, int32_t* block,
+                 std::string* err) {
+    const int S = s.n_seqs, page = m.page_size(), W = s.max_blocks;
+    int32_t* tok = block + s.off_token_ids;
+    int32_t* pos = block + s.off_positions;
+    int32_t* seq = block + s.off_tok_seq;
+    int32_t* starts = block + s.off_seq_starts;
+    int32_t* rows = block + s.off_logit_rows;
+    int32_t* row_slots = block + s.off_logit_slots;
+    rows[0] = 0;
+    row_slots[0] = 0;
+    block[s.off_attn_work] = 0;
+    block[s.off_attn_single] = 0;
+
+    struct Tile {
+        int seq, row, pos, count;
+    };
+    std::vector<Tile> tiles;
+    tiles.reserve(static_cast<size_t>(s.n_tiles));
+    int32_t* single = block + s.off_attn_single;
+    int n_single = 0, row0 = 0, r = 0;
+    for (int i = 0; i < S; ++i) {
+        const int first = m.length(slots[i]), n = q_lens[i];
+        starts[i] = row0;
+        block[s.off_context_lens + i] = first + n;
+        block[s.off_state_slots + i] = slots[i];
+        for (int j = 0; j < n; ++j) {
+            const int64_t id = tokens[row0 + j];
+            if (id >= vocab_size || (id < 0 && (-1 - id) >= m.max_requests()))
+                return fail(err, kInvalidArgument, "token id " + std::to_string(id) + " is outside [0, " + std::to_string(vocab_size) + ")");
+            tok[row0 + j] = static_cast<int32_t>(id);
+            pos[row0 + j] = first + j;
+            seq[row0 + j] = i;
+        }
+        for (int k = 0; k < want_counts[i]; ++k, ++r) {
+            if (wants[r] < 0 || wants[r] >= n)
+                return fail(err, kInvalidArgument, "logits wanted at place " + std::to_string(wants[r]) + " of " + std::to_string(n) + " tokens");
+            rows[r] = row0 + wants[r];
+            row_slots[r] = slots[i];
+        }
+        if (s.mode == 1) {
+            if (n <= decode_q_len) {
+                for (int j = 0; j < n; ++j) single[n_single++] = row0 + j;
+            } else {
+                for (int t0 = 0; t0 < n; t0 += attn_tile) tiles.push_back({i, row0 + t0, first + t0, std::min(attn_tile, n - t0)});
+            }
+        }
+        row0 += n;
+    }
+    starts[S] = row0;
+    // a tile's work grows with its last position: the longest first, so that the short ones
+    // fill the gaps at the end
+    std::stable_sort(tiles.begin(), tiles.end(), [](const Tile& a, const Tile& b) { return a.pos + a.count > b.pos + b.count; });
+    int32_t* work = block + s.off_attn_work;
+    for (size_t t = 0; t < tiles.size(); ++t) {
+        work[4 * t] = tiles[t].seq;
+        work[4 * t + 1] = tiles[t].row;
+        work[4 * t + 2] = tiles[t].pos;
+        work[4 * t + 3] = tiles[t].count;
+    }
+    for (int g = 0; g < s.n_groups; ++g) {
+        int32_t* bt = block + s.off_block_tables[g];
+        int32_t* sl = block + s.off_slots[g];
+        const int32_t* all = m.table_rows(g);
+        for (int i = 0; i < S; ++i) {
+            const int32_t* t = all + static_cast<size_t>(slots[i]) * W;
+            std::copy(t, t + W, bt + static_cast<size_t>(i) * W);
+            const int first = m.length(slots[i]);
+            for (int j = 0; j < q_lens[i]; ++j) {
+                const int p = first + j;
+                const int32_t pg = p / page < W ? t[p / page] : kUnmapped;
+                if (pg < 0) return fail(err, kInternal, "a token of this step maps to a released or unmapped page");
+                sl[starts[i] + j] = pg * page + p % page;
+            }
+        }
+    }
+    return kOk;
+}
+
+}  // namespace liyab_host

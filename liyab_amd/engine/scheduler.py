@@ -189,11 +189,17 @@ class Scheduler:
         groups = self.manager.groups
         need = [0] * len(groups)  # pages this step's batch takes so far, per group
 
+        page, n_groups = self.manager.page_size, len(groups)
+
         def extra(r: Request, count: int) -> List[int]:
-            return self.manager.pages_needed(r.rid, r.computed + count)
+            # new pages per group for positions [computed, computed + count): the request's pages
+            # reach its computed length at least, so this never undercounts
+            return [-(-(r.computed + count) // page) - (-(-r.computed // page))] * n_groups
+
+        free = [g.pool.free_pages for g in groups]  # read again whenever a request is opened or preempted
 
         def fits(r: Request, count: int, pages: Optional[List[int]] = None) -> bool:
-            return all(n + e <= g.pool.free_pages for n, e, g in zip(need, pages or extra(r, count), groups))
+            return all(n + e <= f for n, e, f in zip(need, pages or extra(r, count), free))
 
         def take(r: Request, count: int, pages: Optional[List[int]] = None) -> None:
             nonlocal budget
@@ -232,6 +238,7 @@ class Scheduler:
                 for s in [s for s in batch if s.request is victim]:
                     untake(s)
                 self._preempt(victim)
+                free[:] = [g.pool.free_pages for g in groups]
             if count > 0 and r.state == RUNNING:
                 take(r, count)
         # admission, first come first served
@@ -239,7 +246,7 @@ class Scheduler:
             r = self.waiting[0]
             count = min(r.remaining, self.prefill_chunk, budget)
             pages = -(-count // self.manager.page_size)
-            if self.manager.free_slots() == 0 or any(n + pages > g.pool.free_pages for n, g in zip(need, groups)):
+            if self.manager.free_slots() == 0 or any(n + pages > f for n, f in zip(need, free)):
                 break
             self._open(r)
             self.waiting.popleft()

@@ -19,14 +19,16 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import ctypes
 import itertools
 
 import numpy as np
 import torch
 
-from ..cache.pages import UNMAPPED, CacheManager
+from .. import host
+from ..cache.pages import CacheManager
 from ..cache.storage import CacheStorage
-from ..errors import ContextFull, InvalidArgument
+from ..errors import InvalidArgument
 from ..parts.base import GroupStep, StepContext, StepHost, Workspace
 
 
@@ -126,10 +128,8 @@ class StepFunction:
             for w in it.want:
                 if not (0 <= int(w) < n):
                     raise InvalidArgument(f"request {it.rid!r} wants logits at place {w} of {n} tokens")
-            end = self.manager.length(it.rid) + n
-            if end > self.model.max_positions:
-                raise ContextFull(
-                    f"position {end - 1} is past the model's {self.model.max_positions} learned positions")
+        # a request that would pass the last position is refused by the manager (ContextFull), whose
+        # limit is at most the model's learned positions
 
     # -- eager or replayed ----------------------------------------------------
     def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
@@ -177,109 +177,51 @@ class StepFunction:
         self.last_context = ctx
         return logits
 
-    def commit(self, items: Sequence[StepItem], lengths: Sequence[int]) -> None:
-        """The requests now hold `lengths` positions (after a step's kernels are enqueued)."""
-        for it, n in zip(items, lengths):
-            self.manager.commit(it.rid, n)
+    def commit(self, items: Sequence[StepItem], lengths) -> None:
+        """The requests now hold `lengths` positions (after a step's kernels are enqueued);
+        `lengths` is what `prepare` returned for these items."""
+        slots, new_lengths = lengths
+        self.manager.commit_slots(slots, new_lengths)
         self.steps += 1
         self.tokens += sum(len(it.tokens) for it in items)
 
     def prepare(self, items: Sequence[StepItem]):
         """Checks the items, maps their pages (all or nothing) and puts the step's metadata on
-        the device. Returns (StepContext, the lengths to commit once the step has run)."""
+        the device. Returns (StepContext, what `commit` needs once the step has run). The
+        metadata block is laid out and filled by the host library (csrc/host/step_meta.cpp)
+        straight into pinned memory."""
         self._validate(items)
         mgr = self.manager
-        first = [mgr.length(it.rid) for it in items]
-        q_lens = [len(it.tokens) for it in items]
-        all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64,
-                                 count=sum(q_lens))
-        if any(it.pending_last for it in items):
+        S = len(items)
+        slots = np.fromiter((mgr.slot(it.rid) for it in items), dtype=np.intc, count=S)
+        q_lens = np.fromiter((len(it.tokens) for it in items), dtype=np.intc, count=S)
+        want_counts = np.fromiter((len(it.want) for it in items), dtype=np.intc, count=S)
+        N, R = int(q_lens.sum()), int(want_counts.sum())
+        all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64, count=N)
+        wants = np.fromiter(itertools.chain.from_iterable(it.want for it in items), dtype=np.intc, count=R) if R else \
+            np.zeros(1, dtype=np.intc)
+        pending = [i for i, it in enumerate(items) if it.pending_last]
+        if pending:
             ends = np.cumsum(q_lens) - 1
-            for i, it in enumerate(items):
-                if it.pending_last:
-                    all_tokens[ends[i]] = 0  # checked as a valid id; replaced by a reference below
+            all_tokens[ends[pending]] = 0  # checked as a valid id; replaced by a reference below
         if all_tokens.min() < 0 or all_tokens.max() >= self.model.vocab_size:
             bad = int(all_tokens[(all_tokens < 0) | (all_tokens >= self.model.vocab_size)][0])
             raise InvalidArgument(f"token id {bad} is outside [0, {self.model.vocab_size})")  # src/core/transformer.cpp:6195-6197
-        for i, it in enumerate(items):
-            if it.pending_last:
-                all_tokens[ends[i]] = -1 - mgr.slot(it.rid)
-        mgr.reserve([(it.rid, f + n) for it, f, n in zip(items, first, q_lens)])
+        if pending:
+            all_tokens[ends[pending]] = -1 - slots[pending]  # "the token this slot drew, still on the device"
+        new_lengths = mgr.reserve_more(slots, q_lens)
 
-        S, N = len(items), sum(q_lens)
-        R = sum(len(it.want) for it in items)
-        W = mgr.max_blocks
-        G = len(mgr.groups)
-        page = mgr.page_size
-        starts = np.zeros(S + 1, dtype=np.int64)
-        np.cumsum(q_lens, out=starts[1:])
-
-        # attention's work in a step with long portions: tiles of up to 128 queries for them,
-        # single rows for requests that bring few tokens
-        mode = "decode" if max(q_lens) <= DECODE_Q_LEN else "prefill"
-        tiles, singles = [], []
-        if mode == "prefill":
-            for i, (f, n) in enumerate(zip(first, q_lens)):
-                a = int(starts[i])
-                if n <= DECODE_Q_LEN:
-                    singles.extend(range(a, a + n))
-                else:
-                    for t0 in range(0, n, ATTN_TILE):
-                        tiles.append((i, a + t0, f + t0, min(ATTN_TILE, n - t0)))
-            # a tile's work grows with its last position: the longest first, so that the short
-            # ones fill the gaps at the end
-            tiles.sort(key=lambda t: -(t[2] + t[3]))
-            tiles = [v for t in tiles for v in t]
-        n_tiles = len(tiles) // 4
-
-        # layout of the metadata block (int32 words)
-        off = {}
-        cur = 0
-        for name, size in (("token_ids", N), ("positions", N), ("tok_seq", N), ("seq_starts", S + 1),
-                           ("context_lens", S), ("state_slots", S), ("logit_rows", max(R, 1)),
-                           ("logit_slots", max(R, 1)), ("attn_work", max(len(tiles), 1)), ("attn_single", max(len(singles), 1))):
-            off[name] = (cur, size)
-            cur += size
-        for g in range(G):
-            off[f"bt{g}"] = (cur, S * W)
-            cur += S * W
-            off[f"slots{g}"] = (cur, N)
-            cur += N
-        total = cur
+        lib = host.lib()
+        shape = host.StepShape()
+        ip = lambda a: a.ctypes.data_as(host.IP)  # noqa: E731
+        host.check(lib.liyab_step_shape(mgr.handle, S, ip(slots), ip(q_lens), ip(want_counts), DECODE_Q_LEN, ATTN_TILE,
+                                        ctypes.byref(shape)))
+        total = shape.total
         host_t = self._staging.next(total)
-        host = host_t.numpy()
-
-        def view(name):
-            o, size = off[name]
-            return host[o:o + size]
-
-        tok, pos, seq = view("token_ids"), view("positions"), view("tok_seq")
-        rows = view("logit_rows")
-        q_arr = np.asarray(q_lens, dtype=np.int64)
-        first_arr = np.asarray(first, dtype=np.int64)
-        tok[:] = all_tokens
-        seq[:] = np.repeat(np.arange(S, dtype=np.int32), q_arr)
-        pos[:] = np.repeat(first_arr - starts[:-1], q_arr) + np.arange(N, dtype=np.int64)
-        rows[:] = 0
-        if R:
-            rows[:R] = [int(starts[i]) + int(w) for i, it in enumerate(items) for w in it.want]
-        view("seq_starts")[:] = starts
-        if tiles:
-            view("attn_work")[:] = tiles
-        if singles:
-            view("attn_single")[:] = singles
-        view("context_lens")[:] = first_arr + q_arr
-        slot_ids = np.asarray([mgr.slot(it.rid) for it in items], dtype=np.int64)
-        view("state_slots")[:] = slot_ids
-        if R:
-            view("logit_slots")[:R] = [int(slot_ids[i]) for i, it in enumerate(items) for _ in it.want]
-        for g in range(G):
-            tables = mgr.table_rows(g)[slot_ids]  # [S, W]
-            view(f"bt{g}").reshape(S, W)[:] = tables
-            pages = tables[seq, pos // page]
-            if (pages < 0).any():
-                raise AssertionError("a token of this step maps to a released page")
-            view(f"slots{g}")[:] = pages * page + pos % page
+        host.check(lib.liyab_step_fill(mgr.handle, ctypes.byref(shape), ip(slots), ip(q_lens),
+                                       all_tokens.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), ip(want_counts), ip(wants),
+                                       self.model.vocab_size, DECODE_Q_LEN, ATTN_TILE,
+                                       ctypes.cast(host_t.data_ptr(), ctypes.POINTER(ctypes.c_int32))))
 
         if self._meta_dev is None or self._meta_dev.numel() < total:
             # sized for the largest step of this engine's lifetime where possible: a new block
@@ -290,24 +232,27 @@ class StepFunction:
         dev[:total].copy_(host_t[:total], non_blocking=True)
         self._staging.copied()
 
-        def dview(name):
-            o, size = off[name]
-            return dev[o:o + size]
-
-        max_context = max(f + n for f, n in zip(first, q_lens))
+        W, G, page = shape.max_blocks, shape.n_groups, mgr.page_size
+        prefill = shape.mode == 1
+        starts = np.cumsum(q_lens) - q_lens
         ctx = StepContext(
             n_tokens=N, n_seqs=S,
-            token_ids=dview("token_ids"), positions=dview("positions"), tok_seq=dview("tok_seq"),
-            seq_starts=dview("seq_starts"), context_lens=dview("context_lens"), state_slots=dview("state_slots"),
-            logit_rows=dview("logit_rows"), n_logit_rows=R,
-            groups=[GroupStep(block_tables=dview(f"bt{g}").view(S, W), slots=dview(f"slots{g}")) for g in range(G)],
-            host=StepHost(q_lens=q_lens, starts=[int(s) for s in starts[:-1]], first_pos=first,
-                          max_q_len=max(q_lens), max_context=max_context,
-                          attention_mode=mode, context_bucket=_bucket(max_context), n_attn_tiles=n_tiles, attn_tile=ATTN_TILE,
-                          n_attn_single=len(singles)),
+            token_ids=dev[shape.off_token_ids:shape.off_token_ids + N],
+            positions=dev[shape.off_positions:shape.off_positions + N],
+            tok_seq=dev[shape.off_tok_seq:shape.off_tok_seq + N],
+            seq_starts=dev[shape.off_seq_starts:shape.off_seq_starts + S + 1],
+            context_lens=dev[shape.off_context_lens:shape.off_context_lens + S],
+            state_slots=dev[shape.off_state_slots:shape.off_state_slots + S],
+            logit_rows=dev[shape.off_logit_rows:shape.off_logit_rows + max(R, 1)], n_logit_rows=R,
+            groups=[GroupStep(block_tables=dev[shape.off_block_tables[g]:shape.off_block_tables[g] + S * W].view(S, W),
+                              slots=dev[shape.off_slots[g]:shape.off_slots[g] + N]) for g in range(G)],
+            host=StepHost(q_lens=q_lens.tolist(), starts=starts.tolist(), first_pos=(new_lengths - q_lens).tolist(),
+                          max_q_len=shape.max_q_len, max_context=shape.max_context,
+                          attention_mode="prefill" if prefill else "decode", context_bucket=_bucket(shape.max_context),
+                          n_attn_tiles=shape.n_tiles, attn_tile=ATTN_TILE, n_attn_single=shape.n_single),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
-            logit_slots=dview("logit_slots"), last_tokens=self.last_tokens,
-            attn_work=dview("attn_work") if mode == "prefill" else None,
-            attn_single_rows=dview("attn_single") if mode == "prefill" else None,
+            logit_slots=dev[shape.off_logit_slots:shape.off_logit_slots + max(R, 1)], last_tokens=self.last_tokens,
+            attn_work=dev[shape.off_attn_work:shape.off_attn_work + max(4 * shape.n_tiles, 1)] if prefill else None,
+            attn_single_rows=dev[shape.off_attn_single:shape.off_attn_single + max(shape.n_single, 1)] if prefill else None,
         )
-        return ctx, [f + n for f, n in zip(first, q_lens)]
+        return ctx, (slots, new_lengths)

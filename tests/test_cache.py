@@ -3,7 +3,9 @@ lost, held twice or freed twice under random orders of requests (no GPU)."""
 
 import random
 
+import numpy as np
 import pytest
+
 
 from liyab_amd import Busy, ContextFull, InvalidArgument, OutOfPages
 from liyab_amd.cache import UNMAPPED, CacheManager, KVSpec, PagePool
@@ -172,3 +174,66 @@ def test_random_orders_lose_nothing(seed):
         m.close(rid)
     m.check()
     assert m.pages_in_use(0) == 0 and m.pages_in_use(1) == 0 and m.free_slots() == 5
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_native_manager_does_what_the_plain_one_does(seed):
+    """The same random operations on the native manager and on the plain Python one: the same
+    pages in the same places, the same counters, the same refusals."""
+    import plain_cache
+
+    rng = random.Random(100 + seed)
+    window = rng.choice([0, 24, 70])
+    page_size = rng.choice([4, 16])
+    pages = [rng.randint(10, 40), rng.randint(10, 40)]
+    specs = [(KVSpec(2, 16, 0), [0]), (KVSpec(2, 16, window), [1])]
+    kw = dict(page_size=page_size, num_pages=pages, max_requests=4, max_positions=200)
+    a = CacheManager(specs, **kw)
+    b = plain_cache.CacheManager([(plain_cache.KVSpec(2, 16, 0), [0]), (plain_cache.KVSpec(2, 16, window), [1])], **kw)
+    live, n = {}, 0
+
+    def both(op):
+        """Runs op on both managers; they must agree on the outcome."""
+        out = []
+        for m in (a, b):
+            try:
+                out.append(("ok", op(m)))
+            except (OutOfPages, ContextFull, InvalidArgument, Busy) as e:
+                out.append((type(e).__name__, None))
+        assert out[0] == out[1], out
+        return out[0][0] == "ok"
+
+    for _ in range(500):
+        op = rng.random()
+        if op < 0.15:
+            rid = f"r{n}"
+            n += 1
+            if both(lambda m: m.open(rid)):
+                live[rid] = 0
+        elif op < 0.7 and live:
+            k = rng.randint(1, min(3, len(live)))
+            wants = [(rid, live[rid] + rng.choice([0, 1, 1, 2, 9, 40, 120])) for rid in rng.sample(sorted(live), k)]
+            if both(lambda m: m.reserve(wants)):
+                for rid, length in wants:
+                    if rng.random() < 0.9:
+                        both(lambda m: m.commit(rid, length))
+                        live[rid] = length
+        elif op < 0.8 and live:
+            rid = rng.choice(sorted(live))
+            to = rng.randint(0, live[rid] + 1)
+            if both(lambda m: m.truncate(rid, to)):
+                live[rid] = to
+        elif live:
+            rid = rng.choice(sorted(live))
+            both(lambda m: m.close(rid))
+            del live[rid]
+        a.check()
+        b.check()
+        assert a.free_slots() == b.free_slots()
+        for g in range(2):
+            assert a.free_pages(g) == b.free_pages(g) and a.groups[g].pool.peak_in_use == b.groups[g].pool.peak_in_use
+            assert np.array_equal(a.table_rows(g), b.table_rows(g))
+        for rid, length in live.items():
+            assert a.length(rid) == b.length(rid) == length and a.slot(rid) == b.slot(rid)
+            assert [a.block_table(rid, g) for g in range(2)] == [b.block_table(rid, g) for g in range(2)]
+            assert a.pages_needed(rid, length + 33) == b.pages_needed(rid, length + 33)
