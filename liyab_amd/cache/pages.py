@@ -188,6 +188,14 @@ class CacheManager:
         self._slots[rid] = slot.value
         return slot.value
 
+    def bind(self, rid: Hashable, slot: int) -> None:
+        """The native scheduler opened `slot` for `rid` (it works on the native manager itself)."""
+        self._slots[rid] = slot
+
+    def unbind(self, rid: Hashable) -> None:
+        """The native scheduler closed the request's slot."""
+        self._slots.pop(rid, None)
+
     def is_open(self, rid: Hashable) -> bool:
         return rid in self._slots
 

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "cache_manager.h"
+#include "scheduler.h"
 #include "step_meta.h"
 
 using namespace liyab_host;
@@ -88,6 +89,80 @@ int liyab_step_fill(void* h, const StepShape* shape, const int* slots, const int
                     const int* want_counts, const int* wants, int vocab_size, int decode_q_len, int attn_tile, int32_t* block) {
     return step_fill(*static_cast<CacheManager*>(h), *shape, slots, q_lens, tokens, want_counts, wants, vocab_size, decode_q_len,
                      attn_tile, block, &g_error);
+}
+
+// -- the scheduler --------------------------------------------------------------------
+struct SchedulerHandle {
+    Scheduler sched;
+    std::vector<Scheduled> batch;
+    std::vector<int> opened, preempted;
+};
+
+void* liyab_sched_create(void* manager, int max_num_seqs, int max_batched_tokens, int prefill_chunk) {
+    if (manager == nullptr || max_num_seqs <= 0 || max_batched_tokens <= 0 || prefill_chunk <= 0) {
+        g_error = "max_num_seqs, max_batched_tokens and prefill_chunk must be positive";
+        return nullptr;
+    }
+    return new SchedulerHandle{Scheduler(static_cast<CacheManager*>(manager), max_num_seqs, max_batched_tokens, prefill_chunk), {}, {}, {}};
+}
+void liyab_sched_destroy(void* h) { delete static_cast<SchedulerHandle*>(h); }
+int liyab_sched_add(void* h, int n_prompt, int max_tokens, int* id) {
+    return static_cast<SchedulerHandle*>(h)->sched.add(n_prompt, max_tokens, id, &g_error);
+}
+int liyab_sched_pressure(void* h) { return static_cast<SchedulerHandle*>(h)->sched.pressure() ? 1 : 0; }
+// The step's batch; it stays valid until the next call. counts: [batch, opened, preempted].
+int liyab_sched_schedule(void* h, const Scheduled** batch, const int** opened, const int** preempted, int* counts) {
+    auto* s = static_cast<SchedulerHandle*>(h);
+    const int rc = s->sched.schedule(&s->batch, &s->opened, &s->preempted, &g_error);
+    *batch = s->batch.data();
+    *opened = s->opened.data();
+    *preempted = s->preempted.data();
+    counts[0] = static_cast<int>(s->batch.size());
+    counts[1] = static_cast<int>(s->opened.size());
+    counts[2] = static_cast<int>(s->preempted.size());
+    return rc;
+}
+void liyab_sched_advance(void* h, const Scheduled* batch, int n) { static_cast<SchedulerHandle*>(h)->sched.advance(batch, n); }
+// One sampled token per request named; reasons[i] as Scheduler::token returns it.
+void liyab_sched_tokens(void* h, const int* ids, const int* is_stop, int n, int* reasons) {
+    auto& s = static_cast<SchedulerHandle*>(h)->sched;
+    for (int i = 0; i < n; ++i) reasons[i] = s.token(ids[i], is_stop[i] != 0);
+}
+int liyab_sched_finish(void* h, int id) { return static_cast<SchedulerHandle*>(h)->sched.finish(id, &g_error); }
+// what: 0 state, 1 computed, 2 pending, 3 generated, 4 preemptions, 5 slot
+int liyab_sched_get(void* h, int id, int what) {
+    const auto& s = static_cast<SchedulerHandle*>(h)->sched;
+    if (id < 0 || id >= s.n_requests()) return -1;
+    switch (what) {
+        case 0: return s.state(id);
+        case 1: return s.computed(id);
+        case 2: return s.pending(id);
+        case 3: return s.n_generated(id);
+        case 4: return s.preemptions(id);
+        case 5: return s.slot(id);
+        default: return -1;
+    }
+}
+// ids of the running requests in order of admission (which = 0) or of the waiting ones in queue order (1)
+int liyab_sched_list(void* h, int which, int* out, int cap) {
+    const auto& s = static_cast<SchedulerHandle*>(h)->sched;
+    int n = 0;
+    if (which == 0) {
+        for (int id : s.running())
+            if (n < cap) out[n++] = id;
+    } else {
+        for (int id : s.waiting())
+            if (n < cap) out[n++] = id;
+    }
+    return n;
+}
+void liyab_sched_stats(void* h, long long* out) {
+    const SchedulerStats& st = static_cast<SchedulerHandle*>(h)->sched.stats();
+    out[0] = st.steps;
+    out[1] = st.batched_tokens;
+    out[2] = st.prefill_tokens;
+    out[3] = st.decode_tokens;
+    out[4] = st.preemptions;
 }
 
 }  // extern "C"

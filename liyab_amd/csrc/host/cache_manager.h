@@ -69,6 +69,7 @@ public:
     int max_requests() const { return max_requests_; }
     int max_positions() const { return max_positions_; }
     const PagePool& pool(int g) const { return pools_[g]; }
+    int window(int g) const { return windows_[g]; }
     int free_slots() const { return static_cast<int>(free_slots_.size()); }
 
     Status open(int* slot, std::string* err);

@@ -1,24 +1,15 @@
 """The scheduler: admission, prompt portions under a token budget, decoding,
 finishing, and what happens when pages run out.
 
-The reference schedules by threads: each generating thread submits the pass
-it needs and one of them runs the merged batch (src/core/engine.cpp:1842-2041);
-prompts go in portions of 256 tokens (:2863-2864), a decoding request brings
-one token a pass (:4311-4334), and a request stops at an end-of-generation
-token, at max_tokens or on its callback's word (:4351-4393). When the cache
-cannot grow the reference fails the request (src/core/kv_cache.cpp:249-252,
-src/core/engine.cpp:3878-3882). Here one loop owns all requests:
-
-  * every step first gives each decoding request its one token, then hands
-    the rest of the token budget to prompt portions in order of admission
-    (a portion is as small as the budget leaves, down to one token), then
-    admits waiting requests first come, first served, while a request slot,
-    budget and pages for the first portion are there;
-  * when a request cannot get its pages, the most recently admitted running
-    request is preempted: its pages and slot go back, it returns to the head
-    of the waiting queue and is recomputed from its prompt plus what it has
-    generated. A request is never preempted for its own sake by a later one,
-    and a request that could not fit the pool alone is refused on arrival.
+The decisions are native (`csrc/host/scheduler.{h,cpp}`, where the rules and
+their sources in the reference are written down: decoding requests first,
+then prompt portions under the token budget in order of admission, then
+first-come-first-served admission; when pages run out the most recently
+admitted running request is preempted and recomputed later). This module
+is their Python face: `Request` objects carry what only the caller knows
+(the token ids, the sampling parameters), mirror the counters the native
+side keeps for them, and `Scheduler` turns the native batch into
+`Scheduled` items for the engine.
 
 The scheduler decides on the host from the cache manager's counts only; it
 runs nothing on the GPU and is tested without one.
@@ -26,15 +17,20 @@ runs nothing on the GPU and is tested without one.
 
 from __future__ import annotations
 
+import ctypes
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
+
+from .. import host
 from ..cache.pages import CacheManager
-from ..errors import InvalidArgument, OutOfPages
+from ..errors import InvalidArgument
 from ..sampling import SamplingParams
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+_REASONS = {1: "stop", 2: "length", 3: "context"}
 
 
 @dataclass
@@ -50,6 +46,7 @@ class Request:
     preemptions: int = 0
     arrival: int = 0
     pending: int = 0  # tokens sampled in steps whose result the host has not read yet (at most 1 when scheduling)
+    sid: int = -1  # the native scheduler's id of this request
 
     @property
     def tokens(self) -> List[int]:
@@ -85,6 +82,13 @@ class Scheduled:
     wants_logits: bool  # the portion reaches the request's last token
 
 
+class Batch(list):
+    """A step's `Scheduled` items; `raw` is the native batch they were made from."""
+
+    raw = None
+    n_raw = 0
+
+
 @dataclass
 class SchedulerStats:
     steps: int = 0
@@ -106,30 +110,44 @@ class Scheduler:
         self.prefill_chunk = prefill_chunk
         self.eos_token_id = eos_token_id
         self.on_open = on_open
+        self._lib = host.lib()
+        self._h = self._lib.liyab_sched_create(manager.handle, max_num_seqs, max_batched_tokens, prefill_chunk)
+        if not self._h:
+            raise InvalidArgument(self._lib.liyab_host_last_error().decode())
+        # mirrors of the native queues, as the requests themselves
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
-        self.stats = SchedulerStats()
+        self._by_sid: Dict[int, Request] = {}
         self._arrivals = 0
+        self._peak = 0
+        self._raw = ctypes.POINTER(host.Scheduled)()
+        self._opened, self._preempted = host.IP(), host.IP()
+        self._counts = (ctypes.c_int * 3)()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.liyab_sched_destroy(self._h)
+            self._h = None
+
+    @property
+    def stats(self) -> SchedulerStats:
+        out = (ctypes.c_longlong * 5)()
+        self._lib.liyab_sched_stats(self._h, out)
+        return SchedulerStats(steps=out[0], batched_tokens=out[1], prefill_tokens=out[2], decode_tokens=out[3],
+                              preemptions=out[4], pages_in_use_peak=self._peak)
 
     # -- arrival --------------------------------------------------------------
     def add(self, request: Request) -> None:
-        if not request.prompt:
-            raise InvalidArgument("the prompt is empty")  # src/core/engine.cpp:3867-3871
-        if request.params.max_tokens <= 0:
-            raise InvalidArgument("max_tokens must be positive")
-        if len(request.prompt) >= self.manager.max_positions + 1:
-            raise InvalidArgument(
-                f"the prompt has {len(request.prompt)} tokens; the context holds {self.manager.max_positions}")
-        # the most positions it can come to hold: every token but the last sampled one is run
-        most = min(len(request.prompt) + request.params.max_tokens - 1, self.manager.max_positions)
-        need = -(-most // self.manager.page_size)
-        for g in self.manager.groups:
-            if g.spec.window <= 0 and need > g.pool.num_pages:
-                raise OutOfPages(
-                    f"request {request.rid!r} may need {need} pages; the pool has {g.pool.num_pages} in all")
+        sid = ctypes.c_int(-1)
+        try:
+            host.check(self._lib.liyab_sched_add(self._h, len(request.prompt), int(request.params.max_tokens), ctypes.byref(sid)))
+        except Exception as e:
+            raise type(e)(f"request {request.rid!r}: {e}") from None
+        request.sid = sid.value
         request.state = WAITING
         request.arrival = self._arrivals
         self._arrivals += 1
+        self._by_sid[sid.value] = request
         self.waiting.append(request)
 
     def has_unfinished(self) -> bool:
@@ -144,128 +162,53 @@ class Scheduler:
     def pressure(self) -> bool:
         """Whether the running requests' next portions may not all fit the free pages, so that
         schedule() may have to preempt; the engine then reads pending tokens first."""
-        groups = self.manager.groups
-        free = min(g.pool.free_pages for g in groups)
-        page, chunk = self.manager.page_size, self.prefill_chunk
-        # a portion of c tokens takes at most ceil(c / page) + 1 new pages of a group
-        bound = 0
-        for r in self.running:
-            count = min(r.remaining, chunk)
-            if count > 0:
-                bound += -(-count // page) + 1
-        if bound <= free:
-            return False
-        need = [0] * len(groups)
-        for r in self.running:
-            count = min(r.remaining, chunk)
-            if count <= 0:
-                continue
-            for gi, n in enumerate(self.manager.pages_needed(r.rid, r.computed + count)):
-                need[gi] += n
-        return any(n > g.pool.free_pages for n, g in zip(need, groups))
+        return bool(self._lib.liyab_sched_pressure(self._h))
 
     # -- one step's decisions ---------------------------------------------------
-    def _open(self, r: Request) -> None:
-        self.manager.open(r.rid)
-        if self.on_open is not None:
-            self.on_open(r.rid)
-
-    def _preempt(self, r: Request) -> None:
-        if r.pending > 0:
-            raise AssertionError("a request with a pending token cannot be preempted: read the tokens first")
-        self.manager.close(r.rid)
-        self.running.remove(r)
-        r.computed = 0
-        r.state = WAITING
-        r.preemptions += 1
-        self.stats.preemptions += 1
-        self.waiting.appendleft(r)
-
     def schedule(self) -> List[Scheduled]:
         """Chooses this step's batch and opens/preempts requests accordingly.
         Pages are only counted here; the step function maps them."""
-        budget = self.max_batched_tokens
-        batch: List[Scheduled] = []
-        groups = self.manager.groups
-        need = [0] * len(groups)  # pages this step's batch takes so far, per group
-
-        page, n_groups = self.manager.page_size, len(groups)
-
-        def extra(r: Request, count: int) -> List[int]:
-            # new pages per group for positions [computed, computed + count): the request's pages
-            # reach its computed length at least, so this never undercounts
-            return [-(-(r.computed + count) // page) - (-(-r.computed // page))] * n_groups
-
-        free = [g.pool.free_pages for g in groups]  # read again whenever a request is opened or preempted
-
-        def fits(r: Request, count: int, pages: Optional[List[int]] = None) -> bool:
-            return all(n + e <= f for n, e, f in zip(need, pages or extra(r, count), free))
-
-        def take(r: Request, count: int, pages: Optional[List[int]] = None) -> None:
-            nonlocal budget
-            for gi, e in enumerate(pages or extra(r, count)):
-                need[gi] += e
-            batch.append(Scheduled(r, r.computed, count, r.computed + count == r.n_tokens))
-            budget -= count
-
-        def untake(s: Scheduled) -> None:
-            nonlocal budget
-            for gi, e in enumerate(extra(s.request, s.count)):
-                need[gi] -= e
-            batch.remove(s)
-            budget += s.count
-
-        # running requests: decoding ones first, then prompt portions, each in order of admission
-        active = [r for r in self.running if not self.draining(r)]
-        order = [r for r in active if r.remaining == 1] + [r for r in active if r.remaining > 1]
-        for r in order:
-            if r.state != RUNNING or budget <= 0:
-                continue
-            count = min(r.remaining, self.prefill_chunk, budget)
-            pages = extra(r, count)  # counted once on the common path, where everything fits
-            if fits(r, count, pages):
-                take(r, count, pages)
-                continue
-            while not fits(r, count):
-                victim = self.running[-1]
-                if victim is r:
-                    # nobody later to take pages from: shrink the portion or wait
-                    while count > 1 and not fits(r, count):
-                        count -= 1
-                    if not fits(r, count):
-                        count = 0
-                    break
-                for s in [s for s in batch if s.request is victim]:
-                    untake(s)
-                self._preempt(victim)
-                free[:] = [g.pool.free_pages for g in groups]
-            if count > 0 and r.state == RUNNING:
-                take(r, count)
-        # admission, first come first served
-        while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
-            r = self.waiting[0]
-            count = min(r.remaining, self.prefill_chunk, budget)
-            pages = -(-count // self.manager.page_size)
-            if self.manager.free_slots() == 0 or any(n + pages > f for n, f in zip(need, free)):
-                break
-            self._open(r)
-            self.waiting.popleft()
-            r.state = RUNNING
-            self.running.append(r)
-            take(r, count)
-        if not batch and self.has_unfinished() and not any(r.pending > 0 for r in self.running):
-            raise OutOfPages("no request can make progress: the page pool is too small for any of them")
-        self.stats.steps += 1
-        n = sum(s.count for s in batch)
-        self.stats.batched_tokens += n
-        self.stats.decode_tokens += sum(1 for s in batch if s.count == 1 and s.wants_logits and s.request.generated)
-        self.stats.prefill_tokens = self.stats.batched_tokens - self.stats.decode_tokens
+        rc = self._lib.liyab_sched_schedule(self._h, ctypes.byref(self._raw), ctypes.byref(self._opened),
+                                            ctypes.byref(self._preempted), self._counts)
+        n, n_opened, n_preempted = self._counts
+        # what the native side did to its queues, repeated on the mirrors (preemptions come first)
+        for i in range(n_preempted):
+            r = self._by_sid[self._preempted[i]]
+            self.manager.unbind(r.rid)
+            self.running.remove(r)
+            r.computed = 0
+            r.state = WAITING
+            r.preemptions += 1
+            self.waiting.appendleft(r)
+        host.check(rc)
+        raw = self._raw
+        opened = {self._opened[i] for i in range(n_opened)}
+        batch = Batch()
+        batch.raw, batch.n_raw = raw, n
+        by_sid = self._by_sid
+        for i in range(n):
+            s = raw[i]
+            r = by_sid[s.id]
+            if s.id in opened:
+                self.waiting.popleft()
+                r.state = RUNNING
+                self.running.append(r)
+                self.manager.bind(r.rid, s.slot)
+                if self.on_open is not None:
+                    self.on_open(r.rid)
+            batch.append(Scheduled(r, s.first, s.count, bool(s.wants_logits)))
         return batch
 
     # -- after the step -----------------------------------------------------------
     def advance(self, batch: Sequence[Scheduled]) -> None:
         """The step has been launched: its tokens are in the cache; requests whose portion
         reached their last token have a token pending."""
+        raw, n = getattr(batch, "raw", None), getattr(batch, "n_raw", 0)
+        if raw is None or n != len(batch):
+            raw = (host.Scheduled * len(batch))(*[host.Scheduled(s.request.sid, self.manager.slot(s.request.rid), s.first,
+                                                                 s.count, int(s.wants_logits)) for s in batch])
+            n = len(batch)
+        self._lib.liyab_sched_advance(self._h, raw, n)
         for s in batch:
             s.request.computed += s.count
             if s.wants_logits:
@@ -276,28 +219,30 @@ class Scheduler:
         """The step's sampled tokens have reached the host; returns requests that finished.
         A request that finished meanwhile (its earlier token ended it while this step was in
         flight) is skipped: what this step computed for it is dropped."""
-        done = []
-        for s in batch:
-            r = s.request
-            if not s.wants_logits or r.state == FINISHED:
-                continue
-            token = sampled[r.rid]
-            r.pending -= 1
-            r.generated.append(token)
-            reason = None
-            if self.eos_token_id is not None and token == self.eos_token_id:
-                reason = "stop"
-            elif len(r.generated) >= r.params.max_tokens:
-                reason = "length"
-            elif len(r.prompt) + len(r.generated) > self.manager.max_positions:
-                reason = "context"  # the next token would pass the last position
-            if on_token is not None and on_token(r, token) is False and reason is None:
-                reason = "callback"
-            if reason is not None:
-                self.finish(r, reason)
-                done.append(r)
-        self.stats.pages_in_use_peak = max(self.stats.pages_in_use_peak,
-                                           max((g.pool.peak_in_use for g in self.manager.groups), default=0))
+        wanting = [s.request for s in batch if s.wants_logits]
+        done: List[Request] = []
+        if wanting:
+            tokens = [sampled[r.rid] if r.state != FINISHED else 0 for r in wanting]
+            ids = np.fromiter((r.sid for r in wanting), dtype=np.intc, count=len(wanting))
+            eos = self.eos_token_id
+            stops = np.fromiter((eos is not None and t == eos for t in tokens), dtype=np.intc, count=len(wanting))
+            reasons = np.empty(len(wanting), dtype=np.intc)
+            ip = lambda a: a.ctypes.data_as(host.IP)  # noqa: E731
+            self._lib.liyab_sched_tokens(self._h, ip(ids), ip(stops), len(wanting), ip(reasons))
+            for r, token, code in zip(wanting, tokens, reasons.tolist()):
+                if code < 0:
+                    continue  # finished meanwhile
+                r.pending -= 1
+                r.generated.append(token)
+                reason = _REASONS.get(code)
+                if reason is not None:
+                    self._finished(r, reason)  # the native side has already let go of it
+                if on_token is not None and on_token(r, token) is False and reason is None:
+                    reason = "callback"
+                    self.finish(r, reason)
+                if reason is not None:
+                    done.append(r)
+        self._peak = max(self._peak, max((g.pool.peak_in_use for g in self.manager.groups), default=0))
         return done
 
     def update(self, batch: Sequence[Scheduled], sampled: Dict[Hashable, int],
@@ -306,12 +251,17 @@ class Scheduler:
         self.advance(batch)
         return self.resolve(batch, sampled, on_token)
 
-    def finish(self, r: Request, reason: str) -> None:
+    def _finished(self, r: Request, reason: str) -> None:
         if r.state == RUNNING:
-            self.manager.close(r.rid)
+            self.manager.unbind(r.rid)
             self.running.remove(r)
         elif r.state == WAITING:
             self.waiting.remove(r)
         r.state = FINISHED
         r.pending = 0
         r.finish_reason = reason
+
+    def finish(self, r: Request, reason: str) -> None:
+        if r.state != FINISHED:
+            host.check(self._lib.liyab_sched_finish(self._h, r.sid))
+        self._finished(r, reason)

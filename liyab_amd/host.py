@@ -25,6 +25,12 @@ class StepShape(ctypes.Structure):
         ("off_block_tables", c_int * MAX_GROUPS), ("off_slots", c_int * MAX_GROUPS)]
 
 
+class Scheduled(ctypes.Structure):
+    """Mirror of liyab_host::Scheduled (csrc/host/scheduler.h)."""
+
+    _fields_ = [(n, c_int) for n in ("id", "slot", "first", "count", "wants_logits")]
+
+
 IP = POINTER(c_int)
 _SIGNATURES = {
     "liyab_host_last_error": ([], c_char_p),
@@ -53,6 +59,17 @@ _SIGNATURES = {
     "liyab_cm_free_pages": ([c_void_p, c_int], c_int),
     "liyab_cm_peak_in_use": ([c_void_p, c_int], c_int),
     "liyab_cm_check": ([c_void_p], c_int),
+    "liyab_sched_create": ([c_void_p, c_int, c_int, c_int], c_void_p),
+    "liyab_sched_destroy": ([c_void_p], None),
+    "liyab_sched_add": ([c_void_p, c_int, c_int, IP], c_int),
+    "liyab_sched_pressure": ([c_void_p], c_int),
+    "liyab_sched_schedule": ([c_void_p, POINTER(POINTER(Scheduled)), POINTER(IP), POINTER(IP), IP], c_int),
+    "liyab_sched_advance": ([c_void_p, POINTER(Scheduled), c_int], None),
+    "liyab_sched_tokens": ([c_void_p, IP, IP, c_int, IP], None),
+    "liyab_sched_finish": ([c_void_p, c_int], c_int),
+    "liyab_sched_get": ([c_void_p, c_int, c_int], c_int),
+    "liyab_sched_list": ([c_void_p, c_int, IP, c_int], c_int),
+    "liyab_sched_stats": ([c_void_p, POINTER(ctypes.c_longlong)], None),
     "liyab_step_shape": ([c_void_p, c_int, IP, IP, IP, c_int, c_int, POINTER(StepShape)], c_int),
     "liyab_step_fill": ([c_void_p, POINTER(StepShape), IP, IP, POINTER(c_int64), IP, IP, c_int, c_int, c_int,
                          POINTER(c_int32)], c_int),

@@ -258,3 +258,86 @@ def test_token_slice_equals_a_slice_of_tokens():
         count = rng.randrange(0, r.n_tokens - first + 1)
         assert r.token_slice(first, count) == r.tokens[first:first + count]
         assert len(r.prompt) + len(r.generated) + r.pending == r.n_tokens
+
+
+@pytest.mark.parametrize("lagged", [False, True])
+@pytest.mark.parametrize("seed", range(6))
+def test_native_scheduler_decides_as_the_plain_one(seed, lagged):
+    """The same random arrivals, with few pages, through the native scheduler and the plain Python
+    one (each on a manager of its own): the same batch at every step, the same queues, the same
+    preemptions, the same tokens in the end."""
+    import random
+
+    import plain_cache
+    import plain_scheduler
+
+    rng = random.Random(500 + seed)
+    page_size, num_pages = rng.choice([4, 16]), rng.randint(8, 24)
+    kw = dict(page_size=page_size, num_pages=num_pages, max_requests=5, max_positions=120)
+    skw = dict(max_num_seqs=rng.randint(2, 5), max_batched_tokens=rng.choice([16, 40, 64]), prefill_chunk=rng.choice([5, 16, 48]))
+    arrivals = []
+    for i in range(rng.randint(4, 9)):
+        n = rng.randint(1, min(60, num_pages * page_size - 1))
+        arrivals.append((rng.randint(0, 25), f"q{i}", [rng.randrange(90) for _ in range(n)], rng.randint(1, 40)))
+    eos = rng.choice([None, 7, 50])
+
+    def drive(native):
+        if native:
+            m = CacheManager([(KVSpec(2, 16, 0), [0])], **kw)
+            s = Scheduler(m, eos_token_id=eos, **skw)
+            make = Request
+        else:
+            m = plain_cache.CacheManager([(plain_cache.KVSpec(2, 16, 0), [0])], **kw)
+            s = plain_scheduler.Scheduler(m, eos_token_id=eos, **skw)
+            make = plain_scheduler.Request
+        log, reqs, pending, inflight, step = [], [], sorted(arrivals), None, 0
+
+        def snapshot(batch):
+            log.append(([(b.request.rid, b.first, b.count, b.wants_logits) for b in batch],
+                        [r.rid for r in s.running], [r.rid for r in s.waiting], m.free_pages(0),
+                        s.stats.preemptions, s.stats.decode_tokens, s.stats.batched_tokens))
+
+        while s.has_unfinished() or inflight is not None or pending:
+            while pending and pending[0][0] <= step:
+                _, rid, prompt, max_tokens = pending.pop(0)
+                r = make(rid, list(prompt), SamplingParams(temperature=0, max_tokens=max_tokens))
+                try:
+                    s.add(r)
+                    reqs.append(r)
+                except (InvalidArgument, OutOfPages) as e:
+                    log.append(("refused", rid, type(e).__name__))
+            step += 1
+            if not s.has_unfinished() and inflight is None:
+                continue
+            if inflight is not None and (not lagged or s.pressure()):
+                s.resolve(*inflight)
+                inflight = None
+                if not s.has_unfinished():
+                    continue
+            batch = s.schedule()
+            snapshot(batch)
+            if not batch:
+                assert inflight is not None
+                s.resolve(*inflight)
+                inflight = None
+                continue
+            m.reserve([(b.request.rid, b.first + b.count) for b in batch])
+            truth = {}
+            for b in batch:
+                m.commit(b.request.rid, b.first + b.count)
+                if b.wants_logits:
+                    r = b.request
+                    known = make("x", r.prompt + r.generated + ([r._late] if r.pending else []), r.params)
+                    truth[r.rid] = r._late = next_token(known)
+            s.advance(batch)
+            previous, inflight = inflight, (batch, truth)
+            if previous is not None:
+                s.resolve(*previous)
+            m.check()
+            assert step < 5000
+        assert m.pages_in_use(0) == 0
+        return log, [(r.rid, r.generated, r.finish_reason, r.preemptions, r.state) for r in reqs]
+
+    native, plain = drive(True), drive(False)
+    assert native[0] == plain[0]
+    assert native[1] == plain[1]
