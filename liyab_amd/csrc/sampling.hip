@@ -240,6 +240,392 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
     }
 }
 
+// The same rules with the row held in registers, for vocabularies up to THREADS * EPT entries
+// (1024 threads up to 16 ids each, 512 threads up to 128: the registers of a wave must hold
+// them). Wave w owns the ids [w * 64 * chunk, (w + 1) * 64 * chunk); within it lane l holds
+// groups of 4 consecutive ids, its g-th group starting at (g * 64 + l) * 4, so the order of
+// ids within a wave is (group, lane, place in the group). The row is read once; the
+// bisections for the k-th largest key and for the top-p threshold then cost compares on
+// registers instead of passes over memory. With top-k of at most 64 (the usual case) the
+// kept logits are gathered into LDS and one wave finishes: nucleus cut and draw among at most
+// 64 candidates. Masses are fixed-point integers, exp((l - l_max) / T) * 2^44 rounded down, so
+// that every sum is exact and independent of the order of the additions; a probability below
+// 2^-44 of the largest counts as none.
+constexpr int kMassBits = 44;
+constexpr int kWaveCandidates = 64;
+
+__device__ __forceinline__ unsigned long long fixed_mass(uint32_t key, float lmax, float scale2) {
+    // exp((l - l_max) / T) through the hardware's 2^x (scale2 = log2(e) / T), in [0, 1]; times
+    // 2^44 (exact), then split into the words of a 64-bit integer: the part above 2^32 has at
+    // most 13 bits, so its product with 2^32 and the remainder are exact in 32-bit floats
+    const float x = __builtin_amdgcn_exp2f((key_value(key) - lmax) * scale2) * static_cast<float>(1ull << kMassBits);
+    const uint32_t hi = static_cast<uint32_t>(x * (1.0f / 4294967296.0f));
+    const uint32_t lo = static_cast<uint32_t>(fmaf(-static_cast<float>(hi), 4294967296.0f, x));
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+
+// The same value, opaque to the compiler: what is computed from it is computed again instead of
+// being kept in registers from an earlier pass over the row (two more registers per id held).
+__device__ __forceinline__ uint32_t again(uint32_t key) {
+    asm volatile("" : "+v"(key));
+    return key;
+}
+
+__device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, int delta) {
+    const uint32_t lo = __shfl_up(static_cast<uint32_t>(v), delta, kWave);
+    const uint32_t hi = __shfl_up(static_cast<uint32_t>(v >> 32), delta, kWave);
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+__device__ __forceinline__ unsigned long long shfl_u64(unsigned long long v, int src) {
+    const uint32_t lo = __shfl(static_cast<uint32_t>(v), src, kWave);
+    const uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), src, kWave);
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), off, kWave);
+        const uint32_t hi = __shfl_xor(static_cast<uint32_t>(v >> 32), off, kWave);
+        v += (static_cast<unsigned long long>(hi) << 32) | lo;
+    }
+    return v;
+}
+
+// Sums over a workgroup of WAVES waves, exact; every thread gets the result. `red`: WAVES values.
+template <int WAVES>
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* red) {
+    v = wave_sum_u64(v);
+    __syncthreads();
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    unsigned long long t = 0;
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) t += red[i];
+    return t;
+}
+template <int WAVES>
+__device__ __forceinline__ int block_count(int v, int* red) {
+    v = wave_sum_i(v);
+    __syncthreads();
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = v;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) t += red[i];
+    return t;
+}
+
+template <int EPT, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t ld, int V,
+                        const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
+                        const double* __restrict__ uniform, const int* __restrict__ scatter_index, int* __restrict__ scatter_out) {
+    static_assert(EPT % 4 == 0, "ids are held in groups of 4");
+    constexpr int WAVES = THREADS / kWave, GROUPS = EPT / 4;
+    __shared__ unsigned long long red64[WAVES];
+    __shared__ uint32_t redk[WAVES];
+    __shared__ int redi[WAVES];
+    __shared__ int result, n_cand;
+    __shared__ uint32_t cand_key[kWaveCandidates];
+    __shared__ int cand_id[kWaveCandidates];
+
+    const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const float* row = logits + static_cast<int64_t>(r) * ld;
+    const int chunk = (((V + THREADS - 1) / THREADS + 3) / 4) * 4;  // ids a thread, <= EPT (checked by the launcher)
+    const int span0 = wave * kWave * chunk;
+    auto id_of = [&](int j) { return span0 + ((j / 4) * kWave + lane) * 4 + j % 4; };
+    // keys of this thread's ids; 0 stands for "no element" (no real logit has that key)
+    uint32_t keys[EPT];
+    // every load from a valid address (an id past the row reads the row's last entry), so that no
+    // condition has to live while the loads are in flight; what is past the row is dropped after
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) keys[j] = __float_as_uint(row[min(id_of(j), V - 1)]);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const uint32_t raw = again(keys[j]);
+        keys[j] = (j < chunk && id_of(j) < V) ? ordered_key(__uint_as_float(raw)) : 0u;
+    }
+    // the largest key and its lowest id
+    uint32_t kmax = 0;
+    int imax = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+        if (keys[j] > kmax) { kmax = keys[j]; imax = id_of(j); }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const uint32_t ok = __shfl_xor(kmax, off, kWave);
+        const int oi = __shfl_xor(imax, off, kWave);
+        if (ok > kmax || (ok == kmax && oi < imax)) { kmax = ok; imax = oi; }
+    }
+    if (lane == 0) { redk[wave] = kmax; redi[wave] = imax; }
+    if (tid == 0) { result = -1; n_cand = 0; }
+    __syncthreads();
+    kmax = redk[0]; imax = redi[0];
+#pragma unroll
+    for (int i = 1; i < WAVES; ++i)
+        if (redk[i] > kmax || (redk[i] == kmax && redi[i] < imax)) { kmax = redk[i]; imax = redi[i]; }
+    if (imax == 0x7fffffff) imax = 0;
+    const float T = temperature != nullptr ? temperature[r] : 0.0f;
+    if (!(T > 0.0f)) {
+        if (tid == 0) {
+            out[r] = imax;
+            if (scatter_index != nullptr) scatter_out[scatter_index[r]] = imax;
+        }
+        return;
+    }
+    const float lmax = key_value(kmax), inv_t = 1.4426950408889634f / T;  // exponentials are taken in base 2
+    const int k = top_k != nullptr ? top_k[r] : 0;
+    const float tp = top_p != nullptr ? top_p[r] : 1.0f;
+    const bool use_k = k > 0 && k < V, use_p = tp < 1.0f;
+    const unsigned long long lanes_below = (1ull << lane) - 1ull;
+
+    // Which of this thread's ids are kept, as bits: key > t, or key == t and among the first
+    // `ties` of the ids with that key (ascending ids: waves in order, within a wave groups, lanes,
+    // places). When every tie is kept no ranks are needed.
+    auto kept_bits = [&](uint32_t t, int ties, uint32_t (&bits)[(EPT + 31) / 32]) {
+        int n_ties = 0;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) n_ties += keys[j] == t && keys[j] != 0u;
+        const int all_ties = block_count<WAVES>(n_ties, redi);
+#pragma unroll
+        for (int w = 0; w < (EPT + 31) / 32; ++w) bits[w] = 0u;
+        if (ties >= all_ties) {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j)
+                if (keys[j] != 0u && keys[j] >= t) bits[j / 32] |= 1u << (j % 32);
+            return;
+        }
+        const int in_wave = wave_sum_i(n_ties);
+        __syncthreads();
+        if (lane == 0) redi[wave] = in_wave;
+        __syncthreads();
+        int rank = 0;  // ties before this wave, then before the group at hand
+        for (int w = 0; w < wave; ++w) rank += redi[w];
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            unsigned long long tied[4];
+            int below = 0, in_group = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                tied[e] = __ballot(keys[4 * g + e] == t && keys[4 * g + e] != 0u);
+                below += __popcll(tied[e] & lanes_below);
+                in_group += __popcll(tied[e]);
+            }
+            int mine = rank + below;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t key = keys[4 * g + e];
+                const bool tie = key == t && key != 0u;
+                if (key > t || (tie && mine < ties)) bits[(4 * g + e) / 32] |= 1u << ((4 * g + e) % 32);
+                mine += tie;
+            }
+            rank += in_group;
+        }
+    };
+
+    // ---- top-k: the k-th largest key, and how many of its ties are kept ----
+    uint32_t tau_k = 0;
+    int ties_k = 0x7fffffff;
+    if (use_k) {
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tau_k | (1u << bit);
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) c += keys[j] >= cand;
+            if (block_count<WAVES>(c, redi) >= k) tau_k = cand;
+        }
+        int c = 0;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) c += keys[j] > tau_k;
+        ties_k = k - block_count<WAVES>(c, redi);
+    }
+
+    uint32_t bits[(EPT + 31) / 32];
+    if (use_k && k <= kWaveCandidates) {
+        // ---- few candidates: gathered, then one wave does the rest ----
+        kept_bits(tau_k, ties_k, bits);
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            if (bits[j / 32] >> (j % 32) & 1u) {
+                const int at = atomicAdd(&n_cand, 1);  // the order of arrival does not matter: ranks below are by key and id
+                cand_key[at] = keys[j];
+                cand_id[at] = id_of(j);
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        const int n = n_cand;  // = k
+        const bool has = lane < n;
+        const uint32_t key = has ? cand_key[lane] : 0u;
+        const int id = has ? cand_id[lane] : 0x7fffffff;
+        const unsigned long long q = has ? fixed_mass(key, lmax, inv_t) : 0ull;
+        // place in the descending order of keys (ties by ascending id) and in the ascending order of ids
+        int desc = 0, asc = 0;
+        for (int o = 0; o < n; ++o) {
+            const uint32_t ok = __shfl(key, o, kWave);
+            const int oi = __shfl(id, o, kWave);
+            desc += ok > key || (ok == key && oi < id);
+            asc += oi < id;
+        }
+        bool kept = has;
+        if (use_p) {
+            // cum = mass of the candidates before this one in descending order, itself included
+            unsigned long long cum = 0, total = 0;
+            for (int o = 0; o < n; ++o) {
+                const unsigned long long oq = shfl_u64(q, o);
+                const int od = __shfl(desc, o, kWave);
+                total += oq;
+                if (od <= desc) cum += oq;
+            }
+            const double target = static_cast<double>(tp) * static_cast<double>(total);
+            // the shortest prefix whose mass reaches the target: an element is kept when the prefix
+            // before it has not reached it yet; the first is always kept
+            kept = has && (desc == 0 || static_cast<double>(cum - q) < target);
+        }
+        const unsigned long long mass = kept ? q : 0ull;
+        unsigned long long before = 0, total = 0;
+        for (int o = 0; o < n; ++o) {
+            const unsigned long long om = shfl_u64(mass, o);
+            const int oa = __shfl(asc, o, kWave);
+            total += om;
+            if (oa < asc) before += om;
+        }
+        int token = imax;
+        if (total > 0ull) {
+            unsigned long long rr = static_cast<unsigned long long>(uniform[r] * static_cast<double>(total));
+            if (rr >= total) rr = total - 1;
+            const bool mine = kept && rr >= before && rr - before < mass;
+            const unsigned long long pick = __ballot(mine);
+            if (pick != 0ull) token = __shfl(id, __ffsll(static_cast<long long>(pick)) - 1, kWave);
+        }
+        if (lane == 0) {
+            out[r] = token;
+            if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
+        }
+        return;
+    }
+
+    // ---- top-p over many candidates: the key where the descending cumulative mass reaches top_p ----
+    uint32_t tau = tau_k;
+    int ties = ties_k;
+    if (use_p) {
+        const unsigned long long tie_mass_k = use_k ? static_cast<unsigned long long>(ties_k) * fixed_mass(tau_k, lmax, inv_t) : 0ull;
+        // mass of {key >= cand} within the top-k set (ties at tau_k counted ties_k times)
+        auto mass_ge = [&](uint32_t cand) -> unsigned long long {
+            unsigned long long m = 0;
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const uint32_t key = again(keys[j]);
+                if (key >= cand && key > tau_k) m += fixed_mass(key, lmax, inv_t);
+            }
+            m = block_sum_u64<WAVES>(m, red64);
+            return (use_k && cand <= tau_k) ? m + tie_mass_k : m;
+        };
+        const double target = static_cast<double>(tp) * static_cast<double>(mass_ge(0u));
+        uint32_t tau_p = 0;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tau_p | (1u << bit);
+            if (static_cast<double>(mass_ge(cand)) >= target) tau_p = cand;
+        }
+        if (tau_p < tau_k) tau_p = tau_k;
+        const unsigned long long above = tau_p == 0xffffffffu ? 0ull : mass_ge(tau_p + 1u);
+        int avail;
+        if (use_k && tau_p == tau_k) {
+            avail = ties_k;
+        } else {
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) c += keys[j] == tau_p;
+            avail = block_count<WAVES>(c, redi);
+        }
+        // the prefix grows one tie at a time until its share reaches top_p
+        const unsigned long long p_tie = fixed_mass(tau_p, lmax, inv_t);
+        int need = 1;
+        if (p_tie > 0ull) {
+            unsigned long long cum = above;
+            need = 0;
+            while (need < avail) {
+                cum += p_tie;
+                ++need;
+                if (static_cast<double>(cum) >= target) break;
+            }
+            if (need < 1) need = 1;
+        }
+        tau = tau_p;
+        ties = need < avail ? need : avail;
+    }
+
+    // ---- inverse CDF over ascending ids among the kept ----
+    kept_bits(tau, ties, bits);
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+        if (bits[j / 32] >> (j % 32) & 1u) mine += fixed_mass(again(keys[j]), lmax, inv_t);
+    // the wave where the walk ends, from the waves' masses in order; then that wave alone walks
+    // its ids in their order: group by group, a scan over the lanes' four ids each
+    const unsigned long long wave_mass = wave_sum_u64(mine);
+    __syncthreads();
+    if (lane == 0) red64[wave] = wave_mass;
+    __syncthreads();
+    unsigned long long total = 0, before = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        if (w < wave) before += red64[w];
+        total += red64[w];
+    }
+    if (total > 0ull) {
+        unsigned long long rr = static_cast<unsigned long long>(uniform[r] * static_cast<double>(total));
+        if (rr >= total) rr = total - 1;
+        if (rr >= before && rr - before < wave_mass) {  // wave-uniform
+            unsigned long long left = rr - before;
+            int found = -1;
+#pragma unroll
+            for (int g = 0; g < GROUPS; ++g) {
+                unsigned long long q[4], q4 = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 4 * g + e;
+                    q[e] = (bits[j / 32] >> (j % 32) & 1u) ? fixed_mass(again(keys[j]), lmax, inv_t) : 0ull;
+                    q4 += q[e];
+                }
+                unsigned long long inc = q4;
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1) {
+                    const unsigned long long o = shfl_up_u64(inc, d);
+                    if (lane >= d) inc += o;
+                }
+                const unsigned long long group_total = shfl_u64(inc, kWave - 1);
+                if (found < 0) {
+                    if (left < group_total) {
+                        const unsigned long long pick = __ballot(q4 > 0ull && left >= inc - q4 && left < inc);
+                        const int src = __ffsll(static_cast<long long>(pick)) - 1;
+                        // within the lane's four ids
+                        unsigned long long rest = left - (inc - q4);
+                        int e_pick = 3;
+#pragma unroll
+                        for (int e = 3; e >= 0; --e) {
+                            unsigned long long upto = 0;
+#pragma unroll
+                            for (int e2 = 0; e2 <= e; ++e2) upto += q[e2];
+                            if (q[e] > 0ull && rest < upto) e_pick = e;
+                        }
+                        found = __shfl(id_of(4 * g) + e_pick, src, kWave);
+                    } else {
+                        left -= group_total;
+                    }
+                }
+            }
+            if (lane == 0) result = found;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const int token = result < 0 ? imax : result;
+        out[r] = token;
+        if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
+    }
+}
+
 // Argmax in two stages so that a few rows still use many CUs: chunks of a row give partial
 // (value, id) pairs, then one wave per row picks among them; ties go to the lowest id.
 constexpr int AM_CHUNKS = 64;
@@ -321,6 +707,15 @@ extern "C" int liyab_sample(int* out, const float* logits, int64_t ld, int rows,
     LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d", rows, V);
     if (rows == 0) return 0;
     LIYAB_REQUIRE(scatter_index == nullptr || scatter_out != nullptr, "sample: a scatter index needs a target");
-    sample_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out);
+    // the row in registers where it fits; the general kernel beyond
+#define LIYAB_REGS(E, T) sample_registers_kernel<E, T><<<rows, T, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out)
+    if (V <= 8 * 1024) LIYAB_REGS(8, 1024);
+    else if (V <= 16 * 1024) LIYAB_REGS(16, 1024);
+    else if (V <= 48 * 512) LIYAB_REGS(48, 512);
+    else if (V <= 72 * 512) LIYAB_REGS(72, 512);
+    else if (V <= 104 * 512) LIYAB_REGS(104, 512);
+    else if (V <= 128 * 512) LIYAB_REGS(128, 512);
+    else sample_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out);
+#undef LIYAB_REGS
     return check_launch("sample");
 }

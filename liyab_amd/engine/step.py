@@ -20,6 +20,7 @@ from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
 import ctypes
+import gc
 import itertools
 
 import numpy as np
@@ -154,8 +155,16 @@ class StepFunction:
             return self.model.forward(ctx, self.storage)
         before = self.workspace.generation
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = self.model.forward(ctx, self.storage)
+        # no garbage collection while the stream is capturing: an engine collected then would free
+        # pinned memory and events in the middle of the capture, which the runtime answers by aborting
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ctx, self.storage)
+        finally:
+            if gc_was_on:
+                gc.enable()
         if self.workspace.generation != before:
             # a buffer grew during capture: its old address is baked into the graph; run eagerly
             self._graphs[key] = 1

@@ -55,22 +55,33 @@ def uniform(seed: int, index: int) -> float:
 class Sampler:
     """Samples one token per logits row on the device."""
 
+    _RING = 4  # pinned staging buffers used in turn
+
     def __init__(self, device):
         import torch
 
         self.device = torch.device(device)
         self._cap = 0
+        self._turn = 0
 
     def _buffers(self, rows: int):
+        """Per-row parameters live in one device block, [uniform f64 | temperature f32 | top_k i32 |
+        top_p f32] x capacity, filled from pinned host memory by one asynchronous copy a step."""
         import torch
 
         if rows > self._cap:
             cap = max(rows, 64, 2 * self._cap)
             self._out = torch.empty(cap, dtype=torch.int32, device=self.device)
-            self._temp = torch.empty(cap, dtype=torch.float32, device=self.device)
-            self._topk = torch.empty(cap, dtype=torch.int32, device=self.device)
-            self._topp = torch.empty(cap, dtype=torch.float32, device=self.device)
-            self._u = torch.empty(cap, dtype=torch.float64, device=self.device)
+            self._block = torch.empty(cap * 20, dtype=torch.uint8, device=self.device)
+            self._u = self._block[:cap * 8].view(torch.float64)
+            self._temp = self._block[cap * 8:cap * 12].view(torch.float32)
+            self._topk = self._block[cap * 12:cap * 16].view(torch.int32)
+            self._topp = self._block[cap * 16:cap * 20].view(torch.float32)
+            self._host = [torch.empty(cap * 20, dtype=torch.uint8, pin_memory=True) for _ in range(self._RING)]
+            self._host_np = [(h[:cap * 8].view(torch.float64).numpy(), h[cap * 8:cap * 12].view(torch.float32).numpy(),
+                              h[cap * 12:cap * 16].view(torch.int32).numpy(), h[cap * 16:cap * 20].view(torch.float32).numpy())
+                             for h in self._host]
+            self._events = [None] * self._RING
             self._cap = cap
 
     def sample_on_device(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int],
@@ -91,10 +102,19 @@ class Sampler:
         if all(p.greedy for p in params):
             ops.argmax(out, logits, scatter=scatter)
         else:
-            self._temp[:rows].copy_(torch.tensor([float(p.temperature) for p in params], dtype=torch.float32))
-            self._topk[:rows].copy_(torch.tensor([int(p.top_k) for p in params], dtype=torch.int32))
-            self._topp[:rows].copy_(torch.tensor([float(p.top_p) for p in params], dtype=torch.float32))
-            self._u[:rows].copy_(torch.tensor([uniform(s, i) for s, i in zip(seeds, indices)], dtype=torch.float64))
+            i = self._turn
+            self._turn = (i + 1) % self._RING
+            if self._events[i] is not None:
+                self._events[i].synchronize()  # its last copy has long finished
+            u, temp, topk, topp = self._host_np[i]
+            u[:rows] = [uniform(s, n) for s, n in zip(seeds, indices)]
+            temp[:rows] = [p.temperature for p in params]
+            topk[:rows] = [p.top_k for p in params]
+            topp[:rows] = [p.top_p for p in params]
+            self._block.copy_(self._host[i], non_blocking=True)
+            if self._events[i] is None:
+                self._events[i] = torch.cuda.Event()
+            self._events[i].record()
             ops.sample(out, logits, self._temp[:rows], self._topk[:rows], self._topp[:rows], self._u[:rows],
                        scatter=scatter)
         return out

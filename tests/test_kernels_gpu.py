@@ -404,19 +404,22 @@ def test_argmax_ties_go_to_the_lowest_id(ops, rows, V):
     assert out.tolist() == rnd(rows, V, seed=4).argmax(dim=1).tolist()
 
 
-def test_sampler_against_the_plain_sampler(ops):
-    """Temperature, top-k and top-p per row against the plain implementation's rules."""
+@pytest.mark.parametrize("V", [1000, 50257, 70001])
+def test_sampler_against_the_plain_sampler(ops, V):
+    """Temperature, top-k and top-p per row against the plain implementation's rules, at
+    vocabularies that take each of the sampling kernels (the row in registers with a one-wave
+    finish for top-k <= 64, the same with many candidates, and the general kernel)."""
     import plain_gpt2 as plain
 
-    V = 1000
-    logits = rnd(12, V, scale=2.0, seed=11)
+    logits = rnd(14, V, scale=2.0, seed=11)
     logits[5, 100:140] = 3.0  # many ties at the top-k boundary
+    logits[12, :] = 0.25  # all equal: ties everywhere
     params = [(0.0, 0, 1.0), (1.0, 0, 1.0), (0.8, 0, 1.0), (0.8, 40, 0.95), (1.3, 5, 1.0), (0.7, 20, 1.0), (1.0, 0, 0.5),
-              (1.0, 0, 0.05), (0.5, 1, 1.0), (2.0, 999, 0.9), (1.0, 40, 0.0), (0.8, 0, 0.999)]
+              (1.0, 0, 0.05), (0.5, 1, 1.0), (2.0, 999, 0.9), (1.0, 40, 0.0), (0.8, 0, 0.999), (1.0, 64, 0.7), (0.9, 65, 0.9)]
     cpu = logits.cpu().numpy()
     for trial in range(6):
-        u = [plain.uniform(7 + trial, r) for r in range(12)]
-        out = torch.empty(12, dtype=torch.int32, device=DEV)
+        u = [plain.uniform(7 + trial, r) for r in range(len(params))]
+        out = torch.empty(len(params), dtype=torch.int32, device=DEV)
         ops.sample(out, logits,
                    torch.tensor([p[0] for p in params], dtype=torch.float32, device=DEV),
                    torch.tensor([p[1] for p in params], dtype=torch.int32, device=DEV),
@@ -428,7 +431,7 @@ def test_sampler_against_the_plain_sampler(ops):
             want = plain.sample(probs, u[r])
             if got[r] != want:
                 cdf = np.cumsum(probs)
-                assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (r, params[r], got[r], want)
+                assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, params[r], got[r], want)
 
 
 @pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl5", "auto"])
