@@ -74,6 +74,64 @@ gemm_simple_kernel(OutT* __restrict__ out, int64_t ldo, const T* __restrict__ a,
     }
 }
 
+// The same product for steps of few rows (decoding): a thread per output element walks K in
+// the same order with the same fused multiply-adds as the tiled kernel, so a row's result has
+// the same bits whichever of the two computed it. A wave takes 64 output features of one row;
+// rows of `w` are streamed 16 bytes a lane, the row of `a` through scalar loads.
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int EPI, bool EXACT>
+__global__ void __launch_bounds__(64)
+gemm_rowwise_f32_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ a, int64_t lda,
+                        const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ residual,
+                        int64_t ldr, int N, int K, int vec) {
+    const int n = blockIdx.x * 64 + threadIdx.x, m = blockIdx.y;
+    const float* wr = w + static_cast<int64_t>(min(n, N - 1)) * K;
+    const float* ar = a + static_cast<int64_t>(m) * lda;
+    float acc = 0.0f;
+    int k = 0;
+    if (vec) {
+#pragma unroll 8
+        for (; k + 4 <= K; k += 4) {
+            const f32x4_t wv = *reinterpret_cast<const f32x4_t*>(wr + k);
+            const f32x4_t av = *reinterpret_cast<const f32x4_t*>(ar + k);
+            acc = fmaf(av[0], wv[0], acc);
+            acc = fmaf(av[1], wv[1], acc);
+            acc = fmaf(av[2], wv[2], acc);
+            acc = fmaf(av[3], wv[3], acc);
+        }
+    }
+    for (; k < K; ++k) acc = fmaf(ar[k], wr[k], acc);
+    if (n >= N) return;
+    float v = acc;
+    if (bias != nullptr) v += bias[n];
+    if constexpr (EPI == kEpiGeluTanh) v = gelu_tanh(v);
+    if constexpr (EPI == kEpiGeluErf) v = EXACT ? gelu_erf_exact(v) : gelu_erf_fast(v);
+    if constexpr (EPI == kEpiResidual) {
+        residual[static_cast<int64_t>(m) * ldr + n] += v;
+    } else {
+        out[static_cast<int64_t>(m) * ldo + n] = v;
+    }
+}
+
+constexpr int kRowwiseRows = 16;  // steps of at most this many rows take the row-wise kernel
+
+int launch_rowwise_f32(float* out, int64_t ldo, const float* a, int64_t lda, const float* w, const float* bias,
+                       float* residual, int64_t ldr, int M, int N, int K, int epi, hipStream_t stream) {
+    const dim3 grid((N + 63) / 64, M);
+    const int vec = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && lda % 4 == 0 && K % 4 == 0;
+#define LIYAB_GO(E) gemm_rowwise_f32_kernel<E, true><<<grid, 64, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, N, K, vec)
+    switch (epi) {
+        case kEpiNone: LIYAB_GO(kEpiNone); break;
+        case kEpiGeluTanh: LIYAB_GO(kEpiGeluTanh); break;
+        case kEpiGeluErf: LIYAB_GO(kEpiGeluErf); break;
+        case kEpiResidual: LIYAB_GO(kEpiResidual); break;
+        default: return fail(1, "gemm: unknown epilogue %d", epi);
+    }
+#undef LIYAB_GO
+    return check_launch("gemm_rowwise");
+}
+
 template <typename T, typename OutT, bool EXACT>
 int launch_simple(void* out, int64_t ldo, const void* a, int64_t lda, const void* w, const float* bias,
                   float* residual, int64_t ldr, int M, int N, int K, int epi, hipStream_t stream) {
@@ -114,6 +172,9 @@ extern "C" int liyab_gemm_simple(void* out, int out_dtype, int64_t ldo, const vo
     if (M == 0) return 0;
     if (dtype == kF32) {
         LIYAB_REQUIRE(epi == kEpiResidual || out_dtype == kF32, "gemm: 32-bit operands give a 32-bit output");
+        if (M <= kRowwiseRows)
+            return launch_rowwise_f32(static_cast<float*>(out), ldo, static_cast<const float*>(a), lda, static_cast<const float*>(w),
+                                      bias, residual, ldr, M, N, K, epi, stream);
         return launch_simple<float, float, true>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K, epi, stream);
     }
     if (dtype == kBF16) {
