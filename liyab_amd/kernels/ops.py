@@ -30,8 +30,27 @@ def dtype_code(dt: torch.dtype) -> int:
     raise KernelError(f"the kernels take float32 or bfloat16, not {dt}")
 
 
+_pinned_stream: Optional[int] = None
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _pinned_stream if _pinned_stream is not None else torch.cuda.current_stream().cuda_stream
+
+
+class on_current_stream:
+    """Within this context every launch goes to the stream that was current on entry, looked
+    up once instead of at every call (a model step makes a couple of hundred launches)."""
+
+    def __enter__(self):
+        global _pinned_stream
+        self._before = _pinned_stream
+        _pinned_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self._before
+        return False
 
 
 def _dev(t: torch.Tensor, what: str) -> None:

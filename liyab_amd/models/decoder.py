@@ -16,6 +16,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from ..cache.pages import KVSpec, StateSpec
+from ..kernels import ops
 from ..config.plan import ModelPlan
 from ..parts.base import StepContext
 from ..parts.registry import build_part, find_part
@@ -70,6 +71,10 @@ class DecoderModel:
     def forward(self, ctx: StepContext, storage) -> Optional[torch.Tensor]:
         """Runs the step's tokens through every layer; returns float32 logits
         [n_logit_rows, vocab] or None when no row is wanted."""
+        with ops.on_current_stream():
+            return self._forward(ctx, storage)
+
+    def _forward(self, ctx: StepContext, storage) -> Optional[torch.Tensor]:
         x = ctx.workspace.get("residual", (ctx.n_tokens, self.width), torch.float32)
         fused = self.residual_position.fused_table() if self.residual_position is not None else None
         self.embedding.forward(ctx, x, position_table=fused)
