@@ -266,7 +266,8 @@ using namespace liyab;
 
 // tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep and four waves; 6 = 64x64
 // with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages (deeper rings
-// measured slower: their LDS leaves one workgroup a compute unit, and 288 tiles then take two rounds), 9 = 128x64
+// measured slower: their LDS leaves one workgroup a compute unit, and 288 tiles then take two rounds), 9 = 128x64;
+// 13 = 128x128 two stages on four waves
 // (0 = chosen from the shape).
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
@@ -280,8 +281,9 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
     if (int rc = check_epilogue(epi, M, N)) return rc;
     // measured on {256..2048} x {768, 2304, 3072} x {768, 3072}: 64 x 64 tiles, three workgroups a
     // CU, win or tie nearly everywhere; a long K likes one more stage in flight; a large output
-    // (2,048 x 2,304 and up) likes 128 x 128 tiles on eight waves, two stages deep
-    if (tile == 0) tile = K >= 2048 ? 6 : (static_cast<long>(M) * N >= 2048L * 2048L ? 8 : 2);
+    // (2,048 x 2,304 and up) likes 128 x 128 tiles, two stages deep, on four waves of 64 x 64 each:
+    // a fragment read from LDS then feeds two products (LDS bandwidth is what the loop runs out of)
+    if (tile == 0) tile = K >= 2048 ? 6 : (static_cast<long>(M) * N >= 2048L * 2048L ? 13 : 2);
     switch (tile) {
         case 1: return launch_dl<128, 128, 3>(a, lda, w, M, N, K, epi, stream);
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
@@ -291,6 +293,7 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
         case 7: return launch_dl<128, 128, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 9: return launch_dl<128, 64, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
+        case 13: return launch_dl<128, 128, 2, 2, 2>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }
