@@ -369,3 +369,41 @@ def test_overlapped_steps_give_the_same_tokens(dtype, model_dirs):
             assert engine.core.manager.pages_in_use() == 0
             engine.core.manager.check()
         assert results[False][:2] == results[True][:2]
+
+
+# ---------------------------------------------------------------------------
+# drawn geometries
+# ---------------------------------------------------------------------------
+def drawn_config(seed):
+    """A GPT-2 configuration drawn from the seed: any number of heads, head sizes in steps of
+    16 up to 256, a feed-forward width and a vocabulary that are multiples of nothing."""
+    rng = np.random.default_rng(1000 + seed)
+    hd = int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 192, 256]))
+    n_head = int(rng.integers(1, 8 if hd <= 64 else 4))
+    return {"architectures": ["GPT2LMHeadModel"], "n_layer": int(rng.integers(1, 4)), "n_embd": hd * n_head, "n_head": n_head,
+            "n_inner": int(rng.integers(17, 400)), "vocab_size": int(rng.integers(50, 1500)),
+            "n_positions": int(rng.integers(150, 330)), "layer_norm_epsilon": float(rng.choice([1e-5, 1e-6, 3e-4])),
+            "activation_function": str(rng.choice(["gelu_new", "gelu"])),
+            "scale_attn_by_inverse_layer_idx": bool(rng.integers(0, 2)), "scale_attn_weights": bool(rng.integers(0, 4) > 0)}
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
+    """Ten drawn configurations, each whole and in a mixed schedule, in both precisions: a size
+    the kernels mishandle shows as a wrong logit (or a refusal), never passes silently."""
+    from liyab_amd.weights import write_random_model
+
+    cfg = drawn_config(seed)
+    write_random_model(str(tmp_path), cfg, 200 + seed)
+    config, tensors = plain.read_model(str(tmp_path))
+    P, V = cfg["n_positions"], cfg["vocab_size"]
+    reqs = {f"g{i}": tt.random_tokens(300 + 10 * seed + i, n, V) for i, n in enumerate([P, 41, 1 + seed, 130])}
+    for dtype in DTYPES:
+        weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+        refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+        for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=seed, decode_tail=5))):
+            core = make_core(str(tmp_path), dtype, tt.max_live_tokens(steps))
+            got = tt.run_schedule(core, steps)
+            tt.check_against_plain(got, reqs, refs, TOL[dtype], f"{cfg} {label} {dtype}")
+            core.manager.check()
+            del core
