@@ -6,9 +6,10 @@
 // wave order. With v_mfma_f32_16x16x32_bf16 the weights are the first
 // operand (16 rows) and the tokens the second (16), so an accumulator is a
 // transposed output tile. A lane holds 8 consecutive k of its row per
-// instruction; here each lane reads a run of 16 consecutive k (32 bytes) and
-// feeds two instructions, and both operands use the same assignment of k to
-// (lane group, instruction), which a dot product does not mind. Weights are
+// instruction, the four lane groups of a row 32 consecutive k: one load
+// instruction reads 64 contiguous bytes of each of 16 rows (whole sectors;
+// a lane reading 32 contiguous bytes in two instructions touched every
+// sector twice). Weights are
 // read once, straight from global memory into registers, 16 bytes a lane,
 // one trip ahead of the multiplies; the tokens' rows come from L2 (every
 // workgroup reads all of them: few, wide tiles of N would starve most CUs).
@@ -44,7 +45,7 @@ struct LnParams {
 template <typename OutT, bool LN, int MT, int NT, int MAXW, int MAXV = 32>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
-                   EpiParams epi, LnParams ln) {
+                   EpiParams epi, LnParams ln, int part_k, int64_t part_stride) {
     constexpr int UPT = (MT * NT == 1) ? 2 : 1;  // units of 64 k per trip
     constexpr int TILES = MT * NT;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -57,26 +58,42 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     const int i = lane % 16, g = lane / 16;
     const int n0 = blockIdx.x * 16 * NT;
     const int m0 = blockIdx.y * 16 * MT;  // this workgroup's rows: [m0, m0 + 16 MT) of M
-    const int units = (K + 63) / 64;
+    // K may be cut into parts of part_k (a multiple of 64) over blockIdx.z, each part's sums
+    // going to its own plane of the output; this workgroup's k are [k_begin, k_end)
+    const int k_begin = blockIdx.z * part_k, k_end = min(K, k_begin + part_k);
+    const int units = (k_end - k_begin + 63) / 64;
+    if (gridDim.z > 1) epi.out = static_cast<float*>(epi.out) + blockIdx.z * part_stride;
     const u32x4 zero = {0, 0, 0, 0};
     const bf16_t* wrow[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) wrow[t] = w + static_cast<int64_t>(min(n0 + 16 * t + i, N - 1)) * K;
 
-    // unit u covers k in [64 u, 64 u + 64); this lane's run starts at 64 u + 16 g
+    // 8 consecutive k of a row; past the end it is the last piece, read and dropped: a load under
+    // a branch would make the compiler wait for every load in flight, the next trip's too
+    auto piece = [&](const bf16_t* row, int k) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(row + min(k, k_end - 8));
+        return k < k_end ? v : zero;
+    };
+    // unit u covers k in k_begin + [64 u, 64 u + 64): two instructions of 32 k, this lane's 8 start at 8 g
     auto load_w = [&](int u0, Frag (&f)[UPT][NT][2]) {
 #pragma unroll
         for (int p = 0; p < UPT; ++p) {
-            const int u = u0 + p * ksplit, k = u * 64 + g * 16;
+            const int k = k_begin + (u0 + p) * 64 + g * 8;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                f[p][t][0].u = (u < units && k < K) ? *reinterpret_cast<const u32x4*>(wrow[t] + k) : zero;
-                f[p][t][1].u = (u < units && k + 8 < K) ? *reinterpret_cast<const u32x4*>(wrow[t] + k + 8) : zero;
+                f[p][t][0].u = piece(wrow[t], k);
+                f[p][t][1].u = piece(wrow[t], k + 32);
             }
         }
     };
     Frag wc[UPT][NT][2];
-    load_w(wave, wc);  // issued before the norm's prologue, so the two overlap
+    load_w(wave * UPT, wc);  // issued before the norm's prologue, so the two overlap
+    // what the epilogue will read for this thread's first output (bias, residual) is asked for
+    // now: after the sums it would be one more trip to memory on the critical path
+    const int e_m = m0 + 16 * ((tid / 256) / NT) + (tid % 256) / 16, e_n = n0 + 16 * ((tid / 256) % NT) + tid % 16;
+    const bool e_mine = tid < TILES * 256 && e_m < M && e_n < N;
+    const float e_bias = (e_mine && epi.bias != nullptr) ? epi.bias[e_n] : 0.0f;
+    const float e_res = (e_mine && epi.mode == kEpiResidual) ? epi.residual[static_cast<int64_t>(e_m) * epi.ldr + e_n] : 0.0f;
     __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
 
     const bf16_t* arow[MT];
@@ -119,6 +136,21 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
 #pragma unroll
         for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(m0 + 16 * s + i, M - 1)) * lda;
     }
+    // the tokens' fragments travel with the weights', a trip ahead: asked for after the next
+    // trip's weights they would make every trip wait for those too (loads return in order)
+    auto load_x = [&](int u0, Frag (&x)[UPT][MT][2]) {
+#pragma unroll
+        for (int p = 0; p < UPT; ++p) {
+            const int k = k_begin + (u0 + p) * 64 + g * 8;
+#pragma unroll
+            for (int s = 0; s < MT; ++s) {
+                x[p][s][0].u = piece(arow[s], k);
+                x[p][s][1].u = piece(arow[s], k + 32);
+            }
+        }
+    };
+    Frag xc[UPT][MT][2];
+    load_x(wave * UPT, xc);
 
     floatx4 acc[MT][NT];
 #pragma unroll
@@ -126,34 +158,40 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[s][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    for (int u0 = wave; u0 < units; u0 += UPT * ksplit) {
-        Frag wn[UPT][NT][2];
-        load_w(u0 + UPT * ksplit, wn);
+    auto multiply = [&]() {
 #pragma unroll
-        for (int p = 0; p < UPT; ++p) {
-            const int u = u0 + p * ksplit, k = u * 64 + g * 16;
-            Frag x[MT][2];
-#pragma unroll
-            for (int s = 0; s < MT; ++s) {
-                x[s][0].u = (u < units && k < K) ? *reinterpret_cast<const u32x4*>(arow[s] + k) : zero;
-                x[s][1].u = (u < units && k + 8 < K) ? *reinterpret_cast<const u32x4*>(arow[s] + k + 8) : zero;
-            }
+        for (int p = 0; p < UPT; ++p)
 #pragma unroll
             for (int s = 0; s < MT; ++s)
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, x[s][0].v, acc[s][t], 0, 0, 0);
-                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, x[s][1].v, acc[s][t], 0, 0, 0);
+                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, xc[p][s][0].v, acc[s][t], 0, 0, 0);
+                    acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, xc[p][s][1].v, acc[s][t], 0, 0, 0);
                 }
-        }
+    };
+    // every trip but the last asks for the next trip's operands before it multiplies; the last
+    // one is peeled off, so no trip asks for (and then waits for) operands nobody uses
+    int u0 = wave * UPT;
+    for (; u0 + UPT * ksplit < units; u0 += UPT * ksplit) {
+        Frag wn[UPT][NT][2], xn[UPT][MT][2];
+        load_w(u0 + UPT * ksplit, wn);
+        load_x(u0 + UPT * ksplit, xn);
+        multiply();
 #pragma unroll
-        for (int p = 0; p < UPT; ++p)
+        for (int p = 0; p < UPT; ++p) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 wc[p][t][0] = wn[p][t][0];
                 wc[p][t][1] = wn[p][t][1];
             }
+#pragma unroll
+            for (int s = 0; s < MT; ++s) {
+                xc[p][s][0] = xn[p][s][0];
+                xc[p][s][1] = xn[p][s][1];
+            }
+        }
     }
+    multiply();  // a wave past the end of K holds zeros
     // acc[s][t][r] = partial C^T[n = 16 t + 4 g + r][m = 16 s + i]; kept [tile][m][n] per wave
 #pragma unroll
     for (int s = 0; s < MT; ++s)
@@ -167,14 +205,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
         const int m = m0 + 16 * s + (e % 256) / 16, n = n0 + 16 * t + e % 16;
         float v = 0.0f;
         for (int q = 0; q < ksplit; ++q) v += red[q * TILES * 256 + e];
-        if (m < M && n < N) epilogue_store<OutT>(epi, m, n, v);
+        if (m >= M || n >= N) continue;
+        if (e != tid) epilogue_store<OutT>(epi, m, n, v);
+        else if (epi.mode == kEpiResidual) epi.residual[static_cast<int64_t>(m) * epi.ldr + n] = e_res + (v + e_bias);
+        else epilogue_store_biased<OutT>(epi, m, n, v + e_bias);
     }
 }
 
 template <bool LN, int MT, int NT, int MAXW, int MAXV = 32>
 int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, const EpiParams& epi,
-                  const LnParams& ln, hipStream_t stream) {
-    const dim3 grid((N + 16 * NT - 1) / (16 * NT), LN ? 1 : (M + 16 * MT - 1) / (16 * MT));
+                  const LnParams& ln, int kparts, int64_t part_stride, hipStream_t stream) {
+    // K in kparts parts, each a whole number of units of 64 and none of them empty (the caller's check)
+    const int part_k = ((K + 63) / 64 + kparts - 1) / kparts * 64;
+    const dim3 grid((N + 16 * NT - 1) / (16 * NT), LN ? 1 : (M + 16 * MT - 1) / (16 * MT), kparts);
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
     if (ksplit > MAXW) ksplit = MAXW;
@@ -188,7 +231,7 @@ int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             ready = true;
         }
-        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln);
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln, part_k, part_stride);
     } else {
         auto kern = gemm_skinny_kernel<bf16_t, LN, MT, NT, MAXW, MAXV>;
         static bool ready = false;
@@ -196,13 +239,14 @@ int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             ready = true;
         }
-        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln);
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln, part_k, part_stride);
     }
     return check_launch("gemm_skinny");
 }
 
 static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide, int mtile,
-                           const EpiParams& epi, const LnParams& ln, hipStream_t stream) {
+                           const EpiParams& epi, const LnParams& ln, hipStream_t stream, int kparts = 1,
+                           int64_t part_stride = 0) {
     // tiles of 16 rows a workgroup: all of M in one workgroup reads the weights once; with few
     // output features that leaves most of the chip idle, and the rows are spread over workgroups
     // instead (the weights then come from L2 after their first reading)
@@ -216,7 +260,8 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
     const int nt = wide ? 4 : 1;
     if (ksplit == 0) {
         // enough waves to cover the chip several times over, each with at least 128 k
-        const int tiles = ((N + 16 * nt - 1) / (16 * nt)) * ((M + 16 * mt - 1) / (16 * mt)), units = (K + 63) / 64;
+        const int tiles = ((N + 16 * nt - 1) / (16 * nt)) * ((M + 16 * mt - 1) / (16 * mt)) * kparts;
+        const int units = ((K + 63) / 64 + kparts - 1) / kparts;
         ksplit = 1;
         while (ksplit < 16 && tiles * ksplit < 2048 && units / (ksplit * 2) >= (mt * nt == 1 ? 2 : 1)) ksplit *= 2;
         // a folded norm takes a wave per row: as many waves as rows, so the rows go side by side
@@ -225,17 +270,17 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
     LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || ksplit == 4 || ksplit == 8 || ksplit == 16,
                   "gemm_skinny: ksplit %d is not 1, 2, 4, 8 or 16", ksplit);
     if (ln.x != nullptr) {  // 8 waves: registers for a row's values
-        if (K <= 1024) return launch_skinny<true, 1, 1, 8, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
-        return launch_skinny<true, 1, 1, 8, 32>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+        if (K <= 1024) return launch_skinny<true, 1, 1, 8, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+        return launch_skinny<true, 1, 1, 8, 32>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
     }
     if (nt == 1) {
-        if (mt == 1) return launch_skinny<false, 1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
-        if (mt == 2) return launch_skinny<false, 2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
-        return launch_skinny<false, 4, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+        if (mt == 1) return launch_skinny<false, 1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+        if (mt == 2) return launch_skinny<false, 2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+        return launch_skinny<false, 4, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
     }
-    if (mt == 1) return launch_skinny<false, 1, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
-    if (mt == 2) return launch_skinny<false, 2, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
-    return launch_skinny<false, 4, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, stream);
+    if (mt == 1) return launch_skinny<false, 1, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+    if (mt == 2) return launch_skinny<false, 2, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+    return launch_skinny<false, 4, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
 }
 
 }  // namespace liyab
@@ -257,6 +302,33 @@ extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int 
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
     return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, mtile, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream);
+}
+
+// The product's sums over `kparts` parts of K, one plane [M, N] of 32-bit sums a part:
+// parts[p * part_stride + m * N + n] = sum over the p-th part of K of a[m, k] w[n, k], no bias.
+// For a product with few output features and a long K: cut over K it fills the chip, and
+// whoever reads the result next adds the planes up in their order (the norm kernel does).
+// Every part holds at least one unit of 64 k: (kparts - 1) * ceil(ceil(K / 64) / kparts) * 64 < K.
+extern "C" int liyab_gemm_skinny_parts(const void* a, int64_t lda, const void* w, int M, int N, int K, int kparts,
+                                       int ksplit, float* parts, int64_t part_stride, hipStream_t stream) {
+    LIYAB_REQUIRE(a && w && parts, "gemm: null operand");
+    LIYAB_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_parts: bad sizes M=%d (at most 64) N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(K % 8 == 0 && lda % 8 == 0 && lda >= K, "gemm_skinny_parts: K %d and lda %lld must be multiples of 8", K,
+                  static_cast<long long>(lda));
+    LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0,
+                  "gemm_skinny_parts: operands must be 16-byte aligned");
+    const int units = (K + 63) / 64;
+    LIYAB_REQUIRE(kparts >= 1 && kparts <= 16 && (kparts - 1) * ((units + kparts - 1) / kparts) < units,
+                  "gemm_skinny_parts: K = %d does not cut into %d parts of whole units of 64", K, kparts);
+    LIYAB_REQUIRE(part_stride >= static_cast<int64_t>(M) * N, "gemm_skinny_parts: planes of %lld overlap", static_cast<long long>(part_stride));
+    if (M == 0) return 0;
+    EpiParams epi{};
+    epi.mode = kEpiNone;
+    epi.out_dtype = kF32;
+    epi.out = parts;
+    epi.ldo = N;
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, 0, 1, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream,
+                           kparts, part_stride);
 }
 
 // The same product with a LayerNorm folded in: the first operand is LayerNorm(x[rows[m] or m])

@@ -158,9 +158,24 @@ def add_rows_(x: torch.Tensor, table: torch.Tensor, rows: torch.Tensor) -> None:
     _lib.call("liyab_add_rows", x.data_ptr(), table.data_ptr(), dtype_code(table.dtype), rows.data_ptr(), n, d, _stream())
 
 
+def _part_sums(x: torch.Tensor, sums, what: str):
+    """Checks sums still to be added to the rows of x: (planes float32 [parts, rows of x, d],
+    bias float32 [d] or None). Returns what the launchers take."""
+    planes, bias = sums
+    _dev(planes, "partial sums")
+    if (planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != tuple(x.shape) or not planes.is_contiguous()
+            or not 1 <= planes.shape[0] <= 16):
+        raise KernelError(f"{what}: partial sums must be contiguous float32 [1..16, {x.shape[0]}, {x.shape[1]}], got {tuple(planes.shape)}")
+    _f32vec(bias, "bias of the partial sums", x.shape[1])
+    return planes.data_ptr(), planes.shape[0], planes.stride(0), _ptr(bias)
+
+
 def layernorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
-              eps: float, rows: Optional[torch.Tensor] = None) -> None:
-    """out[r] = LayerNorm(x[rows[r]] or x[r]); x float32 [*, d], out [n, d] float32 or bfloat16."""
+              eps: float, rows: Optional[torch.Tensor] = None, sums=None) -> None:
+    """out[r] = LayerNorm(x[rows[r]] or x[r]); x float32 [*, d], out [n, d] float32 or bfloat16.
+    `sums` = (planes [parts, rows of x, d], bias [d] or None) are added to the rows first, bias
+    then planes in their order; without `rows`, x holds the sums afterwards (with `rows` it
+    must not be read again)."""
     _dev(out, "out")
     _dev(x, "x")
     n, d = out.shape
@@ -172,8 +187,25 @@ def layernorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor]
         _i32(rows, "rows", n)
     elif x.shape[0] < n:
         raise KernelError("layernorm: fewer input rows than output rows")
-    _lib.call("liyab_layernorm", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
-              _ptr(rows), n, d, float(eps), _stream())
+    if sums is None:
+        _lib.call("liyab_layernorm", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
+                  _ptr(rows), n, d, float(eps), _stream())
+        return
+    if rows is None and x.shape[0] != n:
+        raise KernelError("layernorm: with sums to add, every row of x is normalised")
+    planes, n_parts, stride, pbias = _part_sums(x, sums, "layernorm")
+    _lib.call("liyab_layernorm_parts", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
+              _ptr(rows), n, d, float(eps), planes, n_parts, stride, pbias, x.shape[0], _stream())
+
+
+def add_parts(x: torch.Tensor, sums) -> None:
+    """x += bias + planes[0] + planes[1] + ... for `sums` = (planes, bias), in the order the
+    norm kernel adds them."""
+    _dev(x, "x")
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("add_parts: x must be contiguous float32 [rows, d]")
+    planes, n_parts, stride, pbias = _part_sums(x, sums, "add_parts")
+    _lib.call("liyab_add_parts", x.data_ptr(), x.shape[0], x.shape[1], planes, n_parts, stride, pbias, _stream())
 
 
 def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
@@ -360,6 +392,36 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
         raise KernelError(f"gemm_skinny: {M} rows; it takes at most 64")
     e = _epilogue(a, w, bias, out, residual, epilogue, kv)
     _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, wide, mtile, ctypes.byref(e), _stream())
+
+
+def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, ksplit: int = 0) -> None:
+    """planes[p] = a . w^T summed over the p-th of planes.shape[0] parts of K (no bias): the
+    weight-streaming product cut over K, for few output features and a long K. a [M <= 64, K]
+    and w [N, K] bfloat16, planes float32 [parts, M, N]."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    _dev(planes, "planes")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_skinny_parts: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
+    if planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != (M, w.shape[0]) or not planes.is_contiguous():
+        raise KernelError(f"gemm_skinny_parts: planes must be contiguous float32 [parts, {M}, {w.shape[0]}], got {tuple(planes.shape)}")
+    _lib.call("liyab_gemm_skinny_parts", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, planes.shape[0], ksplit,
+              planes.data_ptr(), planes.stride(0), _stream())
+
+
+def k_parts(M: int, N: int, K: int) -> int:
+    """Into how many parts of K the weight-streaming product is best cut (1: not at all). With
+    few output features a product fills a fraction of the chip's compute units, and a long K
+    then streams through those few; cut over K it covers the chip. Measured at 8 rows:
+    3,072 -> 768 takes 7.0 us whole and 4.3 us in four parts; 6,400 -> 1,600 12.6 and 8 us."""
+    if M > 16 or K % 8 != 0 or K < 2048:
+        return 1
+    strips, units = (N + 15) // 16, (K + 63) // 64
+    parts = 1
+    while parts < 4 and strips * parts * 2 <= 256 and units // (parts * 2) >= 8:
+        parts *= 2
+    return parts
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,

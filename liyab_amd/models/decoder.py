@@ -80,15 +80,28 @@ class DecoderModel:
         self.embedding.forward(ctx, x, position_table=fused)
         if self.residual_position is not None and fused is None:
             self.residual_position.add(ctx, x)
+        pending = None  # sums a layer has computed for x and left for the next reader of x to add
         for e in self.order:
-            self.blocks[e.layer].forward(x, ctx, storage.layer(e.cache_layer), storage.state(e.cache_layer),
-                                         writes_cache=e.writes_cache)
+            block = self.blocks[e.layer]
+            args = (x, ctx, storage.layer(e.cache_layer), storage.state(e.cache_layer))
+            if getattr(block, "takes_pending", False):
+                pending = block.forward(*args, writes_cache=e.writes_cache, pending=pending)
+            else:
+                if pending is not None:
+                    pending.settle(x)
+                    pending = None
+                block.forward(*args, writes_cache=e.writes_cache)
         if ctx.n_logit_rows == 0:
-            return None
+            return None  # nobody reads x again: pending sums are dropped
         if self.final_norm is not None:
             norm = self.final_norm
             kw = dict(rows=ctx.logit_rows, n_rows=ctx.n_logit_rows, name="head_in")
-            h = norm.lazy(x, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(x, ctx, **kw)
+            if pending is not None and getattr(norm, "takes_sums", False):
+                h = norm.forward(x, ctx, sums=pending.sums, **kw)
+            else:
+                if pending is not None:
+                    pending.settle(x)
+                h = norm.lazy(x, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(x, ctx, **kw)
         else:
             raise NotImplementedError("a model without a final norm is not implemented")
         return self.head.forward(h, ctx)

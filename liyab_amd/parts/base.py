@@ -30,6 +30,25 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 
+class PendingSums:
+    """What a part has computed for the residual stream but not added to it yet: planes of
+    partial sums [parts, tokens, width] (float32) and a bias [width] or None. Whoever reads
+    the stream next adds them first, bias then planes in their order: a norm that can does
+    so as it loads its rows (`takes_sums`), anything else through `settle`."""
+
+    def __init__(self, planes, bias):
+        self.planes, self.bias = planes, bias
+
+    @property
+    def sums(self):
+        return (self.planes, self.bias)
+
+    def settle(self, x) -> None:
+        from ..kernels import ops
+
+        ops.add_parts(x, self.sums)
+
+
 class Workspace:
     """Named scratch buffers that keep their addresses from step to step."""
 

@@ -16,12 +16,25 @@ class PreNormBlock:
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True) -> None:
-        h = self._normed(self.norm_mixer, x, ctx)
+    takes_pending = True  # forward(..., pending=) takes sums the stream still lacks and may return such
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True, pending=None):
+        """`pending`: PendingSums that x still lacks (the previous layer's), added by this
+        layer's first norm as it reads x. Returns this layer's own, or None."""
+        if pending is not None and getattr(self.norm_mixer, "takes_sums", False):
+            h = self.norm_mixer.forward(x, ctx, sums=pending.sums)
+        else:
+            if pending is not None:
+                pending.settle(x)
+            h = self._normed(self.norm_mixer, x, ctx)
         self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
-        if self.ffn is not None:
-            h = self._normed(self.norm_ffn, x, ctx)
-            self.ffn.forward(h, ctx, x)
+        if self.ffn is None:
+            return None
+        h = self._normed(self.norm_ffn, x, ctx)
+        if getattr(self.ffn, "defers", False):
+            return self.ffn.forward(h, ctx, x, defer=True)
+        self.ffn.forward(h, ctx, x)
+        return None
 
     @staticmethod
     def _normed(norm, x, ctx):

@@ -4,7 +4,8 @@ from __future__ import annotations
 
 import torch
 
-from .base import StepContext
+from ..kernels import ops
+from .base import PendingSums, StepContext
 from .linear import linear
 from .registry import register_ffn
 
@@ -26,10 +27,21 @@ class DenseFFN:
         self.down_weight = store.fetch(t["down_weight"], (self.width, self.inner), "matrix")
         self.down_bias = store.fetch(t["down_bias"], (self.width,), "vector") if "down_bias" in t else None
 
-    def forward(self, h, ctx: StepContext, residual: torch.Tensor) -> None:
+    defers = True  # forward(..., defer=True) may hand its result back as PendingSums
+
+    def forward(self, h, ctx: StepContext, residual: torch.Tensor, defer: bool = False):
+        """Adds the feed-forward's output into `residual`. With `defer`, and where the second
+        product runs faster cut over its inner dimension, the parts' sums come back as
+        PendingSums instead, for the next reader of the residual stream to add."""
         inner = ctx.workspace.get("ffn_inner", (h.shape[0], self.inner), self.dtype)
         linear(h, self.up_weight, self.up_bias, out=inner, activation=self.activation)
+        parts = ops.k_parts(h.shape[0], self.width, self.inner) if defer and self.dtype == torch.bfloat16 else 1
+        if parts > 1:
+            planes = ctx.workspace.get("ffn_parts", (parts, h.shape[0], self.width), torch.float32)
+            ops.gemm_skinny_parts(inner, self.down_weight, planes)
+            return PendingSums(planes, self.down_bias)
         linear(inner, self.down_weight, self.down_bias, residual=residual)
+        return None
 
 
 register_ffn("dense_ffn", DenseFFN)

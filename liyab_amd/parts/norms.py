@@ -55,16 +55,19 @@ class LayerNorm:
         self.bias = store.fetch(b, (self.width,), "vector") if b is not None else None
 
     fusable = "layernorm"  # product kernels know how to fold this norm into their operand
+    takes_sums = True  # forward(..., sums=) adds pending partial sums to the rows as it loads them
 
     def lazy(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
              n_rows: Optional[int] = None, name: str = "normed") -> Normed:
         return Normed(self, x, ctx, rows, n_rows, name)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
-                n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:
+                n_rows: Optional[int] = None, name: str = "normed", sums=None) -> torch.Tensor:
+        """`sums`: a PendingSums' (planes, bias), added to x's rows first. Without `rows` x
+        holds the sums afterwards; with `rows` it does not and must not be read again."""
         n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
         out = ctx.workspace.get(name, (n, self.width), self.dtype)
-        ops.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows)
+        ops.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows, sums=sums)
         return out
 
 

@@ -70,6 +70,58 @@ def test_layernorm(ops, out_dtype, n, d, eps):
     assert (o1 - o2).abs().max() > 1e-2
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,d,parts,with_bias", [(1, 64, 1, True), (9, 96, 4, False), (16, 768, 4, True), (5, 1600, 2, True),
+                                                 (3, 777, 3, True), (7, 2052, 2, False), (6, 200, 16, True)])
+def test_layernorm_adds_pending_sums(ops, out_dtype, n, d, parts, with_bias):
+    """Rows that still lack a product's partial sums: the norm adds bias and planes as it loads
+    the rows and writes the sums back; over gathered rows it leaves x alone (widths that need
+    the general kernel get the sums in a pass of their own, in place); add_parts alone does
+    the same sum."""
+    tol = 1e-6 if out_dtype == torch.float32 else 5e-3
+    x = rnd(n, d, scale=3.0) + 1.5
+    planes = rnd(parts, n, d, seed=4, scale=0.7)
+    pbias = rnd(d, seed=5) if with_bias else None
+    w, b = rnd(d, seed=2) + 1.0, rnd(d, seed=3)
+    total = x.double() + planes.double().sum(0) + (pbias.double() if with_bias else 0)
+    want = torch.nn.functional.layer_norm(total, (d,), w.double(), b.double(), 1e-5)
+    out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    x1 = x.clone()
+    ops.layernorm(out, x1, w, b, 1e-5, sums=(planes, pbias))
+    close(out, want, tol, "layernorm with sums")
+    close(x1, total, 1e-6, "rows written back")
+    x2 = x.clone()
+    ops.add_parts(x2, (planes, pbias))
+    assert torch.equal(x1, x2)  # the same order of additions
+    rows = torch.tensor([(i * 3) % n for i in range(n + 2)], dtype=torch.int32, device=DEV)  # names rows twice
+    out = torch.empty(n + 2, d, dtype=out_dtype, device=DEV)
+    x3 = x.clone()
+    ops.layernorm(out, x3, w, b, 1e-5, rows=rows, sums=(planes, pbias))
+    close(out, want[rows.long()], tol, "gathered layernorm with sums")
+    wave_kernel = d % 4 == 0 and d <= 2048
+    assert torch.equal(x3, x if wave_kernel else x2)
+    with pytest.raises(Exception, match="partial sums"):
+        ops.layernorm(out[:n], x, w, b, 1e-5, sums=(planes[:, :, :-1], pbias))
+
+
+@pytest.mark.parametrize("M,N,K,parts", [(1, 64, 128, 2), (8, 768, 3072, 4), (16, 100, 200, 2), (5, 1600, 6400, 2), (40, 50, 448, 7),
+                                         (64, 264, 1600, 3), (3, 40, 64, 1), (11, 130, 1032, 4)])
+def test_gemm_skinny_parts(ops, M, N, K, parts):
+    """The product cut over K: plane p holds the sums over the p-th part of K (whole units of
+    64, the last one shorter), no bias; the planes add up to the product."""
+    a, w = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16)
+    planes = torch.full((parts, M, N), float("nan"), device=DEV)
+    ops.gemm_skinny_parts(a, w, planes)
+    units = (K + 63) // 64
+    part_k = (units + parts - 1) // parts * 64
+    for q in range(parts):
+        lo, hi = q * part_k, min(K, (q + 1) * part_k)
+        close(planes[q], a[:, lo:hi].double() @ w[:, lo:hi].double().t(), 1e-5, f"part {q}")
+    close(planes.sum(0), a.double() @ w.double().t(), 1e-5, "sum of the parts")
+    with pytest.raises(Exception, match="parts"):
+        ops.gemm_skinny_parts(a, w, torch.empty(K // 64 + 2, M, N, device=DEV))
+
+
 def gemm_reference(a, w, bias, epilogue, residual=None):
     y = a.double() @ w.double().t()
     if bias is not None:

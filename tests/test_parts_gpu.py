@@ -195,6 +195,44 @@ def test_feed_forward_alone(parts, lazy, monkeypatch):
     core.close("f")
 
 
+@pytest.mark.parametrize("reader", ["norm", "gathering norm", "settle"])
+def test_feed_forward_deferred(parts, reader, monkeypatch):
+    """The feed-forward's second product cut over its inner dimension: the parts' sums come
+    back pending, and the next reader of the stream adds them: a norm as it loads its rows
+    (writing them back), a norm over gathered rows (not writing back), or a pass of its own."""
+    from liyab_amd.engine import StepItem
+    from liyab_amd.kernels import ops
+
+    p, dtype = parts
+    if dtype != "bfloat16":
+        pytest.skip("only the bfloat16 products are cut over K")
+    monkeypatch.setattr(ops, "k_parts", lambda M, N, K: 3)  # the sizes here would not be cut
+    core = p.core
+    core.open("f")
+    ctx, _ = core.step_fn.prepare([StepItem("f", [1] * 11, [])])
+    rng = np.random.default_rng(2)
+    x = rand(rng, 11, p.d, scale=1.5).to(DEV)
+    residual = rand(rng, 11, p.d).to(DEV)
+    before = residual.clone()
+    want = f64(residual.cpu()) + plain_ffn(plain_norm(f64(x.cpu()), p.tw, "n2", p.eps), p.tw, "f", p.act)
+    pending = p.block.ffn.forward(p.block.norm_ffn.forward(x, ctx), ctx, residual, defer=True)
+    assert pending is not None and pending.planes.shape == (3, 11, p.d) and torch.equal(residual, before)
+    norm = p.block.norm_mixer
+    if reader == "settle":
+        pending.settle(residual)
+    elif reader == "norm":
+        got = norm.forward(residual, ctx, sums=pending.sums).float().cpu().numpy()
+        assert tt.rel_err(got, plain_norm(want, p.tw, "n1", p.eps)) < 1e-2
+    else:
+        rows = torch.tensor([7, 0, 7, 10], dtype=torch.int32, device=DEV)
+        got = norm.forward(residual, ctx, rows=rows, sums=pending.sums).float().cpu().numpy()
+        assert tt.rel_err(got, plain_norm(want[[7, 0, 7, 10]], p.tw, "n1", p.eps)) < 1e-2
+        assert torch.equal(residual, before)  # gathered rows are not written back
+        pending.settle(residual)
+    assert tt.rel_err(residual.cpu().numpy(), want) < 1e-2
+    core.close("f")
+
+
 @pytest.mark.parametrize("geometry", [dict(H=5, Hkv=5, hd=16), dict(H=6, Hkv=2, hd=32, d=96), dict(H=3, Hkv=1, hd=48, d=64, window=13)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_mixer_alone(dtype, geometry):
