@@ -259,11 +259,12 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
     if (wide < 0) wide = (mt > 1 && static_cast<long>(N) * M > (1L << 20)) ? 1 : 0;
     const int nt = wide ? 4 : 1;
     if (ksplit == 0) {
-        // enough waves to cover the chip several times over, each with at least 128 k
+        // waves until each has one trip's worth of K (everything is then asked for at once),
+        // or they cover the chip several times over
         const int tiles = ((N + 16 * nt - 1) / (16 * nt)) * ((M + 16 * mt - 1) / (16 * mt)) * kparts;
-        const int units = ((K + 63) / 64 + kparts - 1) / kparts;
+        const int units = ((K + 63) / 64 + kparts - 1) / kparts, per_trip = mt * nt == 1 ? 2 : 1;
         ksplit = 1;
-        while (ksplit < 16 && tiles * ksplit < 2048 && units / (ksplit * 2) >= (mt * nt == 1 ? 2 : 1)) ksplit *= 2;
+        while (ksplit < 16 && tiles * ksplit < 2048 && units > ksplit * per_trip) ksplit *= 2;
         // a folded norm takes a wave per row: as many waves as rows, so the rows go side by side
         if (ln.x != nullptr) ksplit = 8;
     }

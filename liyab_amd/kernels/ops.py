@@ -413,13 +413,14 @@ def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *,
 def k_parts(M: int, N: int, K: int) -> int:
     """Into how many parts of K the weight-streaming product is best cut (1: not at all). With
     few output features a product fills a fraction of the chip's compute units, and a long K
-    then streams through those few; cut over K it covers the chip. Measured at 8 rows:
-    3,072 -> 768 takes 7.0 us whole and 4.3 us in four parts; 6,400 -> 1,600 12.6 and 8 us."""
-    if M > 16 or K % 8 != 0 or K < 2048:
+    then streams through those few; cut over K it covers the chip. Measured at 8 rows, whole
+    and in parts (us): 3,072 -> 768 7.2 and 4.5 (four parts), 768 -> 768 4.6 and 3.4 (four),
+    6,400 -> 1,600 13.4 and 8.5 (two), 1,600 -> 1,600 5.4 and 4.6 (two)."""
+    if M > 16 or K % 8 != 0:
         return 1
     strips, units = (N + 15) // 16, (K + 63) // 64
     parts = 1
-    while parts < 4 and strips * parts * 2 <= 256 and units // (parts * 2) >= 8:
+    while parts < 4 and strips * parts * 2 <= 256 and units // (parts * 2) >= 3:
         parts *= 2
     return parts
 

@@ -27,10 +27,19 @@ class PreNormBlock:
             if pending is not None:
                 pending.settle(x)
             h = self._normed(self.norm_mixer, x, ctx)
-        self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
+        pending = None
+        if getattr(self.mixer, "defers", False):
+            pending = self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache, defer=True)
+        else:
+            self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
         if self.ffn is None:
-            return None
-        h = self._normed(self.norm_ffn, x, ctx)
+            return pending
+        if pending is not None and getattr(self.norm_ffn, "takes_sums", False):
+            h = self.norm_ffn.forward(x, ctx, sums=pending.sums)
+        else:
+            if pending is not None:
+                pending.settle(x)
+            h = self._normed(self.norm_ffn, x, ctx)
         if getattr(self.ffn, "defers", False):
             return self.ffn.forward(h, ctx, x, defer=True)
         self.ffn.forward(h, ctx, x)

@@ -4,9 +4,8 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
-from .base import PendingSums, StepContext
-from .linear import linear
+from .base import StepContext
+from .linear import linear, linear_deferred
 from .registry import register_ffn
 
 
@@ -35,13 +34,10 @@ class DenseFFN:
         PendingSums instead, for the next reader of the residual stream to add."""
         inner = ctx.workspace.get("ffn_inner", (h.shape[0], self.inner), self.dtype)
         linear(h, self.up_weight, self.up_bias, out=inner, activation=self.activation)
-        parts = ops.k_parts(h.shape[0], self.width, self.inner) if defer and self.dtype == torch.bfloat16 else 1
-        if parts > 1:
-            planes = ctx.workspace.get("ffn_parts", (parts, h.shape[0], self.width), torch.float32)
-            ops.gemm_skinny_parts(inner, self.down_weight, planes)
-            return PendingSums(planes, self.down_bias)
-        linear(inner, self.down_weight, self.down_bias, residual=residual)
-        return None
+        pending = linear_deferred(inner, self.down_weight, self.down_bias, ctx, "ffn_parts") if defer else None
+        if pending is None:
+            linear(inner, self.down_weight, self.down_bias, residual=residual)
+        return pending
 
 
 register_ffn("dense_ffn", DenseFFN)

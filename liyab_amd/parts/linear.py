@@ -50,6 +50,24 @@ def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[to
     ops.gemm(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
 
 
+def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name: str):
+    """a . w^T + bias as sums still to be added to the residual stream, or None where the
+    product is not worth cutting over its inner dimension (the caller then adds it through
+    `linear(..., residual=)`). The planes live in the step's workspace under `name` until the
+    next reader of the stream has added them."""
+    from .base import PendingSums
+
+    a = a.tensor() if isinstance(a, Normed) else a
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[0] > 64:
+        return None
+    parts = ops.k_parts(a.shape[0], w.shape[0], a.shape[1])
+    if parts <= 1:
+        return None
+    planes = ctx.workspace.get(name, (parts, a.shape[0], w.shape[0]), torch.float32)
+    ops.gemm_skinny_parts(a, w, planes)
+    return PendingSums(planes, bias)
+
+
 def paged_qkv_takes(dtype: torch.dtype, k: int) -> bool:
     """Whether the product kernels for this dtype and inner size can write keys and values
     into cache pages from their epilogue."""
