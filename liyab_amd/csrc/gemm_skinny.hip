@@ -250,9 +250,19 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
     // tiles of 16 rows a workgroup: all of M in one workgroup reads the weights once; with few
     // output features that leaves most of the chip idle, and the rows are spread over workgroups
     // instead (the weights then come from L2 after their first reading)
-    int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    if (mtile > 0) mt = mtile;
-    else if (mt > 1 && N <= 1024) mt = 1;
+    // (measured at 24 to 64 rows over GPT-2 small's, medium's and XL's shapes: the most rows a
+    // workgroup that still leaves 144 workgroups or more is the fastest or close to it)
+    int mt = 1;
+    if (mtile > 0) {
+        mt = mtile;
+    } else {
+        const int strips = (N + 15) / 16;
+        for (int cand = M <= 16 ? 1 : (M <= 32 ? 2 : 4); cand > 1; cand /= 2)
+            if (strips * ((M + 16 * cand - 1) / (16 * cand)) >= 144) {
+                mt = cand;
+                break;
+            }
+    }
     LIYAB_REQUIRE(mt == 1 || mt == 2 || mt == 4, "gemm_skinny: %d tiles of rows a workgroup is not 1, 2 or 4", mt);
     // wide tiles of N (64 features a workgroup) when N is so large that every workgroup
     // re-reading the tokens would cost more than the weights

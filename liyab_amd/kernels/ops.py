@@ -416,11 +416,11 @@ def k_parts(M: int, N: int, K: int) -> int:
     then streams through those few; cut over K it covers the chip. Measured at 8 rows, whole
     and in parts (us): 3,072 -> 768 7.2 and 4.5 (four parts), 768 -> 768 4.6 and 3.4 (four),
     6,400 -> 1,600 13.4 and 8.5 (two), 1,600 -> 1,600 5.4 and 4.6 (two)."""
-    if M > 16 or K % 8 != 0:
+    if M > 32 or K % 8 != 0:
         return 1
-    strips, units = (N + 15) // 16, (K + 63) // 64
+    groups, units = (N + 15) // 16 * ((M + 15) // 16), (K + 63) // 64  # workgroups uncut; units of 64 k
     parts = 1
-    while parts < 4 and strips * parts * 2 <= 256 and units // (parts * 2) >= 3:
+    while parts < 4 and groups * parts * 2 <= 256 and units // (parts * 2) >= 3:
         parts *= 2
     return parts
 
@@ -485,9 +485,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
     q_dim) with the paged QKV epilogue."""
     if mfma_takes(a, w):
         M, N = a.shape[0], w.shape[0]
-        if M <= 16 or (M <= 64 and N <= 8192):
+        if M <= 16 or (M <= 64 and N <= 8192 and not (M > 48 and N > 4096 and a.shape[1] % 64 == 0)):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
-            # kernel's shared loads beat every workgroup re-reading the tokens)
+            # kernel's shared loads beat every workgroup re-reading the tokens; so they do
+            # for a full tile of 64 tokens and a wide N: 12.6 against 19 us for 1,600 -> 4,800)
             gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=0)
         elif a.shape[1] % 64 == 0:
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
