@@ -422,6 +422,74 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
         assert all(core.manager.pages_in_use(g.index) == 0 for g in groups)
 
 
+class BareNorm:
+    """A LayerNorm that knows nothing of pending sums or pending norms (no `takes_sums`, no `lazy`)."""
+
+    def __init__(self, spec, store, dtype):
+        self.width, self.eps, self.dtype = spec.width, float(spec.eps), dtype
+        self.weight = store.fetch(spec.tensors["weight"], (self.width,), "vector")
+        self.bias = store.fetch(spec.tensors["bias"], (self.width,), "vector")
+
+    def forward(self, x, ctx, rows=None, n_rows=None, name="normed"):
+        from liyab_amd.kernels import ops
+
+        n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        out = ctx.workspace.get(name, (n, self.width), self.dtype)
+        ops.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows)
+        return out
+
+
+class BareBlock:
+    """The pre-norm arrangement written without any of the optional interfaces."""
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
+
+    def forward(self, x, ctx, cache, state, writes_cache=True):
+        self.mixer.forward(self.norm_mixer.forward(x, ctx), ctx, cache, state, x, writes_cache=writes_cache)
+        if self.ffn is not None:
+            self.ffn.forward(self.norm_ffn.forward(x, ctx), ctx, x)
+
+
+def test_pending_sums_reach_parts_that_cannot_take_them(monkeypatch):
+    """Products cut over K leave their sums pending for the next reader of the residual
+    stream. Here the cut is forced at the toy model's small sizes; layer 1's second norm (after
+    the attention whose projection is cut) is one that cannot add sums, and layer 2's block
+    (after layer 1's cut feed-forward) one that cannot take them: the sums are settled before
+    those parts run; the last layer's go to the final norm over gathered rows; the logits stay
+    those of the plain model."""
+    import dataclasses
+
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.kernels import ops
+    from liyab_amd.parts import register_block, register_norm
+
+    register_norm("bare_layernorm", BareNorm)
+    register_block("bare_pre_norm", BareBlock)
+    cut = []
+
+    def forced(M, N, K):
+        parts = 2 if M <= 16 and K % 8 == 0 and K > 64 else 1
+        cut.append(parts)
+        return parts
+
+    monkeypatch.setattr(ops, "k_parts", forced)
+    plan, tw, info = toy_model("bfloat16")
+    layers = list(plan.layers)
+    layers[1] = dataclasses.replace(layers[1], norm_ffn=dataclasses.replace(layers[1].norm_ffn, kind="bare_layernorm"))
+    layers[2] = dataclasses.replace(layers[2], arrangement="bare_pre_norm")
+    plan = dataclasses.replace(plan, layers=layers)
+    reqs = {f"t{i}": tt.random_tokens(90 + i, n, info["V"]) for i, n in enumerate([37, 90, 5, 61])}
+    ref = {rid: toy_plain(tw, info, toks) for rid, toks in reqs.items()}
+    for name, steps in (("portions", tt.schedule_portions(reqs, (5, 2, 11, 3, 16))), ("mixed", tt.schedule_mixed(reqs, seed=3))):
+        core = EngineCore.from_plan(plan, tw, dtype="bfloat16", page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4,
+                                    use_graphs=False)
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, TOL["bfloat16"], f"toy with forced cuts, {name}")
+        core.manager.check()
+    assert 2 in cut and 1 in cut  # both ways were taken
+
+
 def test_unknown_kinds_are_refused_by_name():
     from liyab_amd import Unsupported
     from liyab_amd.config import LayerSpec, OrderEntry
