@@ -339,7 +339,7 @@ using namespace liyab;
 // tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep and four waves; 6 = 64x64
 // with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages (deeper rings
 // measured slower: their LDS leaves one workgroup a compute unit, and 288 tiles then take two rounds), 9 = 128x64;
-// 13 = 128x128 two stages on four waves
+// 13 = 128x128 two stages on four waves, 16 = 64x32 four stages on two waves (for one tile of rows)
 // (0 = chosen from the shape).
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
@@ -366,6 +366,7 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 9: return launch_dl<128, 64, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 13: return launch_dl<128, 128, 2, 2, 2>(a, lda, w, M, N, K, epi, stream);
+        case 16: return launch_dl<64, 32, 4, 2, 1>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }

@@ -489,10 +489,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             # a vocabulary's worth of output features: large tiles re-read the tokens least
             # (16 rows: 22.5 against 25.1 us for 768 -> 50,257; 64 rows: 27.9 against 32.9)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=8)
-        elif M <= 16 or (M <= 64 and N <= 8192 and not (M > 48 and N > 4096 and a.shape[1] % 64 == 0)):
+        elif M > 32 and M <= 64 and a.shape[1] % 64 == 0 and N >= (2048 if M > 48 else 4097):
+            # one tile of 64 rows and many output features: 64 x 32 tiles share the tokens' rows
+            # through LDS where the streaming kernel's workgroups each read them again (64 rows:
+            # 6.2 against 7.6 us for 768 -> 2,304, 10.3 against 18.3 for 1,600 -> 4,800)
+            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=16)
+        elif M <= 16 or (M <= 64 and N <= 8192):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
-            # kernel's shared loads beat every workgroup re-reading the tokens; so they do
-            # for a full tile of 64 tokens and a wide N: 12.6 against 19 us for 1,600 -> 4,800)
+            # kernel's shared loads beat every workgroup re-reading the tokens)
             gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=0)
         elif a.shape[1] % 64 == 0:
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)

@@ -161,7 +161,7 @@ def test_gemm_float32(ops, M, N, K, epilogue):
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
-                                    "dl1", "dl2", "dl3", "dl5", "dl6", "dl7", "dl8", "dl9", "dl13"])
+                                    "dl1", "dl2", "dl3", "dl5", "dl6", "dl7", "dl8", "dl9", "dl13", "dl16"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
                                                  (500, 300, 128), (129, 193, 192)])
