@@ -145,8 +145,9 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     // depends on the row (a token's place in the pages) is computed once, and every store is four
     // consecutive columns wide. Tiles wholly inside the output take that path without bounds
     // checks (a guarded store is a branch of its own: on an interior tile they cost as much as
-    // the whole product); edge tiles, and operands that are not aligned for it, go element by element.
-    const bool inside = m0 + BM <= M && n0 + BN <= N;
+    // the whole product); tiles at the bottom edge take the same paths with their rows checked;
+    // tiles at the right edge, and operands that are not aligned for it, go element by element.
+    const bool inside = m0 + BM <= M && n0 + BN <= N, columns_inside = n0 + BN <= N;
     if constexpr (sizeof(OutT) == 2 && EPI >= 0 && EPI != kEpiResidual) {
         // bfloat16 outputs of interior tiles go through LDS once more, so that they leave as whole
         // rows: a wave lays its (BM / WM) x (BN / WN) results out row by row (bias and activation
@@ -155,7 +156,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         // rows with every instruction (measured: 5.7 of 19.7 us on a 2,048 x 2,304 product).
         constexpr int RM = BM / WM, CN = BN / WN, LDO = CN + 8;  // padded rows, 16-byte aligned
         static_assert(WAVES * RM * LDO <= DSTAGES * STAGE, "the output staging must fit the operand stages");
-        if (inside && vec_ok > 1) {
+        if (columns_inside && vec_ok > 1) {
             lds_barrier();  // everyone is done reading the last operand stage
             bf16_t* tile = lds + wave * RM * LDO;
 #pragma unroll
@@ -185,7 +186,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                 // the rows' places in the pages first: a load between two stores would wait for the first
 #pragma unroll
                 for (int t = 0; t < ROUNDS; ++t) {
-                    const int slot = epi.slots[mw + (t * 64 + lane) / CHUNKS];
+                    const int slot = epi.slots[min(mw + (t * 64 + lane) / CHUNKS, M - 1)];
                     const int page = page_shift >= 0 ? slot >> page_shift : slot / epi.page_size;
                     const int off = slot - page * epi.page_size;
                     row_base[t] = slot < 0 ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
@@ -194,6 +195,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
             for (int t = 0; t < ROUNDS; ++t) {
                 const int c = t * 64 + lane, row = c / CHUNKS, n = nw + (c % CHUNKS) * 8;
+                if (!inside && mw + row >= M) continue;
                 const u32x4 piece = *reinterpret_cast<const u32x4*>(tile + row * LDO + (c % CHUNKS) * 8);
                 bf16_t* dst;
                 if constexpr (EPI == kEpiQkvPaged) {
@@ -214,10 +216,11 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
             return;
         }
     }
-    if (EPI >= 0 && inside && vec_ok) {
+    if (EPI >= 0 && columns_inside && vec_ok) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int m = m0 + wm * (BM / WM) + i * 32 + li;
+            if (!inside && m >= M) continue;
             int64_t row_base = -1;
             if constexpr (EPI == kEpiQkvPaged) {
                 const int slot = epi.slots[m];
