@@ -16,10 +16,9 @@
 // K must be a multiple of 8. The order of the sum depends on K and the split
 // only, never on M.
 //
-// A LayerNorm may be folded into the first operand (M <= 16): the rows are
-// read from the 32-bit residual stream, normalised and written to LDS in
-// bfloat16 by the workgroup itself, a wave per row with its statistics in
-// registers (two passes, 32-bit, as the standalone kernel computes them).
+// The product may be cut over K into parts (blockIdx.z), each part's sums going to its own
+// plane of 32-bit sums; the first plane may take the bias and the rows the product is to be
+// added to (themselves a sum of planes), so that the planes together are the new rows.
 #include "common.h"
 #include "epilogue.h"
 
@@ -34,25 +33,23 @@ union Frag {
     bf16x8 v;
 };
 
-struct LnParams {
-    const float* x;      // [*, K] 32-bit rows; null: no norm, `a` holds bfloat16 rows
-    const float* weight; // [K] or null
-    const float* bias;   // [K] or null
-    const int* rows;     // [M] or null
-    float eps;
+// What the first part of a product cut over K adds to its plane: the rows the product is
+// added to, given as a sum of planes [n][M][N] (added in their order), or nothing.
+struct BaseSum {
+    const float* planes;
+    int n;
+    int64_t stride;
 };
 
-template <typename OutT, bool LN, int MT, int NT, int MAXW, int MAXV = 32>
+template <typename OutT, int MT, int NT, int MAXW>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
-                   EpiParams epi, LnParams ln, int part_k, int64_t part_stride) {
+                   EpiParams epi, BaseSum base, int part_k, int64_t part_stride) {
     constexpr int UPT = (MT * NT == 1) ? 2 : 1;  // units of 64 k per trip
     constexpr int TILES = MT * NT;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int ksplit = blockDim.x / 64;
-    const int ldx = K + 8;
-    bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // LN: [M][K + 8]
-    float* red = reinterpret_cast<float*>(smem + (LN ? ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16 : 0));
+    float* red = reinterpret_cast<float*>(smem);
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int i = lane % 16, g = lane / 16;
@@ -63,6 +60,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     const int k_begin = blockIdx.z * part_k, k_end = min(K, k_begin + part_k);
     const int units = (k_end - k_begin + 63) / 64;
     if (gridDim.z > 1) epi.out = static_cast<float*>(epi.out) + blockIdx.z * part_stride;
+    if (blockIdx.z > 0) epi.bias = nullptr;  // a cut product's bias goes to its first plane only
     const u32x4 zero = {0, 0, 0, 0};
     const bf16_t* wrow[NT];
 #pragma unroll
@@ -87,55 +85,33 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
         }
     };
     Frag wc[UPT][NT][2];
-    load_w(wave * UPT, wc);  // issued before the norm's prologue, so the two overlap
+    load_w(wave * UPT, wc);
     // what the epilogue will read for this thread's first output (bias, residual) is asked for
     // now: after the sums it would be one more trip to memory on the critical path
     const int e_m = m0 + 16 * ((tid / 256) / NT) + (tid % 256) / 16, e_n = n0 + 16 * ((tid / 256) % NT) + tid % 16;
     const bool e_mine = tid < TILES * 256 && e_m < M && e_n < N;
     const float e_bias = (e_mine && epi.bias != nullptr) ? epi.bias[e_n] : 0.0f;
     const float e_res = (e_mine && epi.mode == kEpiResidual) ? epi.residual[static_cast<int64_t>(e_m) * epi.ldr + e_n] : 0.0f;
+    // the first part's share of the rows the product is added to: up to four planes asked for
+    // together (a plane past the last is the last one again, read and dropped)
+    const bool based = base.planes != nullptr && blockIdx.z == 0;
+    float e_base[4];
+    {
+        // no branch around the loads (a load under a branch is waited for where the branch ends,
+        // and the weights asked for above with it): whoever has nothing to add reads a word of
+        // the weights instead and drops it
+        const float* src = based ? base.planes : reinterpret_cast<const float*>(w);
+        const int64_t at = (based && e_mine) ? static_cast<int64_t>(e_m) * N + e_n : 0;
+        const int64_t stride = based ? base.stride : 0;
+        const int last = based ? base.n - 1 : 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) e_base[q] = src[min(q, last) * stride + at];
+    }
     __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
 
     const bf16_t* arow[MT];
-    if constexpr (LN) {
-        // a row's values stay in registers: MAXV per lane, K <= 64 * MAXV
-        for (int m = wave; m < M; m += ksplit) {
-            const float* xr = ln.x + static_cast<int64_t>(ln.rows != nullptr ? ln.rows[m] : m) * K;
-            float v[MAXV], gw[MAXV], gb[MAXV];
-            float sum = 0.0f;
 #pragma unroll
-            for (int j = 0; j < MAXV; ++j) {
-                if (64 * j >= K) break;
-                const int k = lane + 64 * j;
-                const bool in = k < K;
-                v[j] = in ? xr[k] : 0.0f;
-                gw[j] = (in && ln.weight != nullptr) ? ln.weight[k] : 1.0f;
-                gb[j] = (in && ln.bias != nullptr) ? ln.bias[k] : 0.0f;
-                sum += v[j];
-            }
-            const float mean = wave_sum(sum) / static_cast<float>(K);
-            float ss = 0.0f;
-#pragma unroll
-            for (int j = 0; j < MAXV; ++j) {
-                if (64 * j >= K) break;
-                const float dev = lane + 64 * j < K ? v[j] - mean : 0.0f;
-                ss += dev * dev;
-            }
-            const float rstd = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(K) + ln.eps);
-#pragma unroll
-            for (int j = 0; j < MAXV; ++j) {
-                if (64 * j >= K) break;
-                const int k = lane + 64 * j;
-                if (k < K) xs[m * ldx + k] = float_to_bf16((v[j] - mean) * rstd * gw[j] + gb[j]);
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int s = 0; s < MT; ++s) arow[s] = xs + min(16 * s + i, M - 1) * ldx;
-    } else {
-#pragma unroll
-        for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(m0 + 16 * s + i, M - 1)) * lda;
-    }
+    for (int s = 0; s < MT; ++s) arow[s] = a + static_cast<int64_t>(min(m0 + 16 * s + i, M - 1)) * lda;
     // the tokens' fragments travel with the weights', a trip ahead: asked for after the next
     // trip's weights they would make every trip wait for those too (loads return in order)
     auto load_x = [&](int u0, Frag (&x)[UPT][MT][2]) {
@@ -206,46 +182,63 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
         float v = 0.0f;
         for (int q = 0; q < ksplit; ++q) v += red[q * TILES * 256 + e];
         if (m >= M || n >= N) continue;
+        if (based) {
+            // this plane = (sums + bias) + (base planes added up in their order)
+            const float* bp = base.planes + static_cast<int64_t>(m) * N + n;
+            float b;
+            if (e == tid) {
+                b = e_base[0];
+#pragma unroll
+                for (int q = 1; q < 4; ++q)
+                    if (q < base.n) b += e_base[q];
+                for (int q = 4; q < base.n; ++q) b += bp[q * base.stride];
+            } else {
+                b = bp[0];
+                for (int q = 1; q < base.n; ++q) b += bp[q * base.stride];
+            }
+            v = (v + (e == tid ? e_bias : epilogue_bias(epi, n))) + b;
+            static_cast<float*>(epi.out)[static_cast<int64_t>(m) * epi.ldo + n] = v;
+            continue;
+        }
         if (e != tid) epilogue_store<OutT>(epi, m, n, v);
         else if (epi.mode == kEpiResidual) epi.residual[static_cast<int64_t>(m) * epi.ldr + n] = e_res + (v + e_bias);
         else epilogue_store_biased<OutT>(epi, m, n, v + e_bias);
     }
 }
 
-template <bool LN, int MT, int NT, int MAXW, int MAXV = 32>
+template <int MT, int NT, int MAXW>
 int launch_skinny(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, const EpiParams& epi,
-                  const LnParams& ln, int kparts, int64_t part_stride, hipStream_t stream) {
+                  const BaseSum& base, int kparts, int64_t part_stride, hipStream_t stream) {
     // K in kparts parts, each a whole number of units of 64 and none of them empty (the caller's check)
     const int part_k = ((K + 63) / 64 + kparts - 1) / kparts * 64;
-    const dim3 grid((N + 16 * NT - 1) / (16 * NT), LN ? 1 : (M + 16 * MT - 1) / (16 * MT), kparts);
+    const dim3 grid((N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT), kparts);
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
     if (ksplit > MAXW) ksplit = MAXW;
     size_t smem = static_cast<size_t>(ksplit) * MT * NT * 256 * sizeof(float);
-    if (LN) smem += ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16;
     const bool f32 = epi.mode == kEpiResidual || epi.out_dtype == kF32;
     if (f32) {
-        auto kern = gemm_skinny_kernel<float, LN, MT, NT, MAXW, MAXV>;
+        auto kern = gemm_skinny_kernel<float, MT, NT, MAXW>;
         static bool ready = false;
         if (!ready) {
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             ready = true;
         }
-        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln, part_k, part_stride);
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, base, part_k, part_stride);
     } else {
-        auto kern = gemm_skinny_kernel<bf16_t, LN, MT, NT, MAXW, MAXV>;
+        auto kern = gemm_skinny_kernel<bf16_t, MT, NT, MAXW>;
         static bool ready = false;
         if (!ready) {
             hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             ready = true;
         }
-        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, ln, part_k, part_stride);
+        kern<<<grid, 64 * ksplit, smem, stream>>>(pa, lda, pw, M, N, K, epi, base, part_k, part_stride);
     }
     return check_launch("gemm_skinny");
 }
 
 static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int N, int K, int ksplit, int wide, int mtile,
-                           const EpiParams& epi, const LnParams& ln, hipStream_t stream, int kparts = 1,
+                           const EpiParams& epi, const BaseSum& base, hipStream_t stream, int kparts = 1,
                            int64_t part_stride = 0) {
     // tiles of 16 rows a workgroup: all of M in one workgroup reads the weights once; with few
     // output features that leaves most of the chip idle, and the rows are spread over workgroups
@@ -277,23 +270,17 @@ static int skinny_dispatch(const void* a, int64_t lda, const void* w, int M, int
         // (with so many output features that one wave a workgroup covers the chip, two or four
         // still pay while a wave keeps more than 8 units: 18.3 against 20.0 us for 768 -> 50,257)
         while (ksplit < 16 && units > ksplit * per_trip && (tiles * ksplit < 2048 || units / ksplit > 8)) ksplit *= 2;
-        // a folded norm takes a wave per row: as many waves as rows, so the rows go side by side
-        if (ln.x != nullptr) ksplit = 8;
     }
     LIYAB_REQUIRE(ksplit == 1 || ksplit == 2 || ksplit == 4 || ksplit == 8 || ksplit == 16,
                   "gemm_skinny: ksplit %d is not 1, 2, 4, 8 or 16", ksplit);
-    if (ln.x != nullptr) {  // 8 waves: registers for a row's values
-        if (K <= 1024) return launch_skinny<true, 1, 1, 8, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-        return launch_skinny<true, 1, 1, 8, 32>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-    }
     if (nt == 1) {
-        if (mt == 1) return launch_skinny<false, 1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-        if (mt == 2) return launch_skinny<false, 2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-        return launch_skinny<false, 4, 1, 16>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+        if (mt == 1) return launch_skinny<1, 1, 16>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
+        if (mt == 2) return launch_skinny<2, 1, 16>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
+        return launch_skinny<4, 1, 16>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
     }
-    if (mt == 1) return launch_skinny<false, 1, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-    if (mt == 2) return launch_skinny<false, 2, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
-    return launch_skinny<false, 4, 4, 4>(a, lda, w, M, N, K, ksplit, epi, ln, kparts, part_stride, stream);
+    if (mt == 1) return launch_skinny<1, 4, 4>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
+    if (mt == 2) return launch_skinny<2, 4, 4>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
+    return launch_skinny<4, 4, 4>(a, lda, w, M, N, K, ksplit, epi, base, kparts, part_stride, stream);
 }
 
 }  // namespace liyab
@@ -314,16 +301,21 @@ extern "C" int liyab_gemm_skinny(const void* a, int64_t lda, const void* w, int 
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
-    return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, mtile, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream);
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, wide, mtile, epi, BaseSum{nullptr, 0, 0}, stream);
 }
 
 // The product's sums over `kparts` parts of K, one plane [M, N] of 32-bit sums a part:
-// parts[p * part_stride + m * N + n] = sum over the p-th part of K of a[m, k] w[n, k], no bias.
+// parts[p * part_stride + m * N + n] = sum over the p-th part of K of a[m, k] w[n, k].
 // For a product with few output features and a long K: cut over K it fills the chip, and
-// whoever reads the result next adds the planes up in their order (the norm kernel does).
-// Every part holds at least one unit of 64 k: (kparts - 1) * ceil(ceil(K / 64) / kparts) * 64 < K.
+// whoever reads the result next adds the planes up in their order (the norm kernels do).
+// With `base` (n_base planes [M, N], base_stride floats apart, not overlapping `parts`), the
+// first plane also takes bias[n] and base[0][m, n] + base[1][m, n] + ...: the planes together
+// are then base + a . w^T + bias, the rows of a residual stream after the product was added.
+// Without `base`, `bias` must be null. Every part holds at least one unit of 64 k:
+// (kparts - 1) * ceil(ceil(K / 64) / kparts) * 64 < K.
 extern "C" int liyab_gemm_skinny_parts(const void* a, int64_t lda, const void* w, int M, int N, int K, int kparts,
-                                       int ksplit, float* parts, int64_t part_stride, hipStream_t stream) {
+                                       int ksplit, float* parts, int64_t part_stride, const float* bias,
+                                       const float* base, int n_base, int64_t base_stride, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && parts, "gemm: null operand");
     LIYAB_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_parts: bad sizes M=%d (at most 64) N=%d K=%d", M, N, K);
     LIYAB_REQUIRE(K % 8 == 0 && lda % 8 == 0 && lda >= K, "gemm_skinny_parts: K %d and lda %lld must be multiples of 8", K,
@@ -334,29 +326,20 @@ extern "C" int liyab_gemm_skinny_parts(const void* a, int64_t lda, const void* w
     LIYAB_REQUIRE(kparts >= 1 && kparts <= 16 && (kparts - 1) * ((units + kparts - 1) / kparts) < units,
                   "gemm_skinny_parts: K = %d does not cut into %d parts of whole units of 64", K, kparts);
     LIYAB_REQUIRE(part_stride >= static_cast<int64_t>(M) * N, "gemm_skinny_parts: planes of %lld overlap", static_cast<long long>(part_stride));
+    LIYAB_REQUIRE(base != nullptr || bias == nullptr, "gemm_skinny_parts: a bias needs the rows it is added to");
+    if (base != nullptr) {
+        LIYAB_REQUIRE(n_base >= 1 && n_base <= 16 && (n_base == 1 || base_stride >= static_cast<int64_t>(M) * N),
+                      "gemm_skinny_parts: bad planes of rows to add to (%d, %lld apart)", n_base, static_cast<long long>(base_stride));
+        const float* base_end = base + (n_base - 1) * base_stride + static_cast<int64_t>(M) * N;
+        const float* parts_end = parts + (kparts - 1) * part_stride + static_cast<int64_t>(M) * N;
+        LIYAB_REQUIRE(base_end <= parts || parts_end <= base, "gemm_skinny_parts: the rows to add to overlap the planes written");
+    }
     if (M == 0) return 0;
     EpiParams epi{};
     epi.mode = kEpiNone;
     epi.out_dtype = kF32;
     epi.out = parts;
     epi.ldo = N;
-    return skinny_dispatch(a, lda, w, M, N, K, ksplit, 0, 1, epi, LnParams{nullptr, nullptr, nullptr, nullptr, 0.0f}, stream,
-                           kparts, part_stride);
-}
-
-// The same product with a LayerNorm folded in: the first operand is LayerNorm(x[rows[m] or m])
-// of the 32-bit rows x [*, K]. M <= 16, K <= 2048, and M * (K + 8) * 2 bytes must fit 64 KiB of LDS.
-extern "C" int liyab_gemm_skinny_ln(const float* x, const float* ln_weight, const float* ln_bias, const int* rows,
-                                    float eps, const void* w, int M, int N, int K, int ksplit,
-                                    const EpiParams* epi_in, hipStream_t stream) {
-    LIYAB_REQUIRE(x && w && epi_in, "gemm: null operand");
-    LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 16) N=%d K=%d", M, N, K);
-    LIYAB_REQUIRE(K % 8 == 0 && K <= 2048, "gemm_skinny_ln: K %d must be a multiple of 8, at most 2048", K);
-    LIYAB_REQUIRE(static_cast<size_t>(M) * (K + 8) * 2 <= 65536, "gemm_skinny_ln: %d rows of %d do not fit the LDS budget", M, K);
-    LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm_skinny_ln: weights must be 16-byte aligned");
-    LIYAB_REQUIRE(eps >= 0.0f, "gemm_skinny_ln: negative eps");
-    EpiParams epi = *epi_in;
-    if (int rc = check_epilogue(epi, M, N)) return rc;
-    if (M == 0) return 0;
-    return skinny_dispatch(nullptr, K + 8, w, M, N, K, ksplit, 0, 0, epi, LnParams{x, ln_weight, ln_bias, rows, eps}, stream);
+    epi.bias = bias;
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, 0, 1, epi, BaseSum{base, n_base, base_stride}, stream, kparts, part_stride);
 }

@@ -8,10 +8,10 @@
 // row r normalises input row rows[r] (the final norm runs only on the rows
 // whose logits are wanted, src/core/transformer.cpp:6569-6572).
 //
-// The rows may come with sums that are still to be added to them: a product cut over its
-// inner dimension leaves one plane of partial sums a part, and the norm that reads the
-// residual stream next adds bias and planes, in their order, as it loads the row (and writes
-// the row back, so that the stream holds the sum from then on).
+// The rows may come as a sum of planes: a product cut over its inner dimension leaves one
+// plane of 32-bit sums a part (the first of them holding the rows the product was added to),
+// and the norm that reads the residual stream next adds the planes up, in their order, as it
+// loads a row.
 #include "common.h"
 
 namespace liyab {
@@ -58,20 +58,16 @@ layernorm_kernel(T* __restrict__ out, const float* __restrict__ x, const float* 
     }
 }
 
-// Sums still to be added to the rows of x: planes [n_parts][rows of x][d] and a bias [d] or null.
+// Rows given as a sum of planes: row r is x[r] + x[stride + r] + ... (n_parts planes, 1: x itself).
 struct PartSums {
-    const float* parts;
     int n_parts;
     int64_t stride;
-    const float* bias;
 };
 
 // The same for rows that fit a wave's registers (d a multiple of 4, at most 256 * MAXV): a
 // wave per row, four rows a workgroup. The row is read once, 16 bytes a lane; sums go over
 // the wave only (no LDS, no barrier); weight and bias are fetched before the sums, so their
-// latency hides behind them. x_back: where rows with their sums added are written back (x
-// itself), or null (rows gathered through `rows` are not written back: a row named twice
-// would get its sums twice).
+// latency hides behind them.
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 template <typename T>
@@ -88,51 +84,39 @@ __device__ __forceinline__ void store_row4<bf16_t>(bf16_t* dst, const f32x4& v) 
 
 template <typename T, int MAXV, bool PARTS>
 __global__ void __launch_bounds__(256)
-layernorm_wave_kernel(T* __restrict__ out, const float* x, float* x_back, const float* __restrict__ w,
+layernorm_wave_kernel(T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
                       const float* __restrict__ b, const int* __restrict__ rows, int n, int d, float eps, PartSums ps) {
     const int lane = threadIdx.x % kWave, r = blockIdx.x * 4 + threadIdx.x / kWave;
     if (r >= n) return;
     const int64_t src = rows != nullptr ? rows[r] : r;
-    const f32x4* xr = reinterpret_cast<const f32x4*>(x + src * d);
+    const float* row0 = x + src * d;
     const int nv = d / 4;
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f}, one = {1.0f, 1.0f, 1.0f, 1.0f};
     f32x4 v[MAXV], gw[MAXV], gb[MAXV];
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) {
         const int i = min(lane + kWave * j, nv - 1);  // past the row: its last piece again, unused
-        v[j] = xr[i];
+        v[j] = reinterpret_cast<const f32x4*>(row0)[i];
         gw[j] = w != nullptr ? reinterpret_cast<const f32x4*>(w)[i] : one;
         gb[j] = b != nullptr ? reinterpret_cast<const f32x4*>(b)[i] : zero;
     }
     if constexpr (PARTS) {
-        // bias, then the planes in their order, four planes' loads in flight together (a plane
+        // the further planes in their order, three planes' loads in flight together (a plane
         // past the last is the last one again, read and dropped: no load under a branch)
-        f32x4 add[MAXV];
+        constexpr int PB = MAXV <= 4 ? 3 : 1;
+        for (int q0 = 1; q0 < ps.n_parts; q0 += PB) {
+            f32x4 plane[PB][MAXV];
 #pragma unroll
-        for (int j = 0; j < MAXV; ++j)
-            add[j] = ps.bias != nullptr ? reinterpret_cast<const f32x4*>(ps.bias)[min(lane + kWave * j, nv - 1)] : zero;
-        for (int q0 = 0; q0 < ps.n_parts; q0 += 4) {
-            f32x4 plane[4][MAXV];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const float* row = ps.parts + min(q0 + u, ps.n_parts - 1) * ps.stride + src * d;
+            for (int u = 0; u < PB; ++u) {
+                const float* row = row0 + min(q0 + u, ps.n_parts - 1) * ps.stride;
 #pragma unroll
                 for (int j = 0; j < MAXV; ++j) plane[u][j] = reinterpret_cast<const f32x4*>(row)[min(lane + kWave * j, nv - 1)];
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < PB; ++u)
 #pragma unroll
                 for (int j = 0; j < MAXV; ++j)
-                    if (q0 + u < ps.n_parts) add[j] += plane[u][j];
-        }
-#pragma unroll
-        for (int j = 0; j < MAXV; ++j) v[j] += add[j];
-    }
-    if constexpr (PARTS) {
-        if (x_back != nullptr) {
-#pragma unroll
-            for (int j = 0; j < MAXV; ++j)
-                if (lane + kWave * j < nv) reinterpret_cast<f32x4*>(x_back + src * d)[lane + kWave * j] = v[j];
+                    if (q0 + u < ps.n_parts) v[j] += plane[u][j];
         }
     }
     float s = 0.0f;
@@ -154,47 +138,42 @@ layernorm_wave_kernel(T* __restrict__ out, const float* x, float* x_back, const 
         if (lane + kWave * j < nv) store_row4<T>(o + 4 * (lane + kWave * j), (v[j] - mean) * scale * gw[j] + gb[j]);
 }
 
-// x[i] += bias[i % d] + parts[0][i] + parts[1][i] + ..., added up in that order (the norm
-// kernel's order), for every row of x.
-__global__ void __launch_bounds__(256) add_parts_kernel(float* __restrict__ x, int64_t total, int d, PartSums ps) {
+// out[i] = planes[0][i] + planes[1][i] + ..., added up in that order (the norm kernels' order).
+__global__ void __launch_bounds__(256) sum_parts_kernel(float* out, const float* planes, int64_t total, PartSums ps) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= total) return;
-    float add = ps.bias != nullptr ? ps.bias[i % d] : 0.0f;
-    for (int q = 0; q < ps.n_parts; ++q) add += ps.parts[q * ps.stride + i];
-    x[i] += add;
+    float v = planes[i];
+    for (int q = 1; q < ps.n_parts; ++q) v += planes[q * ps.stride + i];
+    out[i] = v;
 }
 
 template <typename T, int MAXV>
-void launch_wave(T* out, const float* x, float* x_back, const float* w, const float* b, const int* rows, int n, int d,
-                 float eps, const PartSums& ps, hipStream_t stream) {
+void launch_wave(T* out, const float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
+                 const PartSums& ps, hipStream_t stream) {
     const int grid = (n + 3) / 4;
-    if (ps.n_parts > 0 || ps.bias != nullptr)
-        layernorm_wave_kernel<T, MAXV, true><<<grid, 256, 0, stream>>>(out, x, x_back, w, b, rows, n, d, eps, ps);
-    else
-        layernorm_wave_kernel<T, MAXV, false><<<grid, 256, 0, stream>>>(out, x, nullptr, w, b, rows, n, d, eps, ps);
+    if (ps.n_parts > 1) layernorm_wave_kernel<T, MAXV, true><<<grid, 256, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
+    else layernorm_wave_kernel<T, MAXV, false><<<grid, 256, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
 }
 
-// x_rows: rows of x (and of each plane of ps), for when the sums need a pass of their own.
-template <typename T>
-int launch_layernorm(T* out, float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
-                     const PartSums& ps, int x_rows, hipStream_t stream) {
+// Whether the kernel with a wave per row takes these operands (the only one that adds planes up).
+static bool wave_takes(const void* out, const float* x, const float* w, const float* b, int d, int64_t stride) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    if (d % 4 == 0 && d <= 2048 && al16(out) && al16(x) && al16(w) && al16(b) && al16(ps.parts) && al16(ps.bias) &&
-        ps.stride % 4 == 0) {
-        float* back = rows == nullptr ? x : nullptr;
-        if (d <= 256) launch_wave<T, 1>(out, x, back, w, b, rows, n, d, eps, ps, stream);
-        else if (d <= 512) launch_wave<T, 2>(out, x, back, w, b, rows, n, d, eps, ps, stream);
-        else if (d <= 768) launch_wave<T, 3>(out, x, back, w, b, rows, n, d, eps, ps, stream);
-        else if (d <= 1024) launch_wave<T, 4>(out, x, back, w, b, rows, n, d, eps, ps, stream);
-        else launch_wave<T, 8>(out, x, back, w, b, rows, n, d, eps, ps, stream);
+    return d % 4 == 0 && d <= 2048 && al16(out) && al16(x) && al16(w) && al16(b) && stride % 4 == 0;
+}
+
+template <typename T>
+int launch_layernorm(T* out, const float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
+                     const PartSums& ps, hipStream_t stream) {
+    if (wave_takes(out, x, w, b, d, ps.stride)) {
+        if (d <= 256) launch_wave<T, 1>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else if (d <= 512) launch_wave<T, 2>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else if (d <= 768) launch_wave<T, 3>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else if (d <= 1024) launch_wave<T, 4>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else launch_wave<T, 8>(out, x, w, b, rows, n, d, eps, ps, stream);
         return check_launch("layernorm");
     }
-    if (ps.n_parts > 0 || ps.bias != nullptr) {
-        // the general kernel reads its rows three times: the sums go in first, into every row of x
-        const int64_t total = static_cast<int64_t>(x_rows) * d;
-        add_parts_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(x, total, d, ps);
-        if (int rc = check_launch("add_parts")) return rc;
-    }
+    LIYAB_REQUIRE(ps.n_parts <= 1, "layernorm: rows in %d planes need a width that is a multiple of 4, at most 2048 (got %d), and 16-byte alignment",
+                  ps.n_parts, d);
     if (d <= 256) layernorm_kernel<T, 64><<<n, 64, 0, stream>>>(out, x, w, b, rows, d, eps);
     else layernorm_kernel<T, 256><<<n, 256, 0, stream>>>(out, x, w, b, rows, d, eps);
     return check_launch("layernorm");
@@ -210,42 +189,40 @@ extern "C" int liyab_layernorm(void* out, int out_dtype, const float* x, const f
     LIYAB_REQUIRE(n >= 0 && d > 0, "layernorm: bad sizes n=%d d=%d", n, d);
     LIYAB_REQUIRE(eps >= 0.0f, "layernorm: negative eps");
     if (n == 0) return 0;
-    const PartSums none{nullptr, 0, 0, nullptr};
-    float* rows_of_x = const_cast<float*>(x);  // never written when there are no sums to add
-    if (out_dtype == kF32) return launch_layernorm(static_cast<float*>(out), rows_of_x, w, b, rows, n, d, eps, none, 0, stream);
-    if (out_dtype == kBF16) return launch_layernorm(static_cast<bf16_t*>(out), rows_of_x, w, b, rows, n, d, eps, none, 0, stream);
+    const PartSums none{1, 0};
+    if (out_dtype == kF32) return launch_layernorm(static_cast<float*>(out), x, w, b, rows, n, d, eps, none, stream);
+    if (out_dtype == kBF16) return launch_layernorm(static_cast<bf16_t*>(out), x, w, b, rows, n, d, eps, none, stream);
     return fail(1, "layernorm: unknown output dtype %d", out_dtype);
 }
 
-// The same over rows that still lack sums: x [x_rows, d] += pbias + parts[0] + parts[1] + ...
-// (planes [x_rows, d], part_stride floats apart; pbias [d] or null), then the norm. Without
-// `rows`, every row of x is normalised (n == x_rows) and x holds the sums afterwards. With
-// `rows`, the named rows are summed on the fly and x is left as it was, unless the width
-// needs the general kernel: then x gets the sums first, in a pass of its own.
-extern "C" int liyab_layernorm_parts(void* out, int out_dtype, float* x, const float* w, const float* b, const int* rows,
-                                     int n, int d, float eps, const float* parts, int n_parts, int64_t part_stride,
-                                     const float* pbias, int x_rows, hipStream_t stream) {
-    LIYAB_REQUIRE(out && x, "layernorm: null pointer");
+// The same over rows given as a sum of planes: row r is planes[0][r] + planes[1][r] + ...
+// (n_parts planes [x_rows, d], part_stride floats apart), added in that order. d must be a
+// multiple of 4, at most 2048, and the operands 16-byte aligned (liyab_sum_parts first otherwise).
+extern "C" int liyab_layernorm_parts(void* out, int out_dtype, const float* planes, int n_parts, int64_t part_stride,
+                                     int x_rows, const float* w, const float* b, const int* rows, int n, int d, float eps,
+                                     hipStream_t stream) {
+    LIYAB_REQUIRE(out && planes, "layernorm: null pointer");
     LIYAB_REQUIRE(n >= 0 && d > 0 && x_rows >= 0, "layernorm: bad sizes n=%d d=%d", n, d);
     LIYAB_REQUIRE(eps >= 0.0f, "layernorm: negative eps");
-    LIYAB_REQUIRE(n_parts >= 0 && n_parts <= 16 && (n_parts == 0 || parts != nullptr), "layernorm: bad number of parts %d", n_parts);
-    LIYAB_REQUIRE(n_parts == 0 || part_stride >= static_cast<int64_t>(x_rows) * d, "layernorm: planes of sums overlap");
-    LIYAB_REQUIRE(rows != nullptr || n == x_rows, "layernorm: %d rows to normalise, %d rows of sums", n, x_rows);
+    LIYAB_REQUIRE(n_parts >= 1 && n_parts <= 16, "layernorm: bad number of planes %d", n_parts);
+    LIYAB_REQUIRE(n_parts == 1 || part_stride >= static_cast<int64_t>(x_rows) * d, "layernorm: planes of sums overlap");
+    LIYAB_REQUIRE(rows != nullptr || n <= x_rows, "layernorm: %d rows to normalise, %d rows given", n, x_rows);
     if (n == 0) return 0;
-    const PartSums ps{parts, n_parts, part_stride, pbias};
-    if (out_dtype == kF32) return launch_layernorm(static_cast<float*>(out), x, w, b, rows, n, d, eps, ps, x_rows, stream);
-    if (out_dtype == kBF16) return launch_layernorm(static_cast<bf16_t*>(out), x, w, b, rows, n, d, eps, ps, x_rows, stream);
+    const PartSums ps{n_parts, part_stride};
+    if (out_dtype == kF32) return launch_layernorm(static_cast<float*>(out), planes, w, b, rows, n, d, eps, ps, stream);
+    if (out_dtype == kBF16) return launch_layernorm(static_cast<bf16_t*>(out), planes, w, b, rows, n, d, eps, ps, stream);
     return fail(1, "layernorm: unknown output dtype %d", out_dtype);
 }
 
-// x [x_rows, d] += pbias + parts[0] + parts[1] + ..., for a reader of the rows that is no norm.
-extern "C" int liyab_add_parts(float* x, int x_rows, int d, const float* parts, int n_parts, int64_t part_stride,
-                               const float* pbias, hipStream_t stream) {
-    LIYAB_REQUIRE(x && x_rows >= 0 && d > 0, "add_parts: bad operands");
-    LIYAB_REQUIRE(n_parts >= 0 && n_parts <= 16 && (n_parts == 0 || parts != nullptr), "add_parts: bad number of parts %d", n_parts);
-    LIYAB_REQUIRE(n_parts == 0 || part_stride >= static_cast<int64_t>(x_rows) * d, "add_parts: planes of sums overlap");
+// out [x_rows, d] = planes[0] + planes[1] + ..., for a reader of the rows that cannot add them up itself.
+// `out` may be the first plane.
+extern "C" int liyab_sum_parts(float* out, int x_rows, int d, const float* planes, int n_parts, int64_t part_stride,
+                               hipStream_t stream) {
+    LIYAB_REQUIRE(out && planes && x_rows >= 0 && d > 0, "sum_parts: bad operands");
+    LIYAB_REQUIRE(n_parts >= 1 && n_parts <= 16, "sum_parts: bad number of planes %d", n_parts);
+    LIYAB_REQUIRE(n_parts == 1 || part_stride >= static_cast<int64_t>(x_rows) * d, "sum_parts: planes of sums overlap");
     const int64_t total = static_cast<int64_t>(x_rows) * d;
     if (total == 0) return 0;
-    add_parts_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(x, total, d, PartSums{parts, n_parts, part_stride, pbias});
-    return check_launch("add_parts");
+    sum_parts_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(out, planes, total, PartSums{n_parts, part_stride});
+    return check_launch("sum_parts");
 }

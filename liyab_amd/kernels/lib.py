@@ -40,9 +40,9 @@ _SIGNATURES = {
     "liyab_add_rows": [P, P, c_int, P, c_int, c_int, P],
     "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
     "liyab_layernorm": [P, c_int, P, P, P, P, c_int, c_int, c_float, P],
-    "liyab_layernorm_parts": [P, c_int, P, P, P, P, c_int, c_int, c_float, P, c_int, c_int64, P, c_int, P],
-    "liyab_add_parts": [P, c_int, c_int, P, c_int, c_int64, P, P],
-    "liyab_gemm_skinny_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P],
+    "liyab_layernorm_parts": [P, c_int, P, c_int, c_int64, c_int, P, P, P, c_int, c_int, c_float, P],
+    "liyab_sum_parts": [P, c_int, c_int, P, c_int, c_int64, P],
+    "liyab_gemm_skinny_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_simple": [P, c_int, c_int64, P, c_int64, P, c_int, P, P, c_int64, c_int, c_int, c_int, c_int, P],
     "liyab_gemm_mfma": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_gemm_mfma_dl": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
@@ -51,7 +51,7 @@ _SIGNATURES = {
                                 c_int, c_int, c_int, P],
     "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_int, c_int, P, P],
-    "liyab_gemm_skinny_ln": [P, P, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_skinny_ln": [P, c_int, c_int64, P, P, c_float, P, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],

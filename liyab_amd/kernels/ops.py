@@ -158,54 +158,57 @@ def add_rows_(x: torch.Tensor, table: torch.Tensor, rows: torch.Tensor) -> None:
     _lib.call("liyab_add_rows", x.data_ptr(), table.data_ptr(), dtype_code(table.dtype), rows.data_ptr(), n, d, _stream())
 
 
-def _part_sums(x: torch.Tensor, sums, what: str):
-    """Checks sums still to be added to the rows of x: (planes float32 [parts, rows of x, d],
-    bias float32 [d] or None). Returns what the launchers take."""
-    planes, bias = sums
-    _dev(planes, "partial sums")
-    if (planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != tuple(x.shape) or not planes.is_contiguous()
-            or not 1 <= planes.shape[0] <= 16):
-        raise KernelError(f"{what}: partial sums must be contiguous float32 [1..16, {x.shape[0]}, {x.shape[1]}], got {tuple(planes.shape)}")
-    _f32vec(bias, "bias of the partial sums", x.shape[1])
-    return planes.data_ptr(), planes.shape[0], planes.stride(0), _ptr(bias)
+def _planes(x: torch.Tensor, what: str):
+    """Rows given as they are, float32 [rows, d], or as a sum of planes, float32 [parts, rows, d]
+    (row r is x[0][r] + x[1][r] + ..., added in that order). Returns (pointer, parts, floats
+    between planes, rows, d)."""
+    _dev(x, what)
+    if x.dtype != torch.float32 or x.dim() not in (2, 3) or not x.is_contiguous():
+        raise KernelError(f"{what}: rows must be contiguous float32 [rows, d] or [parts, rows, d], got {tuple(x.shape)} {x.dtype}")
+    if x.dim() == 2:
+        return x.data_ptr(), 1, 0, x.shape[0], x.shape[1]
+    if not 1 <= x.shape[0] <= 16:
+        raise KernelError(f"{what}: {x.shape[0]} planes (1 to 16)")
+    return x.data_ptr(), x.shape[0], x.stride(0), x.shape[1], x.shape[2]
+
+
+def norm_takes_planes(d: int) -> bool:
+    """Whether the norm kernel adds planes up as it loads a row of this width (sum_parts first otherwise)."""
+    return d % 4 == 0 and d <= 2048
 
 
 def layernorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
-              eps: float, rows: Optional[torch.Tensor] = None, sums=None) -> None:
+              eps: float, rows: Optional[torch.Tensor] = None) -> None:
     """out[r] = LayerNorm(x[rows[r]] or x[r]); x float32 [*, d], out [n, d] float32 or bfloat16.
-    `sums` = (planes [parts, rows of x, d], bias [d] or None) are added to the rows first, bias
-    then planes in their order; without `rows`, x holds the sums afterwards (with `rows` it
-    must not be read again)."""
+    x may be a sum of planes [parts, *, d] (widths that `norm_takes_planes`): the planes are
+    added up, in their order, as a row is loaded."""
     _dev(out, "out")
-    _dev(x, "x")
+    ptr, n_parts, stride, x_rows, xd = _planes(x, "layernorm")
     n, d = out.shape
-    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
-        raise KernelError("layernorm: x must be contiguous float32 [*, d] and out contiguous [n, d]")
+    if xd != d or not out.is_contiguous():
+        raise KernelError("layernorm: x must have rows of d and out must be contiguous [n, d]")
     _f32vec(weight, "norm weight", d)
     _f32vec(bias, "norm bias", d)
     if rows is not None:
         _i32(rows, "rows", n)
-    elif x.shape[0] < n:
+    elif x_rows < n:
         raise KernelError("layernorm: fewer input rows than output rows")
-    if sums is None:
-        _lib.call("liyab_layernorm", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
+    if n_parts == 1:
+        _lib.call("liyab_layernorm", out.data_ptr(), dtype_code(out.dtype), ptr, _ptr(weight), _ptr(bias),
                   _ptr(rows), n, d, float(eps), _stream())
         return
-    if rows is None and x.shape[0] != n:
-        raise KernelError("layernorm: with sums to add, every row of x is normalised")
-    planes, n_parts, stride, pbias = _part_sums(x, sums, "layernorm")
-    _lib.call("liyab_layernorm_parts", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias),
-              _ptr(rows), n, d, float(eps), planes, n_parts, stride, pbias, x.shape[0], _stream())
+    _lib.call("liyab_layernorm_parts", out.data_ptr(), dtype_code(out.dtype), ptr, n_parts, stride, x_rows, _ptr(weight),
+              _ptr(bias), _ptr(rows), n, d, float(eps), _stream())
 
 
-def add_parts(x: torch.Tensor, sums) -> None:
-    """x += bias + planes[0] + planes[1] + ... for `sums` = (planes, bias), in the order the
-    norm kernel adds them."""
-    _dev(x, "x")
-    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
-        raise KernelError("add_parts: x must be contiguous float32 [rows, d]")
-    planes, n_parts, stride, pbias = _part_sums(x, sums, "add_parts")
-    _lib.call("liyab_add_parts", x.data_ptr(), x.shape[0], x.shape[1], planes, n_parts, stride, pbias, _stream())
+def sum_parts(out: torch.Tensor, planes: torch.Tensor) -> None:
+    """out = planes[0] + planes[1] + ..., in the order the norm kernels add them; out float32
+    [rows, d] (it may be planes[0])."""
+    _dev(out, "out")
+    ptr, n_parts, stride, x_rows, d = _planes(planes, "sum_parts")
+    if out.dtype != torch.float32 or tuple(out.shape) != (x_rows, d) or not out.is_contiguous():
+        raise KernelError(f"sum_parts: out must be contiguous float32 [{x_rows}, {d}]")
+    _lib.call("liyab_sum_parts", out.data_ptr(), x_rows, d, ptr, n_parts, stride, _stream())
 
 
 def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
@@ -394,20 +397,32 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _lib.call("liyab_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, ksplit, wide, mtile, ctypes.byref(e), _stream())
 
 
-def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, ksplit: int = 0) -> None:
-    """planes[p] = a . w^T summed over the p-th of planes.shape[0] parts of K (no bias): the
+def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+                      base: Optional[torch.Tensor] = None, ksplit: int = 0) -> None:
+    """planes[p] = a . w^T summed over the p-th of planes.shape[0] parts of K: the
     weight-streaming product cut over K, for few output features and a long K. a [M <= 64, K]
-    and w [N, K] bfloat16, planes float32 [parts, M, N]."""
+    and w [N, K] bfloat16, planes float32 [parts, M, N]. With `base` (float32 [M, N] or a sum
+    of planes [*, M, N], not overlapping `planes`) the first plane also takes `bias` and the
+    rows of `base`, so that the planes add up to base + a . w^T + bias."""
     lda = _rows(a, "a")
     M, K = a.shape
     _dev(w, "w")
     _dev(planes, "planes")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
         raise KernelError(f"gemm_skinny_parts: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
-    if planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != (M, w.shape[0]) or not planes.is_contiguous():
-        raise KernelError(f"gemm_skinny_parts: planes must be contiguous float32 [parts, {M}, {w.shape[0]}], got {tuple(planes.shape)}")
-    _lib.call("liyab_gemm_skinny_parts", a.data_ptr(), lda, w.data_ptr(), M, w.shape[0], K, planes.shape[0], ksplit,
-              planes.data_ptr(), planes.stride(0), _stream())
+    N = w.shape[0]
+    if planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != (M, N) or not planes.is_contiguous():
+        raise KernelError(f"gemm_skinny_parts: planes must be contiguous float32 [parts, {M}, {N}], got {tuple(planes.shape)}")
+    bptr, n_base, bstride = None, 0, 0
+    if base is not None:
+        bptr, n_base, bstride, b_rows, b_d = _planes(base, "gemm_skinny_parts: base")
+        if (b_rows, b_d) != (M, N):
+            raise KernelError(f"gemm_skinny_parts: base must have rows [{M}, {N}], got {tuple(base.shape)}")
+        _f32vec(bias, "bias", N)
+    elif bias is not None:
+        raise KernelError("gemm_skinny_parts: a bias needs the rows it is added to (base)")
+    _lib.call("liyab_gemm_skinny_parts", a.data_ptr(), lda, w.data_ptr(), M, N, K, planes.shape[0], ksplit,
+              planes.data_ptr(), planes.stride(0), _ptr(bias), bptr, n_base, bstride, _stream())
 
 
 def k_parts(M: int, N: int, K: int) -> int:
@@ -426,36 +441,29 @@ def k_parts(M: int, N: int, K: int) -> int:
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,
-                   w: torch.Tensor, bias: Optional[torch.Tensor], *, rows: Optional[torch.Tensor] = None,
-                   n_rows: Optional[int] = None, out=None, residual=None, epilogue: int = EPI_NONE, kv=None,
-                   ksplit: int = 0) -> None:
-    """gemm_skinny over LayerNorm(x[rows[m] or m]) of the float32 rows x [*, K], the norm computed
-    inside the product kernel."""
-    _dev(x, "x")
+                   w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, epilogue: int = EPI_NONE, kv=None) -> None:
+    """The weight-streaming product over LayerNorm(x) of the float32 rows x [M, K], or of a sum
+    of planes [parts, M, K], the norm computed inside the product kernel (`skinny_ln_takes`)."""
+    ptr, n_parts, stride, M, K = _planes(x, "gemm_skinny_ln")
     _dev(w, "w")
-    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
-        raise KernelError("gemm_skinny_ln: x must be contiguous float32 [*, K]")
-    K = x.shape[1]
-    M = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
     if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
         raise KernelError(f"gemm_skinny_ln: needs contiguous bfloat16 w [N, {K}], got {tuple(w.shape)} {w.dtype}")
-    if not skinny_ln_takes(M, K, 0):
+    if not skinny_ln_takes(M, K):
         raise KernelError(f"gemm_skinny_ln: {M} rows of {K} are outside what it takes")
+    if epilogue == EPI_RESIDUAL:
+        raise KernelError("gemm_skinny_ln: the residual epilogue is not taken")
     _f32vec(ln_weight, "norm weight", K)
     _f32vec(ln_bias, "norm bias", K)
-    if rows is not None:
-        _i32(rows, "rows", M)
     fake_a = torch.empty((M, 0), dtype=torch.bfloat16, device="meta")  # shapes only, for the epilogue's checks
-    e = _epilogue(fake_a, w, bias, out, residual, epilogue, kv)
+    e = _epilogue(fake_a, w, bias, out, None, epilogue, kv)
     e.exact = 0
-    _lib.call("liyab_gemm_skinny_ln", x.data_ptr(), _ptr(ln_weight), _ptr(ln_bias), _ptr(rows), float(eps),
-              w.data_ptr(), M, w.shape[0], K, ksplit, ctypes.byref(e), _stream())
+    _lib.call("liyab_gemm_skinny_ln", ptr, n_parts, stride, _ptr(ln_weight), _ptr(ln_bias), float(eps),
+              w.data_ptr(), M, w.shape[0], K, ctypes.byref(e), _stream())
 
 
-def skinny_ln_takes(M: int, K: int, N: int = 0) -> bool:
-    """Every workgroup (16 output features) repeats the norm of all rows, so it pays only while
-    the product has few workgroups."""
-    return 0 < M <= 16 and K % 8 == 0 and K <= 2048 and M * (K + 8) * 2 <= 65536 and N <= 8192
+def skinny_ln_takes(M: int, K: int) -> bool:
+    """What the product kernel with the norm inside takes: one tile of rows, a row in a wave's registers."""
+    return 0 < M <= 16 and K % 8 == 0 and K <= 2048
 
 
 def gemm_mfma_dl(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,

@@ -80,7 +80,7 @@ class DecoderModel:
         self.embedding.forward(ctx, x, position_table=fused)
         if self.residual_position is not None and fused is None:
             self.residual_position.add(ctx, x)
-        pending = None  # sums a layer has computed for x and left for the next reader of x to add
+        pending = None  # the stream as a SplitStream while a layer has left it split (x is then stale)
         for e in self.order:
             block = self.blocks[e.layer]
             args = (x, ctx, storage.layer(e.cache_layer), storage.state(e.cache_layer))
@@ -88,20 +88,19 @@ class DecoderModel:
                 pending = block.forward(*args, writes_cache=e.writes_cache, pending=pending)
             else:
                 if pending is not None:
-                    pending.settle(x)
+                    pending.settle()
                     pending = None
                 block.forward(*args, writes_cache=e.writes_cache)
         if ctx.n_logit_rows == 0:
-            return None  # nobody reads x again: pending sums are dropped
+            return None  # nobody reads the stream again
         if self.final_norm is not None:
             norm = self.final_norm
             kw = dict(rows=ctx.logit_rows, n_rows=ctx.n_logit_rows, name="head_in")
-            if pending is not None and getattr(norm, "takes_sums", False):
-                h = norm.forward(x, ctx, sums=pending.sums, **kw)
-            else:
-                if pending is not None:
-                    pending.settle(x)
-                h = norm.lazy(x, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(x, ctx, **kw)
+            rows = x
+            if pending is not None:
+                takes = getattr(norm, "takes_planes", None)
+                rows = pending.planes if takes is not None and takes(pending.planes) else pending.settle()
+            h = norm.lazy(rows, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(rows, ctx, **kw)
         else:
             raise NotImplementedError("a model without a final norm is not implemented")
         return self.head.forward(h, ctx)

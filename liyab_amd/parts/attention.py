@@ -9,7 +9,7 @@ import torch
 from ..cache.pages import KVSpec
 from ..cache.storage import LayerCache
 from ..kernels import ops
-from .base import StepContext
+from .base import StepContext, settled
 from .linear import linear, linear_deferred, paged_qkv_takes
 from .registry import register_mixer
 
@@ -50,13 +50,14 @@ class Attention:
     def state_spec(self):
         return None
 
-    defers = True  # forward(..., defer=True) may hand its result back as PendingSums
+    defers = True  # forward(..., defer=True) takes the stream split or whole and may hand it back split
 
     def forward(self, h: torch.Tensor, ctx: StepContext, cache: LayerCache, state, residual: torch.Tensor,
                 writes_cache: bool = True, defer: bool = False):
-        """Adds attention's output into `residual`; with `defer`, and where the output
-        projection runs faster cut over its inner dimension, returns the parts' sums as
-        PendingSums instead, for the next reader of the residual stream to add."""
+        """Adds attention's output into `residual`. With `defer`, `residual` may be a SplitStream,
+        and where the output projection runs faster cut over its inner dimension the stream
+        with the output added comes back as a SplitStream (None: added in place, to the
+        stream's own tensor)."""
         n = h.shape[0]
         ws = ctx.workspace
         group = ctx.groups[cache.group]
@@ -72,10 +73,10 @@ class Attention:
         att = ws.get("att", (n, self.q_dim), self.dtype)
         ops.attention(att, q[:, :self.q_dim] if q.shape[1] != self.q_dim else q, cache.k, cache.v, group.block_tables, ctx, n_head=self.n_head, scale=self.scale,
                       window=self.window)
-        pending = linear_deferred(att, self.out_weight, self.out_bias, ctx, "att_parts") if defer else None
-        if pending is None:
-            linear(att, self.out_weight, self.out_bias, residual=residual)
-        return pending
+        split = linear_deferred(att, self.out_weight, self.out_bias, ctx, "att_parts", residual) if defer else None
+        if split is None:
+            linear(att, self.out_weight, self.out_bias, residual=settled(residual))
+        return split
 
 
 register_mixer("attention", Attention)

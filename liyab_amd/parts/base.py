@@ -17,6 +17,11 @@ to a class constructed as `cls(spec, store, dtype)`):
   position:  where == "residual": add(ctx, x);  fused_table() -> table | None
   block:     cls(layer_spec, mixer, ffn, norm_mixer, norm_ffn); forward(x, ctx, cache, state, writes_cache)
 
+Optional, and only between parts that declare them: a mixer or feed-forward with `defers`
+may be handed the stream as a `SplitStream` and may return one instead of adding in place;
+a norm with `takes_planes` reads a split stream's planes; a block with `takes_pending` gets
+and returns the split stream. A part without these sees plain tensors only.
+
 `residual` is the float32 residual stream [n, d]; a part adds into it in
 place (the sum is 32-bit whatever the compute dtype), which lets an output
 projection fold the addition into its epilogue.
@@ -30,23 +35,28 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 
-class PendingSums:
-    """What a part has computed for the residual stream but not added to it yet: planes of
-    partial sums [parts, tokens, width] (float32) and a bias [width] or None. Whoever reads
-    the stream next adds them first, bias then planes in their order: a norm that can does
-    so as it loads its rows (`takes_sums`), anything else through `settle`."""
+class SplitStream:
+    """The residual stream as a sum of planes, float32 [parts, tokens, width]: its rows are
+    planes[0] + planes[1] + ..., added in that order. A product cut over its inner dimension
+    leaves the stream so: one plane of sums a part, the first of them also holding the bias
+    and the stream the product was added to. `home` is the stream's own tensor [tokens,
+    width], stale while the stream is split. Whoever reads the stream next adds the planes up
+    as it loads its rows if it can (a norm with `takes_planes`, a product cut over its inner
+    dimension in its turn); anything else gets `settle()`, which writes the sum to `home`."""
 
-    def __init__(self, planes, bias):
-        self.planes, self.bias = planes, bias
+    def __init__(self, planes, home):
+        self.planes, self.home = planes, home
 
-    @property
-    def sums(self):
-        return (self.planes, self.bias)
-
-    def settle(self, x) -> None:
+    def settle(self):
         from ..kernels import ops
 
-        ops.add_parts(x, self.sums)
+        ops.sum_parts(self.home, self.planes)
+        return self.home
+
+
+def settled(stream):
+    """The residual stream as one tensor, its planes added up first if it is split."""
+    return stream.settle() if isinstance(stream, SplitStream) else stream
 
 
 class Workspace:

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import StepContext
+from .base import SplitStream, StepContext, settled
 from .registry import register_block
 
 
@@ -16,40 +16,41 @@ class PreNormBlock:
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
 
-    takes_pending = True  # forward(..., pending=) takes sums the stream still lacks and may return such
+    takes_pending = True  # forward(..., pending=) takes the stream split and may return it split
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True, pending=None):
-        """`pending`: PendingSums that x still lacks (the previous layer's), added by this
-        layer's first norm as it reads x. Returns this layer's own, or None."""
-        if pending is not None and getattr(self.norm_mixer, "takes_sums", False):
-            h = self.norm_mixer.forward(x, ctx, sums=pending.sums)
-        else:
-            if pending is not None:
-                pending.settle(x)
-            h = self._normed(self.norm_mixer, x, ctx)
-        pending = None
+        """x: the residual stream's own tensor. `pending`: the stream as a SplitStream when the
+        previous layer left it split (x is then stale). Returns the stream as a SplitStream if
+        this layer leaves it split, else None (x holds it)."""
+        stream = pending if pending is not None else x
+        h, stream = self._normed(self.norm_mixer, stream, ctx)
         if getattr(self.mixer, "defers", False):
-            pending = self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache, defer=True)
+            stream = self.mixer.forward(h, ctx, cache, state, stream, writes_cache=writes_cache, defer=True) or x
         else:
-            self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
-        if self.ffn is None:
-            return pending
-        if pending is not None and getattr(self.norm_ffn, "takes_sums", False):
-            h = self.norm_ffn.forward(x, ctx, sums=pending.sums)
-        else:
-            if pending is not None:
-                pending.settle(x)
-            h = self._normed(self.norm_ffn, x, ctx)
-        if getattr(self.ffn, "defers", False):
-            return self.ffn.forward(h, ctx, x, defer=True)
-        self.ffn.forward(h, ctx, x)
-        return None
+            self.mixer.forward(h, ctx, cache, state, settled(stream), writes_cache=writes_cache)
+            stream = x
+        if self.ffn is not None:
+            h, stream = self._normed(self.norm_ffn, stream, ctx)
+            if getattr(self.ffn, "defers", False):
+                stream = self.ffn.forward(h, ctx, stream, defer=True) or x
+            else:
+                self.ffn.forward(h, ctx, settled(stream))
+                stream = x
+        return stream if isinstance(stream, SplitStream) else None
 
     @staticmethod
-    def _normed(norm, x, ctx):
-        """The norm's output, left pending when the norm allows it so that the next product
-        may fold it in (parts that need the rows call `as_tensor`)."""
-        return norm.lazy(x, ctx) if hasattr(norm, "lazy") else norm.forward(x, ctx)
+    def _normed(norm, stream, ctx):
+        """The norm of the stream and the stream as it is afterwards (settled if the norm cannot
+        read it split). The norm's output is left pending when the norm allows it, so that the
+        next product may fold it in (parts that need the rows call `as_tensor`)."""
+        rows = stream
+        if isinstance(stream, SplitStream):
+            takes = getattr(norm, "takes_planes", None)
+            if takes is not None and takes(stream.planes):
+                rows = stream.planes
+            else:
+                rows = stream = stream.settle()
+        return (norm.lazy(rows, ctx) if hasattr(norm, "lazy") else norm.forward(rows, ctx)), stream
 
 
 register_block("pre_norm", PreNormBlock)

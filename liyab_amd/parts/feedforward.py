@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import StepContext
+from .base import StepContext, settled
 from .linear import linear, linear_deferred
 from .registry import register_ffn
 
@@ -26,18 +26,19 @@ class DenseFFN:
         self.down_weight = store.fetch(t["down_weight"], (self.width, self.inner), "matrix")
         self.down_bias = store.fetch(t["down_bias"], (self.width,), "vector") if "down_bias" in t else None
 
-    defers = True  # forward(..., defer=True) may hand its result back as PendingSums
+    defers = True  # forward(..., defer=True) takes the stream split or whole and may hand it back split
 
     def forward(self, h, ctx: StepContext, residual: torch.Tensor, defer: bool = False):
-        """Adds the feed-forward's output into `residual`. With `defer`, and where the second
-        product runs faster cut over its inner dimension, the parts' sums come back as
-        PendingSums instead, for the next reader of the residual stream to add."""
+        """Adds the feed-forward's output into `residual`. With `defer`, `residual` may be a
+        SplitStream, and where the second product runs faster cut over its inner dimension the
+        stream with the output added comes back as a SplitStream (None: added in place, to
+        the stream's own tensor)."""
         inner = ctx.workspace.get("ffn_inner", (h.shape[0], self.inner), self.dtype)
         linear(h, self.up_weight, self.up_bias, out=inner, activation=self.activation)
-        pending = linear_deferred(inner, self.down_weight, self.down_bias, ctx, "ffn_parts") if defer else None
-        if pending is None:
-            linear(inner, self.down_weight, self.down_bias, residual=residual)
-        return pending
+        split = linear_deferred(inner, self.down_weight, self.down_bias, ctx, "ffn_parts", residual) if defer else None
+        if split is None:
+            linear(inner, self.down_weight, self.down_bias, residual=settled(residual))
+        return split
 
 
 register_ffn("dense_ffn", DenseFFN)

@@ -3,9 +3,9 @@
 W is [out, in], a row per output feature, the layout the reference works in
 (include/liyab/types.h:165-184; y = x . W^T, include/liyab/backend.h:35).
 The kernel is chosen here by dtype and shape; callers only say what they
-want computed. The first operand may be a pending norm (`Normed`): the norm
-runs first as its own kernel, unless FOLD_NORM asks for the product kernel
-that applies the norm itself where the shape allows it.
+want computed. The first operand may be a pending norm (`Normed`): where the
+shape allows it the product kernel applies the norm itself (FOLD_NORM),
+otherwise the norm runs first as its own kernel.
 """
 
 from __future__ import annotations
@@ -18,16 +18,18 @@ from ..kernels import ops
 from .norms import Normed
 
 
-# Folding the norm into a decode step's products saves a launch, but every workgroup of the
-# product then repeats the norm ahead of its multiplies. Measured at GPT-2 small's sizes the
-# standalone norm (a wave per row, 2.6 us) plus the plain product is faster: 464 against 506 us
-# a step at batch 1, 526 against 574 at batch 8. Off; the folded kernel stays available.
-FOLD_NORM = False
+# Folding the norm into a decode step's products saves a launch of the seven a layer has; every
+# workgroup of the product then repeats the norm of all rows ahead of its multiplies, which
+# pays while the rows are few.
+FOLD_NORM = True
+FOLD_NORM_ROWS = 16  # at most (the kernel's own limit is one tile of 16 rows)
 
 
-def _fuses(a, w: torch.Tensor) -> bool:
-    return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and w.dtype == torch.bfloat16
-            and a.x.dtype == torch.float32 and a.x.is_contiguous() and ops.skinny_ln_takes(a.n_rows, a.norm.width, w.shape[0]))
+def _fuses(a, w: torch.Tensor, residual) -> bool:
+    return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and residual is None
+            and a.rows is None and a._tensor is None and w.dtype == torch.bfloat16 and a.x.dtype == torch.float32
+            and a.x.is_contiguous() and a.n_rows <= FOLD_NORM_ROWS and w.shape[0] <= 8192
+            and ops.skinny_ln_takes(a.n_rows, a.norm.width))
 
 
 def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,
@@ -40,22 +42,27 @@ def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[to
         epilogue = ops.EPI_QKV_PAGED
     else:
         epilogue = ops.ACTIVATION_EPILOGUE[activation]
-    if _fuses(a, w):
+    if _fuses(a, w, residual):
         n = a.norm
-        ops.gemm_skinny_ln(a.x, n.weight, n.bias, n.eps, w, bias, rows=a.rows, n_rows=a.n_rows, out=out,
-                           residual=residual, epilogue=epilogue, kv=kv)
+        ops.gemm_skinny_ln(a.x, n.weight, n.bias, n.eps, w, bias, out=out, epilogue=epilogue, kv=kv)
         return
     if isinstance(a, Normed):
         a = a.tensor()
     ops.gemm(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
 
 
-def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name: str):
-    """a . w^T + bias as sums still to be added to the residual stream, or None where the
-    product is not worth cutting over its inner dimension (the caller then adds it through
-    `linear(..., residual=)`). The planes live in the step's workspace under `name` until the
-    next reader of the stream has added them."""
-    from .base import PendingSums
+def _overlap(a: torch.Tensor, b: torch.Tensor) -> bool:
+    a0, b0 = a.data_ptr(), b.data_ptr()
+    return a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
+
+
+def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name: str, stream):
+    """stream + a . w^T + bias as a split residual stream, or None where the product is not
+    worth cutting over its inner dimension (the caller then adds it through `linear(...,
+    residual=settled(stream))`). `stream` is the residual stream the product is added to, a
+    tensor or a SplitStream; the planes live in the step's workspace under `name` until the
+    next product cut this way writes its own under another name."""
+    from .base import SplitStream
 
     a = a.tensor() if isinstance(a, Normed) else a
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[0] > 64:
@@ -63,9 +70,13 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     parts = ops.k_parts(a.shape[0], w.shape[0], a.shape[1])
     if parts <= 1:
         return None
+    split = isinstance(stream, SplitStream)
+    base = stream.planes if split else stream
     planes = ctx.workspace.get(name, (parts, a.shape[0], w.shape[0]), torch.float32)
-    ops.gemm_skinny_parts(a, w, planes)
-    return PendingSums(planes, bias)
+    if _overlap(planes, base):
+        return None  # the stream's planes are where these would go
+    ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
+    return SplitStream(planes, stream.home if split else stream)
 
 
 def paged_qkv_takes(dtype: torch.dtype, k: int) -> bool:

@@ -18,7 +18,8 @@ class Normed:
 
     def __init__(self, norm, x: torch.Tensor, ctx: StepContext, rows=None, n_rows=None, name="normed"):
         self.norm, self.x, self.ctx, self.rows, self.name = norm, x, ctx, rows, name
-        self.n_rows = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        # x: the rows [n, d], or a sum of planes [parts, n, d] for a norm that `takes_planes`
+        self.n_rows = x.shape[-2] if rows is None else (n_rows if n_rows is not None else rows.numel())
         self._tensor = None
 
     @property
@@ -55,19 +56,21 @@ class LayerNorm:
         self.bias = store.fetch(b, (self.width,), "vector") if b is not None else None
 
     fusable = "layernorm"  # product kernels know how to fold this norm into their operand
-    takes_sums = True  # forward(..., sums=) adds pending partial sums to the rows as it loads them
+
+    def takes_planes(self, planes: torch.Tensor) -> bool:
+        """Whether forward() and lazy() take these planes [parts, n, d] of a split residual stream
+        in place of rows, adding them up as the rows are loaded."""
+        return ops.norm_takes_planes(self.width)
 
     def lazy(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
              n_rows: Optional[int] = None, name: str = "normed") -> Normed:
         return Normed(self, x, ctx, rows, n_rows, name)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
-                n_rows: Optional[int] = None, name: str = "normed", sums=None) -> torch.Tensor:
-        """`sums`: a PendingSums' (planes, bias), added to x's rows first. Without `rows` x
-        holds the sums afterwards; with `rows` it does not and must not be read again."""
-        n = x.shape[0] if rows is None else (n_rows if n_rows is not None else rows.numel())
+                n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:
+        n = x.shape[-2] if rows is None else (n_rows if n_rows is not None else rows.numel())
         out = ctx.workspace.get(name, (n, self.width), self.dtype)
-        ops.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows, sums=sums)
+        ops.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows)
         return out
 
 

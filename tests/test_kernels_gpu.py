@@ -71,44 +71,50 @@ def test_layernorm(ops, out_dtype, n, d, eps):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,d,parts,with_bias", [(1, 64, 1, True), (9, 96, 4, False), (16, 768, 4, True), (5, 1600, 2, True),
-                                                 (3, 777, 3, True), (7, 2052, 2, False), (6, 200, 16, True)])
-def test_layernorm_adds_pending_sums(ops, out_dtype, n, d, parts, with_bias):
-    """Rows that still lack a product's partial sums: the norm adds bias and planes as it loads
-    the rows and writes the sums back; over gathered rows it leaves x alone (widths that need
-    the general kernel get the sums in a pass of their own, in place); add_parts alone does
-    the same sum."""
+@pytest.mark.parametrize("n,d,parts", [(1, 64, 1), (9, 96, 4), (16, 768, 4), (5, 1600, 2), (7, 2048, 5), (6, 200, 16), (70, 768, 3)])
+def test_layernorm_over_rows_in_planes(ops, out_dtype, n, d, parts):
+    """Rows given as a sum of planes: the norm adds the planes up, in their order, as it loads a
+    row, also over gathered rows; sum_parts alone does the same sum (into a tensor of its own or
+    into the first plane); widths the kernel does not take in planes are refused."""
     tol = 1e-6 if out_dtype == torch.float32 else 5e-3
-    x = rnd(n, d, scale=3.0) + 1.5
-    planes = rnd(parts, n, d, seed=4, scale=0.7)
-    pbias = rnd(d, seed=5) if with_bias else None
+    planes = rnd(parts, n + 3, d, seed=4, scale=0.7)
+    planes[0] += 1.5
     w, b = rnd(d, seed=2) + 1.0, rnd(d, seed=3)
-    total = x.double() + planes.double().sum(0) + (pbias.double() if with_bias else 0)
+    total = planes.double().sum(0)
     want = torch.nn.functional.layer_norm(total, (d,), w.double(), b.double(), 1e-5)
     out = torch.empty(n, d, dtype=out_dtype, device=DEV)
-    x1 = x.clone()
-    ops.layernorm(out, x1, w, b, 1e-5, sums=(planes, pbias))
-    close(out, want, tol, "layernorm with sums")
-    close(x1, total, 1e-6, "rows written back")
-    x2 = x.clone()
-    ops.add_parts(x2, (planes, pbias))
-    assert torch.equal(x1, x2)  # the same order of additions
-    rows = torch.tensor([(i * 3) % n for i in range(n + 2)], dtype=torch.int32, device=DEV)  # names rows twice
+    before = planes.clone()
+    ops.layernorm(out, planes, w, b, 1e-5)
+    close(out, want[:n], tol, "layernorm over planes")
+    assert torch.equal(planes, before)  # the planes stay as they are
+    summed = torch.empty(n + 3, d, device=DEV)
+    ops.sum_parts(summed, planes)
+    close(summed, total, 1e-6, "sum of the planes")
+    whole = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    ops.layernorm(whole, summed, w, b, 1e-5)
+    assert torch.equal(whole, out)  # the same order of additions
+    rows = torch.tensor([(i * 3) % (n + 3) for i in range(n + 2)], dtype=torch.int32, device=DEV)  # names rows twice
     out = torch.empty(n + 2, d, dtype=out_dtype, device=DEV)
-    x3 = x.clone()
-    ops.layernorm(out, x3, w, b, 1e-5, rows=rows, sums=(planes, pbias))
-    close(out, want[rows.long()], tol, "gathered layernorm with sums")
-    wave_kernel = d % 4 == 0 and d <= 2048
-    assert torch.equal(x3, x if wave_kernel else x2)
-    with pytest.raises(Exception, match="partial sums"):
-        ops.layernorm(out[:n], x, w, b, 1e-5, sums=(planes[:, :, :-1], pbias))
+    ops.layernorm(out, planes, w, b, 1e-5, rows=rows)
+    close(out, want[rows.long()], tol, "gathered layernorm over planes")
+    ops.sum_parts(planes[0], planes)
+    assert torch.equal(planes[0], summed)
+    if parts > 1:
+        odd = rnd(parts, 3, 777, seed=6)
+        assert not ops.norm_takes_planes(777)
+        with pytest.raises(Exception, match="planes"):
+            ops.layernorm(torch.empty(3, 777, device=DEV), odd, rnd(777), rnd(777), 1e-5)
+    with pytest.raises(Exception, match="rows of d"):
+        ops.layernorm(torch.empty(n, d, device=DEV), planes[:, :, :-4].contiguous(), w, b, 1e-5)
 
 
 @pytest.mark.parametrize("M,N,K,parts", [(1, 64, 128, 2), (8, 768, 3072, 4), (16, 100, 200, 2), (5, 1600, 6400, 2), (40, 50, 448, 7),
                                          (64, 264, 1600, 3), (3, 40, 64, 1), (11, 130, 1032, 4)])
 def test_gemm_skinny_parts(ops, M, N, K, parts):
     """The product cut over K: plane p holds the sums over the p-th part of K (whole units of
-    64, the last one shorter), no bias; the planes add up to the product."""
+    64, the last one shorter); the planes add up to the product. With rows to add to (a tensor
+    or planes of their own), the first plane also takes them and the bias, and the planes add
+    up to rows + product + bias."""
     a, w = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16)
     planes = torch.full((parts, M, N), float("nan"), device=DEV)
     ops.gemm_skinny_parts(a, w, planes)
@@ -117,9 +123,25 @@ def test_gemm_skinny_parts(ops, M, N, K, parts):
     for q in range(parts):
         lo, hi = q * part_k, min(K, (q + 1) * part_k)
         close(planes[q], a[:, lo:hi].double() @ w[:, lo:hi].double().t(), 1e-5, f"part {q}")
-    close(planes.sum(0), a.double() @ w.double().t(), 1e-5, "sum of the parts")
+    product = a.double() @ w.double().t()
+    close(planes.sum(0), product, 1e-5, "sum of the parts")
+    bias = rnd(N, seed=7)
+    for n_base in (0, 1, 3, 6):
+        base = rnd(M, N, seed=8, scale=3.0) if n_base == 0 else rnd(n_base, M, N, seed=9, scale=3.0)
+        for with_bias in (True, False):
+            based = torch.full((parts, M, N), float("nan"), device=DEV)
+            ops.gemm_skinny_parts(a, w, based, bias=bias if with_bias else None, base=base)
+            assert torch.equal(based[1:], planes[1:])
+            rows = base.double() if n_base == 0 else base.double().sum(0)
+            want0 = planes[0].double() + rows + (bias.double() if with_bias else 0)
+            close(based[0], want0, 1e-6, f"first plane over {n_base} planes of rows")
+            close(based.double().sum(0), product + rows + (bias.double() if with_bias else 0), 1e-5, "sum with rows")
     with pytest.raises(Exception, match="parts"):
         ops.gemm_skinny_parts(a, w, torch.empty(K // 64 + 2, M, N, device=DEV))
+    with pytest.raises(Exception, match="bias needs"):
+        ops.gemm_skinny_parts(a, w, planes, bias=bias)
+    with pytest.raises(Exception, match="overlap"):
+        ops.gemm_skinny_parts(a, w, planes, base=planes[:1])
 
 
 def gemm_reference(a, w, bias, epilogue, residual=None):
@@ -201,28 +223,33 @@ def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
             close(out, gemm_reference(a, w, bias, epilogue), tol, f"gemm bf16 {epilogue} {kernel} -> {out_dtype}")
 
 
-@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
-@pytest.mark.parametrize("M,N,K,eps", [(1, 64, 64, 1e-5), (8, 2304, 768, 1e-5), (16, 100, 1600, 1e-6), (5, 777, 144, 1e-5), (3, 50, 2048, 1e-3)])
-def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, epilogue):
-    x = rnd(M + 4, K, scale=2.0) + 0.5
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf"])
+@pytest.mark.parametrize("M,N,K,eps,parts", [(1, 64, 64, 1e-5, 1), (8, 2304, 768, 1e-5, 4), (16, 100, 1600, 1e-6, 2), (5, 777, 144, 1e-5, 3),
+                                             (3, 50, 2048, 1e-3, 5), (13, 520, 1024, 1e-5, 1), (9, 3072, 768, 1e-5, 2), (16, 48, 96, 1e-6, 16)])
+def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, parts, epilogue):
+    """The product kernel that normalises its own rows, given whole or as a sum of planes: the
+    same bits as the standalone norm followed by the streaming product."""
+    planes = rnd(parts, M, K, scale=2.0)
+    planes[0] += 0.5
     lw, lb = rnd(K, seed=5) + 1.0, rnd(K, seed=6)
     w, bias = rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
-    rows = torch.tensor([(3 * i + 1) % (M + 4) for i in range(M)], dtype=torch.int32, device=DEV)
-    for use_rows in (False, True):
-        src = x[rows.long()] if use_rows else x[:M]
-        h = torch.nn.functional.layer_norm(src.double(), (K,), lw.double(), lb.double(), eps).to(torch.bfloat16)
-        kw = dict(rows=rows) if use_rows else {}
-        xin = x if use_rows else x[:M].contiguous()
-        if epilogue == "residual":
-            res = rnd(M, N, seed=3)
-            want = gemm_reference(h, w, bias, epilogue, res)
-            ops.gemm_skinny_ln(xin, lw, lb, eps, w, bias, residual=res, epilogue=ops.EPI_RESIDUAL, **kw)
-            close(res, want, 2e-3, "gemm+ln residual")
-        else:
-            out = torch.empty(M, N, device=DEV)
-            ops.gemm_skinny_ln(xin, lw, lb, eps, w, bias, out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue], **kw)
-            # the folded norm rounds to bfloat16 where the standalone kernel does: allow one ulp of the operand
-            close(out, gemm_reference(h, w, bias, epilogue), 4e-3, f"gemm+ln {epilogue}")
+    x = planes if parts > 1 else planes[0]
+    h = torch.nn.functional.layer_norm(planes.double().sum(0), (K,), lw.double(), lb.double(), eps).to(torch.bfloat16)
+    epi = ops.ACTIVATION_EPILOGUE[epilogue]
+    for out_dtype in (torch.float32, torch.bfloat16):
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=epi)
+        # the folded norm rounds to bfloat16 where the standalone kernel does: allow one ulp of the operand
+        close(out, gemm_reference(h, w, bias, epilogue), 4e-3 if out_dtype == torch.float32 else 8e-3, f"gemm+ln {epilogue}")
+        normed = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+        ops.layernorm(normed, x, lw, lb, eps)
+        two = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops.gemm_skinny(normed, w, bias, out=two, epilogue=epi, ksplit=8, wide=0, mtile=1)
+        assert torch.equal(out, two)
+    with pytest.raises(Exception, match="residual"):
+        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=ops.EPI_RESIDUAL)
+    with pytest.raises(Exception, match="outside"):
+        ops.gemm_skinny_ln(rnd(17, K), lw, lb, eps, w, bias, out=torch.empty(17, N, device=DEV))
 
 
 def test_gemm_strided_rows_and_refusals(ops):

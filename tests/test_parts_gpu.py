@@ -174,13 +174,13 @@ def test_norm_alone(parts):
     core.close("n")
 
 
-@pytest.mark.parametrize("lazy", [False, True, "folded"])
+@pytest.mark.parametrize("lazy", [False, True, "unfolded"])
 def test_feed_forward_alone(parts, lazy, monkeypatch):
     from liyab_amd.engine import StepItem
     from liyab_amd.parts import linear
 
-    if lazy == "folded":  # the product kernel that applies a pending norm itself (off by default)
-        monkeypatch.setattr(linear, "FOLD_NORM", True)
+    if lazy == "unfolded":  # without the product kernel that applies a pending norm itself
+        monkeypatch.setattr(linear, "FOLD_NORM", False)
     p, dtype = parts
     core = p.core
     core.open("f")
@@ -195,13 +195,17 @@ def test_feed_forward_alone(parts, lazy, monkeypatch):
     core.close("f")
 
 
-@pytest.mark.parametrize("reader", ["norm", "gathering norm", "settle"])
-def test_feed_forward_deferred(parts, reader, monkeypatch):
-    """The feed-forward's second product cut over its inner dimension: the parts' sums come
-    back pending, and the next reader of the stream adds them: a norm as it loads its rows
-    (writing them back), a norm over gathered rows (not writing back), or a pass of its own."""
+@pytest.mark.parametrize("reader", ["norm", "gathering norm", "settle", "product"])
+@pytest.mark.parametrize("split_before", [False, True])
+def test_feed_forward_deferred(parts, reader, split_before, monkeypatch):
+    """The feed-forward's second product cut over its inner dimension: the stream comes back
+    split into planes (the stream's own tensor untouched), and the next reader adds them up: a
+    norm as it loads its rows, a norm over gathered rows, a product with the norm folded in, or
+    a pass of its own into the stream's tensor. The stream may have been split already."""
     from liyab_amd.engine import StepItem
     from liyab_amd.kernels import ops
+    from liyab_amd.parts.base import SplitStream
+    from liyab_amd.parts.linear import linear
 
     p, dtype = parts
     if dtype != "bfloat16":
@@ -213,23 +217,33 @@ def test_feed_forward_deferred(parts, reader, monkeypatch):
     rng = np.random.default_rng(2)
     x = rand(rng, 11, p.d, scale=1.5).to(DEV)
     residual = rand(rng, 11, p.d).to(DEV)
-    before = residual.clone()
     want = f64(residual.cpu()) + plain_ffn(plain_norm(f64(x.cpu()), p.tw, "n2", p.eps), p.tw, "f", p.act)
-    pending = p.block.ffn.forward(p.block.norm_ffn.forward(x, ctx), ctx, residual, defer=True)
-    assert pending is not None and pending.planes.shape == (3, 11, p.d) and torch.equal(residual, before)
+    stream = residual
+    if split_before:  # the stream arrives as two planes that add up to `residual`; its tensor is stale
+        half = rand(rng, 11, p.d).to(DEV)
+        stream = SplitStream(torch.stack([residual - half, half]), torch.full_like(residual, float("nan")))
+    home = stream.home if split_before else residual
+    before = home.clone()
+    split = p.block.ffn.forward(p.block.norm_ffn.forward(x, ctx), ctx, stream, defer=True)
+    assert isinstance(split, SplitStream) and split.planes.shape == (3, 11, p.d) and split.home is home
+    assert split_before or torch.equal(home, before)  # untouched (NaN never equals itself)
     norm = p.block.norm_mixer
-    if reader == "settle":
-        pending.settle(residual)
-    elif reader == "norm":
-        got = norm.forward(residual, ctx, sums=pending.sums).float().cpu().numpy()
+    assert norm.takes_planes(split.planes)
+    if reader == "norm":
+        got = norm.forward(split.planes, ctx).float().cpu().numpy()
         assert tt.rel_err(got, plain_norm(want, p.tw, "n1", p.eps)) < 1e-2
-    else:
+    elif reader == "gathering norm":
         rows = torch.tensor([7, 0, 7, 10], dtype=torch.int32, device=DEV)
-        got = norm.forward(residual, ctx, rows=rows, sums=pending.sums).float().cpu().numpy()
+        got = norm.forward(split.planes, ctx, rows=rows).float().cpu().numpy()
         assert tt.rel_err(got, plain_norm(want[[7, 0, 7, 10]], p.tw, "n1", p.eps)) < 1e-2
-        assert torch.equal(residual, before)  # gathered rows are not written back
-        pending.settle(residual)
-    assert tt.rel_err(residual.cpu().numpy(), want) < 1e-2
+    elif reader == "product":
+        w = rand(rng, 24, p.d).to(DEV).to(torch.bfloat16)
+        out = torch.empty(11, 24, dtype=torch.bfloat16, device=DEV)
+        linear(norm.lazy(split.planes, ctx), w, None, out=out)
+        ref = plain_norm(want, p.tw, "n1", p.eps) @ f64(w.float().cpu()).T
+        assert tt.rel_err(out.float().cpu().numpy(), ref) < 2e-2
+    assert split.settle() is home
+    assert tt.rel_err(home.cpu().numpy(), want) < 1e-2
     core.close("f")
 
 
@@ -423,7 +437,7 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
 
 
 class BareNorm:
-    """A LayerNorm that knows nothing of pending sums or pending norms (no `takes_sums`, no `lazy`)."""
+    """A LayerNorm that knows nothing of split streams or pending norms (no `takes_planes`, no `lazy`)."""
 
     def __init__(self, spec, store, dtype):
         self.width, self.eps, self.dtype = spec.width, float(spec.eps), dtype
@@ -451,13 +465,13 @@ class BareBlock:
             self.ffn.forward(self.norm_ffn.forward(x, ctx), ctx, x)
 
 
-def test_pending_sums_reach_parts_that_cannot_take_them(monkeypatch):
-    """Products cut over K leave their sums pending for the next reader of the residual
-    stream. Here the cut is forced at the toy model's small sizes; layer 1's second norm (after
-    the attention whose projection is cut) is one that cannot add sums, and layer 2's block
-    (after layer 1's cut feed-forward) one that cannot take them: the sums are settled before
-    those parts run; the last layer's go to the final norm over gathered rows; the logits stay
-    those of the plain model."""
+def test_split_streams_reach_parts_that_cannot_take_them(monkeypatch):
+    """Products cut over K leave the residual stream split into planes for its next reader.
+    Here the cut is forced at the toy model's small sizes; layer 1's second norm (after the
+    attention whose projection is cut) is one that cannot read planes, and layer 2's block
+    (after layer 1's cut feed-forward) one that cannot take a split stream: the planes are
+    added up before those parts run; the last layer's go to the final norm over gathered rows;
+    the logits stay those of the plain model."""
     import dataclasses
 
     from liyab_amd.engine import EngineCore
