@@ -162,8 +162,9 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = float_to_bf16(st.acc[e] * inv);
         } else {
-            // partials [token slot][head][split][hd + 2]: values, then maximum and sum
-            float* p = partials + ((static_cast<int64_t>(blockIdx.x) * n_head + h) * n_splits + z) * (hd + 2);
+            // partials [token slot][head][split][hd + 4]: values, then maximum and sum (and two
+            // unused, which keep every split's values 16-byte aligned)
+            float* p = partials + ((static_cast<int64_t>(blockIdx.x) * n_head + h) * n_splits + z) * (hd + 4);
 #pragma unroll
             for (int e = 0; e < 8; ++e) p[c * 8 + e] = st.acc[e];
             if (c == 0) {
@@ -180,16 +181,16 @@ __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_str
     const int slot = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
     if (e >= hd) return;
     const int t = tok_list != nullptr ? tok_list[slot] : slot;
-    const float* p = partials + (static_cast<int64_t>(slot) * n_head + h) * n_splits * (hd + 2);
+    const float* p = partials + (static_cast<int64_t>(slot) * n_head + h) * n_splits * (hd + 4);
     float M = -INFINITY;
-    for (int z = 0; z < n_splits; ++z) M = fmaxf(M, p[z * (hd + 2) + hd]);
+    for (int z = 0; z < n_splits; ++z) M = fmaxf(M, p[z * (hd + 4) + hd]);
     float sum = 0.0f, o = 0.0f;
     for (int z = 0; z < n_splits; ++z) {
-        const float m = p[z * (hd + 2) + hd];
+        const float m = p[z * (hd + 4) + hd];
         if (m == -INFINITY) continue;
         const float w = __expf(m - M);
-        sum += w * p[z * (hd + 2) + hd + 1];
-        o += w * p[z * (hd + 2) + e];
+        sum += w * p[z * (hd + 4) + hd + 1];
+        o += w * p[z * (hd + 4) + e];
     }
     out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = float_to_bf16(o / sum);
 }
@@ -199,13 +200,17 @@ __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_str
 using namespace liyab;
 
 // Tokens tok_list[0..n) (or 0..n-1 when tok_list is null), each on its own. `partials` must hold
-// n * n_head * n_splits * (hd + 2) floats when n_splits > 1.
+// n * n_head * n_splits * (hd + 4) floats when n_splits > 1. With `leave_splits` (n_splits > 1)
+// the splits are not merged and `out` is not written: partials[token slot][head][split] holds
+// hd weighted values, then the split's maximum and sum (an empty split: -inf and 0), for a
+// reader that merges them as it loads them (the output projection cut over its inner dimension).
 extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                       const void* vc, const int* block_tables, int max_blocks, const int* tok_list,
                                       const int* tok_seq, const int* tok_pos, int n, float scale, int window,
                                       int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
-                                      int rows_are_requests, float* partials, hipStream_t stream) {
-    LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
+                                      int rows_are_requests, float* partials, int leave_splits, hipStream_t stream) {
+    LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
+    LIYAB_REQUIRE(!leave_splits || n_splits > 1, "attention_decode: splits are left only when there are several");
     LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
     LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
     LIYAB_REQUIRE(hd >= 8 && hd <= 256 && hd % 8 == 0, "attention_decode: head size %d is not a multiple of 8 in 8..256", hd);
@@ -247,9 +252,22 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     else LIYAB_GO(32);
 #undef LIYAB_GO
     if (int rc = check_launch("attention_decode")) return rc;
-    if (n_splits > 1) {
+    if (n_splits > 1 && !leave_splits) {
         attention_merge_kernel<<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits);
         return check_launch("attention_merge");
     }
     return 0;
+}
+
+// out[m, h * hd + e] = the splits of (m, h) merged in split order: for splits that
+// liyab_attention_decode left unmerged and no reader takes as they are.
+extern "C" int liyab_attention_merge(void* out, int64_t out_stride, const float* partials, int n, int n_head, int hd,
+                                     int n_splits, hipStream_t stream) {
+    LIYAB_REQUIRE(out && partials, "attention_merge: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_head <= 65535 && hd > 0 && hd <= 1024 && n_splits >= 1, "attention_merge: bad sizes");
+    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd, "attention_merge: the row stride is shorter than heads x head size");
+    if (n == 0) return 0;
+    attention_merge_kernel<<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, nullptr, partials,
+                                                                                 n_head, hd, n_splits);
+    return check_launch("attention_merge");
 }

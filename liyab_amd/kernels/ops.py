@@ -425,6 +425,42 @@ def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *,
               planes.data_ptr(), planes.stride(0), _ptr(bias), bptr, n_base, bstride, _stream())
 
 
+def gemm_att_parts(partials: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+                   base: Optional[torch.Tensor] = None) -> None:
+    """The product cut over K (as `gemm_skinny_parts`) whose first operand is attention's output
+    still in splits: partials float32 [M <= 16, heads, splits <= 8, head size + 4] as
+    `attention_decode(..., leave_splits=True)` leaves them, merged as they are loaded.
+    w [N, heads * head size] bfloat16, planes float32 [parts, M, N]."""
+    _dev(partials, "partials")
+    _dev(w, "w")
+    _dev(planes, "planes")
+    if partials.dtype != torch.float32 or partials.dim() != 4 or not partials.is_contiguous():
+        raise KernelError(f"gemm_att_parts: partials must be contiguous float32 [M, heads, splits, head size + 4], got {tuple(partials.shape)}")
+    M, H, S, hd4 = partials.shape
+    K = H * (hd4 - 4)
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_att_parts: needs contiguous bfloat16 w [N, {K}], got {tuple(w.shape)} {w.dtype}")
+    N = w.shape[0]
+    if not att_parts_takes(M, S, hd4 - 4):
+        raise KernelError(f"gemm_att_parts: {M} rows in {S} splits of heads of {hd4 - 4} are outside what it takes")
+    if planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != (M, N) or not planes.is_contiguous():
+        raise KernelError(f"gemm_att_parts: planes must be contiguous float32 [parts, {M}, {N}], got {tuple(planes.shape)}")
+    bptr, n_base, bstride = None, 0, 0
+    if base is not None:
+        bptr, n_base, bstride, b_rows, b_d = _planes(base, "gemm_att_parts: base")
+        if (b_rows, b_d) != (M, N):
+            raise KernelError(f"gemm_att_parts: base must have rows [{M}, {N}], got {tuple(base.shape)}")
+        _f32vec(bias, "bias", N)
+    elif bias is not None:
+        raise KernelError("gemm_att_parts: a bias needs the rows it is added to (base)")
+    _lib.call("liyab_gemm_att_parts", partials.data_ptr(), S, H, hd4 - 4, w.data_ptr(), M, N, planes.shape[0],
+              planes.data_ptr(), planes.stride(0), _ptr(bias), bptr, n_base, bstride, _stream())
+
+
+def att_parts_takes(M: int, splits: int, hd: int) -> bool:
+    return 0 < M <= 16 and 1 <= splits <= 8 and hd % 8 == 0 and 8 <= hd <= 256
+
+
 def k_parts(M: int, N: int, K: int) -> int:
     """Into how many parts of K the weight-streaming product is best cut (1: not at all). With
     few output features a product fills a fraction of the chip's compute units, and a long K
@@ -522,10 +558,13 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
-                     rows_are_requests: bool = False) -> None:
+                     rows_are_requests: bool = False, leave_splits: bool = False) -> None:
     """Each token on its own over its request's bfloat16 cache, its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
-    request t (every request brings one token), which saves the kernel a lookup."""
+    request t (every request brings one token), which saves the kernel a lookup. With
+    `leave_splits` (several splits) `out` is not written: `partials`, viewed as [tokens, heads,
+    splits, head size + 4], keeps each split's weighted values, maximum and sum for a reader
+    that merges them (`gemm_att_parts`)."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
     _, hkv, page, hd = k_cache.shape
@@ -545,14 +584,29 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
         _i32(tok_list, "tok_list", n)
     elif n != rows:
         raise KernelError("attention_decode: n_tokens needs tok_list")
+    if leave_splits and n_splits <= 1:
+        raise KernelError("attention_decode: splits are left only when there are several")
     if n_splits > 1:
-        need = n * n_head * n_splits * (hd + 2)
+        need = n * n_head * n_splits * (hd + 4)
         if partials is None or partials.dtype != torch.float32 or partials.numel() < need or not partials.is_contiguous():
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
               n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, 1 if rows_are_requests else 0,
-              _ptr(partials), _stream())
+              _ptr(partials), 1 if leave_splits else 0, _stream())
+
+
+def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
+    """out [tokens, heads * head size] bfloat16 = the splits that `attention_decode(...,
+    leave_splits=True)` left in partials [tokens, heads, splits, head size + 4], merged in split order."""
+    _dev(partials, "partials")
+    os_ = _rows(out, "out")
+    if partials.dtype != torch.float32 or partials.dim() != 4 or not partials.is_contiguous():
+        raise KernelError("attention_merge: partials must be contiguous float32 [tokens, heads, splits, head size + 4]")
+    n, H, S, hd4 = partials.shape
+    if out.dtype != torch.bfloat16 or tuple(out.shape) != (n, H * (hd4 - 4)):
+        raise KernelError(f"attention_merge: out must be bfloat16 [{n}, {H * (hd4 - 4)}]")
+    _lib.call("liyab_attention_merge", out.data_ptr(), os_, partials.data_ptr(), n, H, hd4 - 4, S, _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -596,10 +650,24 @@ def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
     return max(1, min(context_bucket // 2048, 32)), 16
 
 
+def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int) -> int:
+    """Into how many splits a (token, head) pair's keys are cut when whoever reads attention's
+    output merges the splits itself (1: not at all): until the workgroups cover the chip, a split
+    keeping 128 keys or more of the longest context."""
+    pairs = max(1, n_tokens * n_head)
+    splits = 1
+    while splits < 8 and pairs * splits < 256 and context_bucket // (2 * splits) >= 128:
+        splits *= 2
+    return splits
+
+
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-              block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0) -> None:
+              block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0,
+              splits_ok: bool = False) -> Optional[torch.Tensor]:
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
-    is chosen from the step's shape (`ctx` is the step's StepContext)."""
+    is chosen from the step's shape (`ctx` is the step's StepContext). With `splits_ok`, a
+    step of few tokens may leave `out` unwritten and return the splits of each (token, head)
+    pair instead, float32 [tokens, heads, splits, head size + 4], for `gemm_att_parts`."""
     hd = k_cache.shape[3]
     host = ctx.host
     fast = q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and out.stride(0) % 8 == 0
@@ -608,15 +676,23 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         splits, waves = decode_plan(n, n_head, host.context_bucket)
         partials = None
         if splits > 1:
-            partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 2),), torch.float32)
+            partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32)
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
                          scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
                          rows_are_requests=tok_list is None and host.max_q_len == 1)
 
     if fast and host.attention_mode == "decode" and block_tables.shape[1] <= 2048:
-        decode(None, out.shape[0])
-        return
+        n = out.shape[0]
+        splits = decode_split_plan(n, n_head, host.context_bucket) if splits_ok else 1
+        if splits > 1 and att_parts_takes(n, splits, hd):
+            partials = ctx.workspace.get("attn_partials", (n, n_head, splits, hd + 4), torch.float32)
+            attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
+                             scale=scale, window=window, n_splits=splits, partials=partials, waves=4,
+                             rows_are_requests=host.max_q_len == 1, leave_splits=True)
+            return partials
+        decode(None, n)
+        return None
     if fast and prefill_takes(hd) and scale > 0 and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
         # long portions in tiles on the matrix cores, the short ones token by token
         if host.n_attn_tiles:

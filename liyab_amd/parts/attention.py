@@ -71,10 +71,15 @@ class Attention:
             if writes_cache:
                 ops.kv_write(cache.k, cache.v, q, self.q_dim, self.q_dim + self.kv_dim, group.slots)
         att = ws.get("att", (n, self.q_dim), self.dtype)
-        ops.attention(att, q[:, :self.q_dim] if q.shape[1] != self.q_dim else q, cache.k, cache.v, group.block_tables, ctx, n_head=self.n_head, scale=self.scale,
-                      window=self.window)
-        split = linear_deferred(att, self.out_weight, self.out_bias, ctx, "att_parts", residual) if defer else None
+        # with few tokens attention may leave each (token, head) pair's keys cut into splits, for
+        # an output projection that is cut over its inner dimension and merges them as it loads
+        cut = defer and self.dtype == torch.bfloat16 and ops.k_parts(n, self.width, self.q_dim) > 1
+        splits = ops.attention(att, q[:, :self.q_dim] if q.shape[1] != self.q_dim else q, cache.k, cache.v, group.block_tables, ctx,
+                               n_head=self.n_head, scale=self.scale, window=self.window, splits_ok=cut)
+        split = linear_deferred(splits if splits is not None else att, self.out_weight, self.out_bias, ctx, "att_parts", residual) if defer else None
         if split is None:
+            if splits is not None:
+                ops.attention_merge(att, splits)
             linear(att, self.out_weight, self.out_bias, residual=settled(residual))
         return split
 

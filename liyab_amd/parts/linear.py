@@ -57,7 +57,8 @@ def _overlap(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name: str, stream):
-    """stream + a . w^T + bias as a split residual stream, or None where the product is not
+    """stream + a . w^T + bias as a split residual stream (`a` may be attention's output still
+    in splits, float32 [tokens, heads, splits, head size + 4]), or None where the product is not
     worth cutting over its inner dimension (the caller then adds it through `linear(...,
     residual=settled(stream))`). `stream` is the residual stream the product is added to, a
     tensor or a SplitStream; the planes live in the step's workspace under `name` until the
@@ -65,17 +66,22 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     from .base import SplitStream
 
     a = a.tensor() if isinstance(a, Normed) else a
-    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[0] > 64:
+    in_splits = a.dim() == 4  # attention's output as its splits [tokens, heads, splits, head size + 4]
+    M, K = (a.shape[0], a.shape[1] * (a.shape[3] - 4)) if in_splits else a.shape
+    if (a.dtype != torch.bfloat16 and not in_splits) or w.dtype != torch.bfloat16 or M > 64:
         return None
-    parts = ops.k_parts(a.shape[0], w.shape[0], a.shape[1])
+    parts = ops.k_parts(M, w.shape[0], K)
     if parts <= 1:
         return None
     split = isinstance(stream, SplitStream)
     base = stream.planes if split else stream
-    planes = ctx.workspace.get(name, (parts, a.shape[0], w.shape[0]), torch.float32)
+    planes = ctx.workspace.get(name, (parts, M, w.shape[0]), torch.float32)
     if _overlap(planes, base):
         return None  # the stream's planes are where these would go
-    ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
+    if in_splits:
+        ops.gemm_att_parts(a, w, planes, bias=bias, base=base)
+    else:
+        ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
     return SplitStream(planes, stream.home if split else stream)
 
 

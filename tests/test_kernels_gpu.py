@@ -349,7 +349,7 @@ def run_attention(ops, case, H, hd, scale, window, kernel, splits=1, tok_list=No
         ops.attention_prefill(out, qv, kc, vc, bt, wk, len(work) // 4, n_head=H, scale=scale, window=window, tile=tile,
                               ksplit=ksplit)
     elif kernel == "decode":
-        partials = torch.empty(case["n"] * H * splits * (hd + 2), device=DEV) if splits > 1 else None
+        partials = torch.empty(case["n"] * H * splits * (hd + 4), device=DEV) if splits > 1 else None
         tl = torch.tensor(tok_list, dtype=torch.int32, device=DEV) if tok_list is not None else None
         ops.attention_decode(out, qv, kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
                              n_splits=splits, partials=partials, tok_list=tl, waves=waves,
@@ -395,6 +395,54 @@ def test_attention_decode(ops, case_id, splits, waves, window):
         rows = list(range(case["n"]))[::2]
         part = run_attention(ops, case, H, hd, scale, window, "decode", splits, tok_list=rows, waves=waves)
         assert torch.equal(part[rows], out[rows]) and (part[1::2] == 0).all()
+
+
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("splits", [2, 4, 7, 8])
+@pytest.mark.parametrize("case_id", [0, 1, 3, 5, 6])
+def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window):
+    """Attention that leaves each (token, head) pair's keys in splits, and the projection cut
+    over its inner dimension that merges them as it loads them: the planes add up to rows +
+    attention . W^T + bias; the merge kernel gives attention's output from the same splits.
+    Contexts shorter than the number of splits leave splits empty."""
+    ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
+    scale = 0.7 / math.sqrt(hd)
+    n = case["n"]
+    dev = lambda x: x.to(DEV)  # noqa: E731
+    q, kc, vc, bt = dev(case["q"]), dev(case["kc"]), dev(case["vc"]), dev(case["bt"])
+    tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor(case["tok_pos"], dtype=torch.int32, device=DEV)
+    partials = torch.full((n, H, splits, hd + 4), float("nan"), device=DEV)
+    untouched = torch.full((n, H * hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(untouched, q[:, :H * hd], kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
+                         n_splits=splits, partials=partials, waves=4, leave_splits=True)
+    assert (untouched == 7.0).all()
+    want = attention_reference(case, H, Hkv, hd, scale, window)
+    merged = torch.empty(n, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_merge(merged, partials)
+    close(merged, want, 8e-3, "merged splits")
+    N, K = 72, H * hd
+    w, bias = rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    for parts in (1, 2, 3):
+        if (parts - 1) * (((K + 63) // 64 + parts - 1) // parts) >= (K + 63) // 64:
+            continue
+        for n_base in (None, 0, 2):
+            base = None if n_base is None else (rnd(n, N, seed=8, scale=3.0) if n_base == 0 else rnd(n_base, n, N, seed=9, scale=3.0))
+            planes = torch.full((parts, n, N), float("nan"), device=DEV)
+            if n > 16:
+                with pytest.raises(Exception, match="outside"):
+                    ops.gemm_att_parts(partials, w, planes, bias=bias if base is not None else None, base=base)
+                continue
+            ops.gemm_att_parts(partials, w, planes, bias=bias if base is not None else None, base=base)
+            total = merged.double() @ w.double().t()
+            if base is not None:
+                total = total + bias.double() + (base.double() if n_base == 0 else base.double().sum(0))
+            close(planes.double().sum(0), total, 1e-5, f"projection over splits, {parts} parts, base {n_base}")
+            # the same bits as the plain cut product over the merged rows
+            two = torch.empty_like(planes)
+            ops.gemm_skinny_parts(merged, w, two, bias=bias if base is not None else None, base=base, ksplit=8)
+            assert torch.equal(planes, two)
 
 
 PREFILL_CASES = [
