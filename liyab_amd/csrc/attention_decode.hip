@@ -223,7 +223,7 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
     LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
     LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
-    LIYAB_REQUIRE(waves == 4 || waves == 16, "attention_decode: %d waves per workgroup is not 4 or 16", waves);
+    LIYAB_REQUIRE(waves == 4 || waves == 8 || waves == 16, "attention_decode: %d waves per workgroup is not 4, 8 or 16", waves);
     if (n == 0) return 0;
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
@@ -237,6 +237,10 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     do {                                                                                                             \
         if (waves == 4)                                                                                              \
             attention_decode_kernel<L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+                                                                    max_blocks, tok_list, tok_seq, tok_pos, scale,   \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
+        else if (waves == 8)                                                                                         \
+            attention_decode_kernel<L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
                                                                     window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
         else                                                                                                         \

@@ -650,15 +650,18 @@ def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
     return max(1, min(context_bucket // 2048, 32)), 16
 
 
-def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int) -> int:
-    """Into how many splits a (token, head) pair's keys are cut when whoever reads attention's
-    output merges the splits itself (1: not at all): until the workgroups cover the chip, a split
-    keeping 128 keys or more of the longest context."""
+def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int):
+    """(splits, waves per workgroup) for a step whose attention output is read by somebody who
+    merges a (token, head) pair's splits himself (1 split: not cut). Measured at 12 heads of 64
+    and contexts of 512 to 1,024 (us a decode step at batch 1 / 8 / 16, uncut: 376 / 430 / 499):
+    8 splits of 4 waves 347 / 418 / 505, 4 of 4 360 / 425 / 496, 4 of 8 353 / 426 / 503, 2 of
+    16 390 / 444 / 588. So: workgroups of 4 waves, 8 splits (4 from a hundred pairs on), a
+    split keeping 128 keys or more of the longest context."""
     pairs = max(1, n_tokens * n_head)
     splits = 1
-    while splits < 8 and pairs * splits < 256 and context_bucket // (2 * splits) >= 128:
+    while splits < (8 if pairs <= 96 else 4) and context_bucket // (2 * splits) >= 128:
         splits *= 2
-    return splits
+    return splits, 4
 
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -684,11 +687,11 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
 
     if fast and host.attention_mode == "decode" and block_tables.shape[1] <= 2048:
         n = out.shape[0]
-        splits = decode_split_plan(n, n_head, host.context_bucket) if splits_ok else 1
+        splits, waves = decode_split_plan(n, n_head, host.context_bucket) if splits_ok else (1, 4)
         if splits > 1 and att_parts_takes(n, splits, hd):
             partials = ctx.workspace.get("attn_partials", (n, n_head, splits, hd + 4), torch.float32)
             attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
-                             scale=scale, window=window, n_splits=splits, partials=partials, waves=4,
+                             scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
                              rows_are_requests=host.max_q_len == 1, leave_splits=True)
             return partials
         decode(None, n)

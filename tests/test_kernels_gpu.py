@@ -381,7 +381,7 @@ def test_attention_generic(ops, case_id, dtype, window):
 
 
 @pytest.mark.parametrize("window", [0, 37])
-@pytest.mark.parametrize("splits,waves", [(1, 4), (1, 16), (2, 4), (5, 16), (32, 4)])
+@pytest.mark.parametrize("splits,waves", [(1, 4), (1, 16), (2, 4), (5, 16), (32, 4), (1, 8), (3, 8)])
 @pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
 def test_attention_decode(ops, case_id, splits, waves, window):
     ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
