@@ -26,7 +26,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-namespace {
+namespace ln_fold {
 
 union Frag {
     u32x4 u;
@@ -44,20 +44,22 @@ struct NormParams {
     float eps;
 };
 
-template <typename OutT, int MAXV>
+template <typename OutT, int MAXV, int NT>
 __global__ void __launch_bounds__(64 * LN_WAVES)
 gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N, int K, EpiParams epi) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int ldx = K + 8;  // rows 16 bytes apart modulo the banks: a group of 16 lanes reads 16 rows without conflict
     bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // [min(M, 16)][K + 8]
-    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][256]
+    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][NT][256]
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int i = lane % 16, g = lane / 16;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * 16 * NT;  // NT tiles of 16 output features a workgroup
     const int units = (K + 63) / 64;
     const u32x4 zero = {0, 0, 0, 0};
-    const bf16_t* wrow = w + static_cast<int64_t>(min(n0 + i, N - 1)) * K;
+    const bf16_t* wrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) wrow[t] = w + static_cast<int64_t>(min(n0 + 16 * t + i, N - 1)) * K;
 
     // 8 consecutive k of a row; past the end it is the last piece, read and dropped
     auto piece = [&](const bf16_t* row, int k) {
@@ -66,17 +68,20 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
     };
     // a trip of a wave is two units of 64 k: unit u covers k in [64 u, 64 u + 64), two
     // instructions of 32 k, this lane's 8 start at 8 g
-    auto load_w = [&](int u0, Frag (&f)[2][2]) {
+    auto load_w = [&](int u0, Frag (&f)[2][NT][2]) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int k = (u0 + p) * 64 + g * 8;
-            f[p][0].u = piece(wrow, k);
-            f[p][1].u = piece(wrow, k + 32);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                f[p][t][0].u = piece(wrow[t], k);
+                f[p][t][1].u = piece(wrow[t], k + 32);
+            }
         }
     };
-    Frag wc[2][2];
-    const int e_m = tid / 16, e_n = n0 + tid % 16;
-    const bool e_mine = tid < 256 && e_m < M && e_n < N;
+    Frag wc[2][NT][2];
+    const int e_m = (tid % 256) / 16, e_n = n0 + 16 * (tid / 256) + tid % 16;
+    const bool e_mine = tid < NT * 256 && e_m < M && e_n < N;
     float e_bias = 0.0f;
 
     // -- the norm: a wave per row, the row in registers ---------------------------------
@@ -85,22 +90,16 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
     // `between` runs once the row's first loads are asked for and before anything waits for them
     auto norm_row = [&](int m, bool keep, auto&& between) {
         const float* row0 = ln.planes + static_cast<int64_t>(m) * K;
-        // the norm's weight and bias travel with the row where the registers hold them all; for
-        // the widest rows they are asked for once the planes are added up
-        constexpr bool AFFINE_EARLY = MAXV <= 4;
+        // the norm's weight and bias travel with the row: asked for after the weights of the
+        // product, a wait for them would be a wait for those
         floatx4 v[MAXV], gw[MAXV], gb[MAXV];
-        auto load_affine = [&]() {
 #pragma unroll
-            for (int j = 0; j < MAXV; ++j) {
-                const int at = min(lane + kWave * j, nv - 1);
-                gw[j] = ln.weight != nullptr ? reinterpret_cast<const floatx4*>(ln.weight)[at] : fone;
-                gb[j] = ln.bias != nullptr ? reinterpret_cast<const floatx4*>(ln.bias)[at] : fzero;
-            }
-        };
-#pragma unroll
-        for (int j = 0; j < MAXV; ++j)  // past the row: its last piece again, unused
-            v[j] = reinterpret_cast<const floatx4*>(row0)[min(lane + kWave * j, nv - 1)];
-        if constexpr (AFFINE_EARLY) load_affine();
+        for (int j = 0; j < MAXV; ++j) {
+            const int at = min(lane + kWave * j, nv - 1);  // past the row: its last piece again, unused
+            v[j] = reinterpret_cast<const floatx4*>(row0)[at];
+            gw[j] = ln.weight != nullptr ? reinterpret_cast<const floatx4*>(ln.weight)[at] : fone;
+            gb[j] = ln.bias != nullptr ? reinterpret_cast<const floatx4*>(ln.bias)[at] : fzero;
+        }
         // further planes, PB together (a plane past the last is the last one again, read and dropped)
         constexpr int PB = MAXV <= 4 ? 3 : 1;  // what the registers hold
         bool first = true;
@@ -123,7 +122,6 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
                 for (int j = 0; j < MAXV; ++j)
                     if (q0 + u < ln.n_planes) v[j] += plane[u][j];
         }
-        if constexpr (!AFFINE_EARLY) load_affine();
         float s = 0.0f;
 #pragma unroll
         for (int j = 0; j < MAXV; ++j)
@@ -160,7 +158,9 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
 
     // -- the product ------------------------------------------------------------------
     const bf16_t* arow = xs + min(i, M - 1) * ldx;
-    floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    floatx4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     auto multiply = [&](int u0) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -168,72 +168,80 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
             Frag x0, x1;
             x0.u = piece(arow, k);
             x1.u = piece(arow, k + 32);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][0].v, x0.v, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][1].v, x1.v, acc, 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, x0.v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, x1.v, acc[t], 0, 0, 0);
+            }
         }
     };
     // every trip but the last asks for the next trip's weights before it multiplies; the last
     // one is peeled off, so no trip asks for (and then waits for) weights nobody uses
     int u0 = wave * 2;
     for (; u0 + 2 * LN_WAVES < units; u0 += 2 * LN_WAVES) {
-        Frag wn[2][2];
+        Frag wn[2][NT][2];
         load_w(u0 + 2 * LN_WAVES, wn);
         multiply(u0);
 #pragma unroll
-        for (int p = 0; p < 2; ++p) {
-            wc[p][0] = wn[p][0];
-            wc[p][1] = wn[p][1];
-        }
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                wc[p][t][0] = wn[p][t][0];
+                wc[p][t][1] = wn[p][t][1];
+            }
     }
     multiply(u0);  // a wave past the end of K holds zeros
-    // acc[r] = partial C^T[n = 4 g + r][m = i]; kept [m][n] per wave, added up in wave order
+    // acc[t][r] = partial C^T[n = 16 t + 4 g + r][m = i]; kept [tile][m][n] per wave, added up in wave order
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave * 256 + i * 16 + 4 * g + r] = acc[r];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[(wave * NT + t) * 256 + i * 16 + 4 * g + r] = acc[t][r];
     __syncthreads();
-    if (tid < 256) {
+    if (tid < NT * 256) {
         float v = 0.0f;
 #pragma unroll
-        for (int q = 0; q < LN_WAVES; ++q) v += red[q * 256 + tid];
+        for (int q = 0; q < LN_WAVES; ++q) v += red[q * NT * 256 + tid];
         if (e_mine) epilogue_store_biased<OutT>(epi, e_m, e_n, v + e_bias);
     }
 }
 
-template <int MAXV>
-int launch_ln(const NormParams& ln, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
-    const dim3 grid((N + 15) / 16);
-    const size_t smem = ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16 + LN_WAVES * 256 * sizeof(float);
-    auto* pw = static_cast<const bf16_t*>(w);
-    if (epi.out_dtype == kF32) {
-        auto kern = gemm_skinny_ln_kernel<float, MAXV>;
-        static bool ready = false;
-        if (!ready) {
-            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            ready = true;
-        }
-        kern<<<grid, 64 * LN_WAVES, smem, stream>>>(ln, pw, M, N, K, epi);
-    } else {
-        auto kern = gemm_skinny_ln_kernel<bf16_t, MAXV>;
-        static bool ready = false;
-        if (!ready) {
-            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            ready = true;
-        }
-        kern<<<grid, 64 * LN_WAVES, smem, stream>>>(ln, pw, M, N, K, epi);
+template <typename OutT, int MAXV, int NT>
+int launch_kernel(const NormParams& ln, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
+    const dim3 grid((N + 16 * NT - 1) / (16 * NT));
+    const size_t smem = ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16 + LN_WAVES * NT * 256 * sizeof(float);
+    auto kern = gemm_skinny_ln_kernel<OutT, MAXV, NT>;
+    static bool ready = false;
+    if (!ready) {
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        ready = true;
     }
+    kern<<<grid, 64 * LN_WAVES, smem, stream>>>(ln, static_cast<const bf16_t*>(w), M, N, K, epi);
     return check_launch("gemm_skinny_ln");
 }
 
-}  // namespace
+// A workgroup keeps a row in registers and so fills a compute unit: with more strips of 16
+// output features than compute units a workgroup takes two strips, or the workgroups would run
+// in two rounds.
+template <int MAXV>
+int launch_ln(const NormParams& ln, const void* w, int M, int N, int K, int wide, const EpiParams& epi, hipStream_t stream) {
+    if (epi.out_dtype == kF32)
+        return wide ? launch_kernel<float, MAXV, 2>(ln, w, M, N, K, epi, stream) : launch_kernel<float, MAXV, 1>(ln, w, M, N, K, epi, stream);
+    return wide ? launch_kernel<bf16_t, MAXV, 2>(ln, w, M, N, K, epi, stream) : launch_kernel<bf16_t, MAXV, 1>(ln, w, M, N, K, epi, stream);
+}
+
+}  // namespace ln_fold
 }  // namespace liyab
 
 using namespace liyab;
+using namespace liyab::ln_fold;
 
 // out = epilogue(LayerNorm(planes[0] + planes[1] + ...) . w^T + bias). planes: float32
 // [n_planes][M][K], plane_stride floats apart (n_planes = 1: the rows themselves); w [N, K]
-// bfloat16. M <= 16; K a multiple of 8, at most 2048. The residual epilogue is not taken
-// (the product of a norm is never added to the stream as it is).
+// bfloat16. M <= 16; K a multiple of 8, at most 2048. wide: 32 instead of 16 output features a
+// workgroup (-1: when there are more strips of 16 than compute units). The residual epilogue
+// is not taken (the product of a norm is never added to the stream as it is).
 extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight,
-                                    const float* ln_bias, float eps, const void* w, int M, int N, int K,
+                                    const float* ln_bias, float eps, const void* w, int M, int N, int K, int wide,
                                     const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(planes && w && epi_in, "gemm_skinny_ln: null operand");
     LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 16) N=%d K=%d", M, N, K);
@@ -249,10 +257,19 @@ extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t p
     LIYAB_REQUIRE(epi.mode != kEpiResidual, "gemm_skinny_ln: the residual epilogue is not taken");
     if (int rc = check_epilogue(epi, M, N)) return rc;
     if (M == 0) return 0;
+    if (wide < 0) {
+        static int units = 0;  // compute units of the device (one device a process)
+        if (units == 0) {
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
+                units = 256;
+        }
+        wide = (N + 15) / 16 > units ? 1 : 0;
+    }
     const NormParams ln{planes, n_planes, plane_stride, ln_weight, ln_bias, eps};
-    if (K <= 256) return launch_ln<1>(ln, w, M, N, K, epi, stream);
-    if (K <= 512) return launch_ln<2>(ln, w, M, N, K, epi, stream);
-    if (K <= 768) return launch_ln<3>(ln, w, M, N, K, epi, stream);
-    if (K <= 1024) return launch_ln<4>(ln, w, M, N, K, epi, stream);
-    return launch_ln<8>(ln, w, M, N, K, epi, stream);
+    if (K <= 256) return launch_ln<1>(ln, w, M, N, K, wide, epi, stream);
+    if (K <= 512) return launch_ln<2>(ln, w, M, N, K, wide, epi, stream);
+    if (K <= 768) return launch_ln<3>(ln, w, M, N, K, wide, epi, stream);
+    if (K <= 1024) return launch_ln<4>(ln, w, M, N, K, wide, epi, stream);
+    return launch_ln<8>(ln, w, M, N, K, wide, epi, stream);
 }

@@ -477,9 +477,11 @@ def k_parts(M: int, N: int, K: int) -> int:
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,
-                   w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, epilogue: int = EPI_NONE, kv=None) -> None:
+                   w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, epilogue: int = EPI_NONE, kv=None,
+                   wide: int = -1) -> None:
     """The weight-streaming product over LayerNorm(x) of the float32 rows x [M, K], or of a sum
-    of planes [parts, M, K], the norm computed inside the product kernel (`skinny_ln_takes`)."""
+    of planes [parts, M, K], the norm computed inside the product kernel (`skinny_ln_takes`).
+    wide: 32 instead of 16 output features a workgroup (-1: chosen from the shape)."""
     ptr, n_parts, stride, M, K = _planes(x, "gemm_skinny_ln")
     _dev(w, "w")
     if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
@@ -494,12 +496,31 @@ def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: 
     e = _epilogue(fake_a, w, bias, out, None, epilogue, kv)
     e.exact = 0
     _lib.call("liyab_gemm_skinny_ln", ptr, n_parts, stride, _ptr(ln_weight), _ptr(ln_bias), float(eps),
-              w.data_ptr(), M, w.shape[0], K, ctypes.byref(e), _stream())
+              w.data_ptr(), M, w.shape[0], K, wide, ctypes.byref(e), _stream())
 
 
 def skinny_ln_takes(M: int, K: int) -> bool:
     """What the product kernel with the norm inside takes: one tile of rows, a row in a wave's registers."""
     return 0 < M <= 16 and K % 8 == 0 and K <= 2048
+
+
+_compute_units = 0
+
+
+def compute_units() -> int:
+    global _compute_units
+    if not _compute_units:
+        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    return _compute_units
+
+
+def skinny_ln_pays(M: int, N: int, K: int) -> bool:
+    """Whether folding the norm into the product beats the norm kernel followed by the plain
+    product. The folded kernel keeps a row in registers, so one workgroup fills a compute unit:
+    with more workgroups (16 or 32 output features each) than compute units they run in two
+    rounds, which costs more than the norm's kernel (GPT-2 XL's 1,600 -> 4,800 at 8 rows in
+    strips of 16: 15.2 us folded against 9 + 4.5)."""
+    return skinny_ln_takes(M, K) and (N + 31) // 32 <= compute_units()
 
 
 def gemm_mfma_dl(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,

@@ -28,8 +28,8 @@ FOLD_NORM_ROWS = 16  # at most (the kernel's own limit is one tile of 16 rows)
 def _fuses(a, w: torch.Tensor, residual) -> bool:
     return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and residual is None
             and a.rows is None and a._tensor is None and w.dtype == torch.bfloat16 and a.x.dtype == torch.float32
-            and a.x.is_contiguous() and a.n_rows <= FOLD_NORM_ROWS and w.shape[0] <= 8192
-            and ops.skinny_ln_takes(a.n_rows, a.norm.width))
+            and a.x.is_contiguous() and a.n_rows <= FOLD_NORM_ROWS
+            and ops.skinny_ln_pays(a.n_rows, w.shape[0], a.norm.width))
 
 
 def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[torch.Tensor] = None,

@@ -238,7 +238,10 @@ def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, parts, epilogue):
     epi = ops.ACTIVATION_EPILOGUE[epilogue]
     for out_dtype in (torch.float32, torch.bfloat16):
         out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=epi)
+        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=epi, wide=0)
+        strips_of_32 = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=strips_of_32, epilogue=epi, wide=1)
+        assert torch.equal(out, strips_of_32)
         # the folded norm rounds to bfloat16 where the standalone kernel does: allow one ulp of the operand
         close(out, gemm_reference(h, w, bias, epilogue), 4e-3 if out_dtype == torch.float32 else 8e-3, f"gemm+ln {epilogue}")
         normed = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
