@@ -1,4 +1,4 @@
-// out[M,N] = LayerNorm(x)[M,K] . w[N,K]^T in bfloat16 for steps of at most 16 tokens,
+// out[M,N] = LayerNorm(x)[M,K] . w[N,K]^T in bfloat16 for steps of at most 32 tokens,
 // the norm computed by the product kernel itself: a decode step is a chain of
 // small kernels, each of which costs its launch and a first trip to memory
 // whatever its work, and the norm is two of the seven kernels of a layer.
@@ -9,7 +9,7 @@
 // added in that order. A workgroup owns 16 output features and all M rows.
 // Its eight waves first ask for their share of the weights (K is split over
 // the waves, as in the plain streaming kernel), then each wave normalises
-// rows m = wave, wave + 8: the row's pieces of every plane are asked for
+// rows m = wave, wave + 8, ...: the row's pieces of every plane are asked for
 // together, 16 bytes a lane, no load under a branch; statistics are two
 // passes over registers with the standalone kernel's reduction tree (the
 // reference's layernorm, src/core/transformer.cpp:77-106), so both kernels
@@ -44,13 +44,14 @@ struct NormParams {
     float eps;
 };
 
-template <typename OutT, int MAXV, int NT>
+template <typename OutT, int MAXV, int MT, int NT>
 __global__ void __launch_bounds__(64 * LN_WAVES)
 gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N, int K, EpiParams epi) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int ldx = K + 8;  // rows 16 bytes apart modulo the banks: a group of 16 lanes reads 16 rows without conflict
-    bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // [min(M, 16)][K + 8]
-    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][NT][256]
+    constexpr int TILES = MT * NT;  // MT tiles of 16 rows (all M rows), NT tiles of 16 output features
+    bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // [M][K + 8]
+    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][TILES][256]
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int i = lane % 16, g = lane / 16;
@@ -80,8 +81,9 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
         }
     };
     Frag wc[2][NT][2];
-    const int e_m = (tid % 256) / 16, e_n = n0 + 16 * (tid / 256) + tid % 16;
-    const bool e_mine = tid < NT * 256 && e_m < M && e_n < N;
+    // this thread's first output: tile tid / 256 = (row tile, feature tile)
+    const int e_m = 16 * ((tid / 256) / NT) + (tid % 256) / 16, e_n = n0 + 16 * ((tid / 256) % NT) + tid % 16;
+    const bool e_mine = tid < TILES * 256 && e_m < M && e_n < N;
     float e_bias = 0.0f;
 
     // -- the norm: a wave per row, the row in registers ---------------------------------
@@ -157,21 +159,28 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
     lds_barrier();  // the weights may still be on their way
 
     // -- the product ------------------------------------------------------------------
-    const bf16_t* arow = xs + min(i, M - 1) * ldx;
-    floatx4 acc[NT];
+    const bf16_t* arow[MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int r = 0; r < MT; ++r) arow[r] = xs + min(16 * r + i, M - 1) * ldx;
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int r = 0; r < MT; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     auto multiply = [&](int u0) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int k = (u0 + p) * 64 + g * 8;
-            Frag x0, x1;
-            x0.u = piece(arow, k);
-            x1.u = piece(arow, k + 32);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, x0.v, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, x1.v, acc[t], 0, 0, 0);
+            for (int r = 0; r < MT; ++r) {
+                Frag x0, x1;
+                x0.u = piece(arow[r], k);
+                x1.u = piece(arow[r], k + 32);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][0].v, x0.v, acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][t][1].v, x1.v, acc[r][t], 0, 0, 0);
+                }
             }
         }
     };
@@ -191,25 +200,31 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
             }
     }
     multiply(u0);  // a wave past the end of K holds zeros
-    // acc[t][r] = partial C^T[n = 16 t + 4 g + r][m = i]; kept [tile][m][n] per wave, added up in wave order
+    // acc[r][t][c] = partial C^T[n = 16 t + 4 g + c][m = 16 r + i]; kept [tile][m][n] per wave, added up in wave order
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int r = 0; r < MT; ++r)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[(wave * NT + t) * 256 + i * 16 + 4 * g + r] = acc[t][r];
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) red[(wave * TILES + r * NT + t) * 256 + i * 16 + 4 * g + c] = acc[r][t][c];
     __syncthreads();
-    if (tid < NT * 256) {
+    for (int e = tid; e < TILES * 256; e += 64 * LN_WAVES) {
+        const int tile = e / 256, m = 16 * (tile / NT) + (e % 256) / 16, n = n0 + 16 * (tile % NT) + e % 16;
         float v = 0.0f;
 #pragma unroll
-        for (int q = 0; q < LN_WAVES; ++q) v += red[q * NT * 256 + tid];
-        if (e_mine) epilogue_store_biased<OutT>(epi, e_m, e_n, v + e_bias);
+        for (int q = 0; q < LN_WAVES; ++q) v += red[q * TILES * 256 + e];
+        if (m >= M || n >= N) continue;
+        if (e == tid) epilogue_store_biased<OutT>(epi, m, n, v + e_bias);
+        else epilogue_store<OutT>(epi, m, n, v);
     }
 }
 
-template <typename OutT, int MAXV, int NT>
+template <typename OutT, int MAXV, int MT, int NT>
 int launch_kernel(const NormParams& ln, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
-    const size_t smem = ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16 + LN_WAVES * NT * 256 * sizeof(float);
-    auto kern = gemm_skinny_ln_kernel<OutT, MAXV, NT>;
+    const size_t smem = ((static_cast<size_t>(M) * (K + 8) * 2 + 15) / 16) * 16 + LN_WAVES * MT * NT * 256 * sizeof(float);
+    LIYAB_REQUIRE(smem <= 160 * 1024, "gemm_skinny_ln: %d rows of %d need %zu bytes of LDS", M, K, smem);
+    auto kern = gemm_skinny_ln_kernel<OutT, MAXV, MT, NT>;
     static bool ready = false;
     if (!ready) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -221,12 +236,16 @@ int launch_kernel(const NormParams& ln, const void* w, int M, int N, int K, cons
 
 // A workgroup keeps a row in registers and so fills a compute unit: with more strips of 16
 // output features than compute units a workgroup takes two strips, or the workgroups would run
-// in two rounds.
+// in two rounds (one tile of rows only: with more rows the sums across waves fill the LDS).
+template <typename OutT, int MAXV>
+int launch_rows(const NormParams& ln, const void* w, int M, int N, int K, int wide, const EpiParams& epi, hipStream_t stream) {
+    if (M <= 16) return wide ? launch_kernel<OutT, MAXV, 1, 2>(ln, w, M, N, K, epi, stream) : launch_kernel<OutT, MAXV, 1, 1>(ln, w, M, N, K, epi, stream);
+    return launch_kernel<OutT, MAXV, 2, 1>(ln, w, M, N, K, epi, stream);
+}
 template <int MAXV>
 int launch_ln(const NormParams& ln, const void* w, int M, int N, int K, int wide, const EpiParams& epi, hipStream_t stream) {
-    if (epi.out_dtype == kF32)
-        return wide ? launch_kernel<float, MAXV, 2>(ln, w, M, N, K, epi, stream) : launch_kernel<float, MAXV, 1>(ln, w, M, N, K, epi, stream);
-    return wide ? launch_kernel<bf16_t, MAXV, 2>(ln, w, M, N, K, epi, stream) : launch_kernel<bf16_t, MAXV, 1>(ln, w, M, N, K, epi, stream);
+    if (epi.out_dtype == kF32) return launch_rows<float, MAXV>(ln, w, M, N, K, wide, epi, stream);
+    return launch_rows<bf16_t, MAXV>(ln, w, M, N, K, wide, epi, stream);
 }
 
 }  // namespace ln_fold
@@ -237,14 +256,16 @@ using namespace liyab::ln_fold;
 
 // out = epilogue(LayerNorm(planes[0] + planes[1] + ...) . w^T + bias). planes: float32
 // [n_planes][M][K], plane_stride floats apart (n_planes = 1: the rows themselves); w [N, K]
-// bfloat16. M <= 16; K a multiple of 8, at most 2048. wide: 32 instead of 16 output features a
-// workgroup (-1: when there are more strips of 16 than compute units). The residual epilogue
+// bfloat16. M <= 32 (measured: from 32 rows on the norm's own kernel is faster; with 64 rows
+// every workgroup normalising them all cost 950 against 810 us a step); K a multiple of 8, at
+// most 2048. wide: 32 instead of 16 output features a workgroup, for M <= 16 (-1: when
+// there are more strips of 16 than compute units). The residual epilogue
 // is not taken (the product of a norm is never added to the stream as it is).
 extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight,
                                     const float* ln_bias, float eps, const void* w, int M, int N, int K, int wide,
                                     const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(planes && w && epi_in, "gemm_skinny_ln: null operand");
-    LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 16) N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(M >= 0 && M <= 32 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 32) N=%d K=%d", M, N, K);
     LIYAB_REQUIRE(K % 8 == 0 && K <= 2048, "gemm_skinny_ln: K %d must be a multiple of 8, at most 2048", K);
     LIYAB_REQUIRE(n_planes >= 1 && n_planes <= 16, "gemm_skinny_ln: %d planes (1 to 16)", n_planes);
     LIYAB_REQUIRE(n_planes == 1 || plane_stride >= static_cast<int64_t>(M) * K, "gemm_skinny_ln: planes of %lld floats overlap",
@@ -266,6 +287,7 @@ extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t p
         }
         wide = (N + 15) / 16 > units ? 1 : 0;
     }
+    LIYAB_REQUIRE(!wide || M <= 16, "gemm_skinny_ln: strips of 32 output features go with at most 16 rows (%d)", M);
     const NormParams ln{planes, n_planes, plane_stride, ln_weight, ln_bias, eps};
     if (K <= 256) return launch_ln<1>(ln, w, M, N, K, wide, epi, stream);
     if (K <= 512) return launch_ln<2>(ln, w, M, N, K, wide, epi, stream);

@@ -500,8 +500,9 @@ def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: 
 
 
 def skinny_ln_takes(M: int, K: int) -> bool:
-    """What the product kernel with the norm inside takes: one tile of rows, a row in a wave's registers."""
-    return 0 < M <= 16 and K % 8 == 0 and K <= 2048
+    """What the product kernel with the norm inside takes: one or two tiles of 16 rows, a row in
+    a wave's registers."""
+    return 0 < M <= 32 and K % 8 == 0 and K <= 2048
 
 
 _compute_units = 0
@@ -520,7 +521,7 @@ def skinny_ln_pays(M: int, N: int, K: int) -> bool:
     with more workgroups (16 or 32 output features each) than compute units they run in two
     rounds, which costs more than the norm's kernel (GPT-2 XL's 1,600 -> 4,800 at 8 rows in
     strips of 16: 15.2 us folded against 9 + 4.5)."""
-    return skinny_ln_takes(M, K) and (N + 31) // 32 <= compute_units()
+    return skinny_ln_takes(M, K) and (N + (31 if M <= 16 else 15)) // (32 if M <= 16 else 16) <= compute_units()
 
 
 def gemm_mfma_dl(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,

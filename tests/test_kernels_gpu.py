@@ -225,7 +225,9 @@ def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
 
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf"])
 @pytest.mark.parametrize("M,N,K,eps,parts", [(1, 64, 64, 1e-5, 1), (8, 2304, 768, 1e-5, 4), (16, 100, 1600, 1e-6, 2), (5, 777, 144, 1e-5, 3),
-                                             (3, 50, 2048, 1e-3, 5), (13, 520, 1024, 1e-5, 1), (9, 3072, 768, 1e-5, 2), (16, 48, 96, 1e-6, 16)])
+                                             (3, 50, 2048, 1e-3, 5), (13, 520, 1024, 1e-5, 1), (9, 3072, 768, 1e-5, 2), (16, 48, 96, 1e-6, 16),
+                                             (17, 200, 768, 1e-5, 2), (32, 2304, 768, 1e-5, 1), (24, 130, 1600, 1e-6, 3), (29, 3072, 768, 1e-5, 1),
+                                             (32, 90, 1024, 1e-5, 4)])
 def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, parts, epilogue):
     """The product kernel that normalises its own rows, given whole or as a sum of planes: the
     same bits as the standalone norm followed by the streaming product."""
@@ -239,20 +241,24 @@ def test_gemm_with_layernorm_folded_in(ops, M, N, K, eps, parts, epilogue):
     for out_dtype in (torch.float32, torch.bfloat16):
         out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
         ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=epi, wide=0)
-        strips_of_32 = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-        ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=strips_of_32, epilogue=epi, wide=1)
-        assert torch.equal(out, strips_of_32)
+        if M <= 16:
+            strips_of_32 = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+            ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=strips_of_32, epilogue=epi, wide=1)
+            assert torch.equal(out, strips_of_32)
         # the folded norm rounds to bfloat16 where the standalone kernel does: allow one ulp of the operand
         close(out, gemm_reference(h, w, bias, epilogue), 4e-3 if out_dtype == torch.float32 else 8e-3, f"gemm+ln {epilogue}")
         normed = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
         ops.layernorm(normed, x, lw, lb, eps)
         two = torch.empty(M, N, dtype=out_dtype, device=DEV)
-        ops.gemm_skinny(normed, w, bias, out=two, epilogue=epi, ksplit=8, wide=0, mtile=1)
-        assert torch.equal(out, two)
+        ops.gemm_skinny(normed, w, bias, out=two, epilogue=epi, ksplit=8, wide=0, mtile=1 if M <= 16 else 0)
+        if M <= 16:
+            assert torch.equal(out, two)
+        else:  # more tiles of rows: the plain kernel deals K out to its waves in another order
+            close(out, two, 1e-5 if out_dtype == torch.float32 else 8e-3, "folded against norm + product")
     with pytest.raises(Exception, match="residual"):
         ops.gemm_skinny_ln(x, lw, lb, eps, w, bias, out=out, epilogue=ops.EPI_RESIDUAL)
     with pytest.raises(Exception, match="outside"):
-        ops.gemm_skinny_ln(rnd(17, K), lw, lb, eps, w, bias, out=torch.empty(17, N, device=DEV))
+        ops.gemm_skinny_ln(rnd(33, K), lw, lb, eps, w, bias, out=torch.empty(33, N, device=DEV))
 
 
 def test_gemm_strided_rows_and_refusals(ops):
@@ -596,3 +602,31 @@ def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
     close(kc, kc2, 1e-2, "keys")
     close(vc, vc2, 1e-2, "values")
     assert (kc == 0).sum() == (kc2 == 0).sum()  # nothing written outside the tokens' slots
+
+
+@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(1, 4, 4, 16, 64, 16), (9, 6, 2, 32, 192, 8), (16, 12, 12, 64, 768, 64), (27, 5, 5, 48, 240, 16),
+                                               (32, 12, 12, 64, 768, 64)])
+def test_folded_norm_with_the_paged_qkv_epilogue(ops, M, H, Hkv, hd, K, page):
+    """The product that normalises its own rows, writing queries to a dense buffer and keys and
+    values into shuffled cache slots: what the standalone norm followed by the streaming
+    product writes."""
+    q_dim, kv_dim = H * hd, Hkv * hd
+    N = q_dim + 2 * kv_dim
+    x = rnd(2, M, K, scale=2.0)
+    lw, lb = rnd(K, seed=5) + 1.0, rnd(K, seed=6)
+    w, bias = rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    pages = -(-M // page) + 3
+    slots = torch.randperm(pages * page)[:M].to(torch.int32).to(DEV)
+    got = [torch.zeros(pages, Hkv, page, hd, dtype=torch.bfloat16, device=DEV) for _ in range(2)] + [torch.zeros(M, q_dim, dtype=torch.bfloat16, device=DEV)]
+    ops.gemm_skinny_ln(x, lw, lb, 1e-5, w, bias, out=got[2], epilogue=ops.EPI_QKV_PAGED, kv=(got[0], got[1], slots, q_dim))
+    normed = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    ops.layernorm(normed, x, lw, lb, 1e-5)
+    want = [torch.zeros_like(got[0]), torch.zeros_like(got[1]), torch.zeros_like(got[2])]
+    ops.gemm_skinny(normed, w, bias, out=want[2], epilogue=ops.EPI_QKV_PAGED, kv=(want[0], want[1], slots, q_dim), ksplit=8, wide=0,
+                    mtile=1 if M <= 16 else 0)
+    for g, t, what in zip(got, want, ("keys", "values", "queries")):
+        if M <= 16:
+            assert torch.equal(g, t), what
+        else:
+            close(g, t, 8e-3, what)
+    assert (got[0] == 0).sum() == (want[0] == 0).sum()  # nothing written outside the tokens' slots
