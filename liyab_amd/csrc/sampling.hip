@@ -253,6 +253,7 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
 // 2^-44 of the largest counts as none.
 constexpr int kMassBits = 44;
 constexpr int kWaveCandidates = 64;
+constexpr int kPool = 1024;  // keys that may be among the k largest, for one wave to choose from
 
 __device__ __forceinline__ unsigned long long fixed_mass(uint32_t key, float lmax, float scale2) {
     // exp((l - l_max) / T) through the hardware's 2^x (scale2 = log2(e) / T), in [0, 1]; times
@@ -279,6 +280,15 @@ __device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, 
 __device__ __forceinline__ unsigned long long shfl_u64(unsigned long long v, int src) {
     const uint32_t lo = __shfl(static_cast<uint32_t>(v), src, kWave);
     const uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), src, kWave);
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+// Lane `src`'s value for every lane, `src` being the same for the whole wave: a register read,
+// where an exchange through the lanes' crossbar would take a hundred cycles to come back.
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int src) { return __builtin_amdgcn_readlane(v, src); }
+__device__ __forceinline__ int lane_value(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
+__device__ __forceinline__ unsigned long long lane_value64(unsigned long long v, int src) {
+    const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(v), src);
+    const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(v >> 32), src);
     return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
@@ -328,22 +338,41 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     __shared__ int result, n_cand;
     __shared__ uint32_t cand_key[kWaveCandidates];
     __shared__ int cand_id[kWaveCandidates];
+    // top-k of at most 64: the threads' largest keys, and the pool of keys that may be among the k largest
+    __shared__ uint32_t thread_max[THREADS];
+    __shared__ uint32_t pool_key[kPool];
+    __shared__ int pool_id[kPool];
+    __shared__ int n_pool;
+    __shared__ uint32_t pool_floor;
 
     const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const float* row = logits + static_cast<int64_t>(r) * ld;
-    const int chunk = (((V + THREADS - 1) / THREADS + 3) / 4) * 4;  // ids a thread, <= EPT (checked by the launcher)
-    const int span0 = wave * kWave * chunk;
+    // A thread's groups of 4 ids are read as 16 bytes each, so the groups start at addresses that
+    // are multiples of 16: the ids are counted from `shift` entries before the row (a row of an odd
+    // width starts anywhere), and an id before the row is no element.
+    const int shift = static_cast<int>((reinterpret_cast<uintptr_t>(row) >> 2) & 3u);
+    const int chunk = (((V + shift + THREADS - 1) / THREADS + 3) / 4) * 4;  // ids a thread, <= EPT (the launcher's check)
+    const int span0 = wave * kWave * chunk - shift;
     auto id_of = [&](int j) { return span0 + ((j / 4) * kWave + lane) * 4 + j % 4; };
     // keys of this thread's ids; 0 stands for "no element" (no real logit has that key)
     uint32_t keys[EPT];
-    // every load from a valid address (an id past the row reads the row's last entry), so that no
-    // condition has to live while the loads are in flight; what is past the row is dropped after
+    // every load from a valid address (a group past the row reads the row's last group), so that no
+    // condition has to live while the loads are in flight; what is outside the row is dropped after.
+    // The first and the last group may reach up to 12 bytes outside the row, within its aligned 16.
+    {
+        typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+        const int last_group = ((V - 1 + shift) / 4) * 4 - shift;  // first id of the group that holds the row's last entry
 #pragma unroll
-    for (int j = 0; j < EPT; ++j) keys[j] = __float_as_uint(row[min(id_of(j), V - 1)]);
+        for (int g = 0; g < GROUPS; ++g) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(row + min(id_of(4 * g), last_group));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) keys[4 * g + e] = v[e];
+        }
+    }
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
         const uint32_t raw = again(keys[j]);
-        keys[j] = (j < chunk && id_of(j) < V) ? ordered_key(__uint_as_float(raw)) : 0u;
+        keys[j] = (j < chunk && id_of(j) >= 0 && id_of(j) < V) ? ordered_key(__uint_as_float(raw)) : 0u;
     }
     // the largest key and its lowest id
     uint32_t kmax = 0;
@@ -351,6 +380,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
 #pragma unroll
     for (int j = 0; j < EPT; ++j)
         if (keys[j] > kmax) { kmax = keys[j]; imax = id_of(j); }
+    thread_max[tid] = kmax;
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
         const uint32_t ok = __shfl_xor(kmax, off, kWave);
@@ -358,7 +388,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         if (ok > kmax || (ok == kmax && oi < imax)) { kmax = ok; imax = oi; }
     }
     if (lane == 0) { redk[wave] = kmax; redi[wave] = imax; }
-    if (tid == 0) { result = -1; n_cand = 0; }
+    if (tid == 0) { result = -1; n_cand = 0; n_pool = 0; }
     __syncthreads();
     kmax = redk[0]; imax = redi[0];
 #pragma unroll
@@ -423,6 +453,145 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         }
     };
 
+    // ---- one wave among at most 64 candidates in cand_key / cand_id: nucleus cut and draw ----
+    auto wave_finish = [&]() {
+        const int n = n_cand;  // = k
+        const bool has = lane < n;
+        const uint32_t key = has ? cand_key[lane] : 0u;
+        const int id = has ? cand_id[lane] : 0x7fffffff;
+        const unsigned long long q = has ? fixed_mass(key, lmax, inv_t) : 0ull;
+        // place in the descending order of keys (ties by ascending id) and in the ascending order of ids
+        int desc = 0, asc = 0;
+        for (int o = 0; o < n; ++o) {
+            const uint32_t ok = lane_value(key, o);
+            const int oi = lane_value(id, o);
+            desc += ok > key || (ok == key && oi < id);
+            asc += oi < id;
+        }
+        bool kept = has;
+        if (use_p) {
+            // cum = mass of the candidates before this one in descending order, itself included
+            unsigned long long cum = 0, total = 0;
+            for (int o = 0; o < n; ++o) {
+                const unsigned long long oq = lane_value64(q, o);
+                const int od = lane_value(desc, o);
+                total += oq;
+                if (od <= desc) cum += oq;
+            }
+            const double target = static_cast<double>(tp) * static_cast<double>(total);
+            // the shortest prefix whose mass reaches the target: an element is kept when the prefix
+            // before it has not reached it yet; the first is always kept
+            kept = has && (desc == 0 || static_cast<double>(cum - q) < target);
+        }
+        const unsigned long long mass = kept ? q : 0ull;
+        unsigned long long before = 0, total = 0;
+        for (int o = 0; o < n; ++o) {
+            const unsigned long long om = lane_value64(mass, o);
+            const int oa = lane_value(asc, o);
+            total += om;
+            if (oa < asc) before += om;
+        }
+        int token = imax;
+        if (total > 0ull) {
+            unsigned long long rr = static_cast<unsigned long long>(uniform[r] * static_cast<double>(total));
+            if (rr >= total) rr = total - 1;
+            const bool mine = kept && rr >= before && rr - before < mass;
+            const unsigned long long pick = __ballot(mine);
+            if (pick != 0ull) token = __shfl(id, __ffsll(static_cast<long long>(pick)) - 1, kWave);
+        }
+        if (lane == 0) {
+            out[r] = token;
+            if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
+        }
+    };
+
+    // ---- top-k of at most 64 (the usual case) without passes of the whole workgroup over the row ----
+    // The k-th largest of the threads' largest keys is a floor for the k-th largest key of the
+    // row (k keys reach it): one wave finds it among THREADS values; every thread then puts its
+    // keys from that floor up into a pool (about k of them, unless many keys are equal); one wave
+    // finds the k-th largest of the pool exactly, keeps ties by ascending id, and finishes. A pool
+    // that overflows falls through to the bisection over the whole row below.
+    if (use_k && k <= kWaveCandidates) {
+        if (wave == 0) {
+            constexpr int PER = THREADS / kWave;
+            uint32_t mine[PER];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) mine[i] = thread_max[lane + kWave * i];
+            uint32_t floor_key = 0;
+            for (int bit = 31; bit >= 0; --bit) {
+                const uint32_t cand = floor_key | (1u << bit);
+                int c = 0;  // counted through the lanes' votes: sums across lanes would cost six dependent exchanges a bit
+#pragma unroll
+                for (int i = 0; i < PER; ++i) c += __popcll(__ballot(mine[i] >= cand));
+                if (c >= k) floor_key = cand;
+            }
+            if (lane == 0) pool_floor = floor_key;
+        }
+        __syncthreads();
+        const uint32_t floor_key = pool_floor;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            if (keys[j] != 0u && keys[j] >= floor_key) {
+                const int at = atomicAdd(&n_pool, 1);  // the order of arrival does not matter: ranks below are by key and id
+                if (at < kPool) {
+                    pool_key[at] = keys[j];
+                    pool_id[at] = id_of(j);
+                }
+            }
+        }
+        __syncthreads();
+        const int n = n_pool;
+        if (n <= kPool) {
+            if (wave == 0) {
+                constexpr int PER = kPool / kWave;
+                uint32_t pk[PER];
+                int pid[PER];
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    const int e = lane + kWave * i;
+                    pk[i] = e < n ? pool_key[e] : 0u;
+                    pid[i] = e < n ? pool_id[e] : 0x7fffffff;
+                }
+                uint32_t tau = 0;
+                for (int bit = 31; bit >= 0; --bit) {
+                    const uint32_t cand = tau | (1u << bit);
+                    int c = 0;
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) c += __popcll(__ballot(pk[i] >= cand));
+                    if (c >= k) tau = cand;
+                }
+                int above = 0, tied = 0;
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    above += __popcll(__ballot(pk[i] > tau));
+                    tied += __popcll(__ballot(pk[i] == tau && pk[i] != 0u));
+                }
+                const int ties = k - above;  // ties at tau that are kept: those of the lowest ids
+                int base = 0;
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    bool keep = pk[i] != 0u && pk[i] >= tau;
+                    if (ties < tied && pk[i] == tau && pk[i] != 0u) {
+                        int rank = 0;  // ties of a lower id
+                        for (int o = 0; o < n; ++o) rank += pool_key[o] == tau && pool_id[o] < pid[i];
+                        keep = rank < ties;
+                    }
+                    const unsigned long long kept_lanes = __ballot(keep);
+                    if (keep) {
+                        const int at = base + __popcll(kept_lanes & lanes_below);
+                        cand_key[at] = pk[i];
+                        cand_id[at] = pid[i];
+                    }
+                    base += __popcll(kept_lanes);
+                }
+                if (lane == 0) n_cand = base;
+            }
+            __syncthreads();
+            if (wave == 0) wave_finish();
+            return;
+        }
+    }
+
     // ---- top-k: the k-th largest key, and how many of its ties are kept ----
     uint32_t tau_k = 0;
     int ties_k = 0x7fffffff;
@@ -442,7 +611,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
 
     uint32_t bits[(EPT + 31) / 32];
     if (use_k && k <= kWaveCandidates) {
-        // ---- few candidates: gathered, then one wave does the rest ----
+        // ---- few candidates (the pool overflowed): gathered, then one wave does the rest ----
         kept_bits(tau_k, ties_k, bits);
 #pragma unroll
         for (int j = 0; j < EPT; ++j) {
@@ -453,55 +622,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
             }
         }
         __syncthreads();
-        if (wave != 0) return;
-        const int n = n_cand;  // = k
-        const bool has = lane < n;
-        const uint32_t key = has ? cand_key[lane] : 0u;
-        const int id = has ? cand_id[lane] : 0x7fffffff;
-        const unsigned long long q = has ? fixed_mass(key, lmax, inv_t) : 0ull;
-        // place in the descending order of keys (ties by ascending id) and in the ascending order of ids
-        int desc = 0, asc = 0;
-        for (int o = 0; o < n; ++o) {
-            const uint32_t ok = __shfl(key, o, kWave);
-            const int oi = __shfl(id, o, kWave);
-            desc += ok > key || (ok == key && oi < id);
-            asc += oi < id;
-        }
-        bool kept = has;
-        if (use_p) {
-            // cum = mass of the candidates before this one in descending order, itself included
-            unsigned long long cum = 0, total = 0;
-            for (int o = 0; o < n; ++o) {
-                const unsigned long long oq = shfl_u64(q, o);
-                const int od = __shfl(desc, o, kWave);
-                total += oq;
-                if (od <= desc) cum += oq;
-            }
-            const double target = static_cast<double>(tp) * static_cast<double>(total);
-            // the shortest prefix whose mass reaches the target: an element is kept when the prefix
-            // before it has not reached it yet; the first is always kept
-            kept = has && (desc == 0 || static_cast<double>(cum - q) < target);
-        }
-        const unsigned long long mass = kept ? q : 0ull;
-        unsigned long long before = 0, total = 0;
-        for (int o = 0; o < n; ++o) {
-            const unsigned long long om = shfl_u64(mass, o);
-            const int oa = __shfl(asc, o, kWave);
-            total += om;
-            if (oa < asc) before += om;
-        }
-        int token = imax;
-        if (total > 0ull) {
-            unsigned long long rr = static_cast<unsigned long long>(uniform[r] * static_cast<double>(total));
-            if (rr >= total) rr = total - 1;
-            const bool mine = kept && rr >= before && rr - before < mass;
-            const unsigned long long pick = __ballot(mine);
-            if (pick != 0ull) token = __shfl(id, __ffsll(static_cast<long long>(pick)) - 1, kWave);
-        }
-        if (lane == 0) {
-            out[r] = token;
-            if (scatter_index != nullptr) scatter_out[scatter_index[r]] = token;
-        }
+        if (wave == 0) wave_finish();
         return;
     }
 
@@ -578,9 +699,48 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         if (rr >= total) rr = total - 1;
         if (rr >= before && rr - before < wave_mass) {  // wave-uniform
             unsigned long long left = rr - before;
+            // The group where the walk ends, from the groups' masses in order. The sums over the
+            // lanes are taken for 8 groups at a time, their exchanges interleaved: one after the
+            // other (a scan per group, each waiting for the one before) they cost 16 us a row.
+            int gstar = -1;
+#pragma unroll
+            for (int g0 = 0; g0 < GROUPS; g0 += 8) {
+                unsigned long long tot[8];
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    tot[b] = 0ull;
+                    if (g0 + b < GROUPS) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int j = 4 * (g0 + b) + e;
+                            if (bits[j / 32] >> (j % 32) & 1u) tot[b] += fixed_mass(again(keys[j]), lmax, inv_t);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int off = kWave / 2; off > 0; off >>= 1) {
+#pragma unroll
+                    for (int b = 0; b < 8; ++b) {
+                        if (g0 + b < GROUPS) {
+                            const uint32_t lo = __shfl_xor(static_cast<uint32_t>(tot[b]), off, kWave);
+                            const uint32_t hi = __shfl_xor(static_cast<uint32_t>(tot[b] >> 32), off, kWave);
+                            tot[b] += (static_cast<unsigned long long>(hi) << 32) | lo;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    if (g0 + b < GROUPS && gstar < 0) {
+                        if (left < tot[b]) gstar = g0 + b;
+                        else left -= tot[b];
+                    }
+                }
+            }
+            // within that group: a scan over the lanes' four ids each
             int found = -1;
 #pragma unroll
             for (int g = 0; g < GROUPS; ++g) {
+                if (g != gstar) continue;  // the same for the whole wave
                 unsigned long long q[4], q4 = 0;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -594,25 +754,20 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
                     const unsigned long long o = shfl_up_u64(inc, d);
                     if (lane >= d) inc += o;
                 }
-                const unsigned long long group_total = shfl_u64(inc, kWave - 1);
-                if (found < 0) {
-                    if (left < group_total) {
-                        const unsigned long long pick = __ballot(q4 > 0ull && left >= inc - q4 && left < inc);
-                        const int src = __ffsll(static_cast<long long>(pick)) - 1;
-                        // within the lane's four ids
-                        unsigned long long rest = left - (inc - q4);
-                        int e_pick = 3;
+                const unsigned long long pick = __ballot(q4 > 0ull && left >= inc - q4 && left < inc);
+                if (pick != 0ull) {
+                    const int src = __ffsll(static_cast<long long>(pick)) - 1;
+                    // within the lane's four ids
+                    unsigned long long rest = left - (inc - q4);
+                    int e_pick = 3;
 #pragma unroll
-                        for (int e = 3; e >= 0; --e) {
-                            unsigned long long upto = 0;
+                    for (int e = 3; e >= 0; --e) {
+                        unsigned long long upto = 0;
 #pragma unroll
-                            for (int e2 = 0; e2 <= e; ++e2) upto += q[e2];
-                            if (q[e] > 0ull && rest < upto) e_pick = e;
-                        }
-                        found = __shfl(id_of(4 * g) + e_pick, src, kWave);
-                    } else {
-                        left -= group_total;
+                        for (int e2 = 0; e2 <= e; ++e2) upto += q[e2];
+                        if (q[e] > 0ull && rest < upto) e_pick = e;
                     }
+                    found = __shfl(id_of(4 * g) + e_pick, src, kWave);
                 }
             }
             if (lane == 0) result = found;
@@ -709,12 +864,13 @@ extern "C" int liyab_sample(int* out, const float* logits, int64_t ld, int rows,
     LIYAB_REQUIRE(scatter_index == nullptr || scatter_out != nullptr, "sample: a scatter index needs a target");
     // the row in registers where it fits; the general kernel beyond
 #define LIYAB_REGS(E, T) sample_registers_kernel<E, T><<<rows, T, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out)
-    if (V <= 8 * 1024) LIYAB_REGS(8, 1024);
-    else if (V <= 16 * 1024) LIYAB_REGS(16, 1024);
-    else if (V <= 48 * 512) LIYAB_REGS(48, 512);
-    else if (V <= 72 * 512) LIYAB_REGS(72, 512);
-    else if (V <= 104 * 512) LIYAB_REGS(104, 512);
-    else if (V <= 128 * 512) LIYAB_REGS(128, 512);
+    // (3 more ids than the row has: a row may start up to 3 entries past a multiple of 16 bytes)
+    if (V + 3 <= 8 * 1024) LIYAB_REGS(8, 1024);
+    else if (V + 3 <= 16 * 1024) LIYAB_REGS(16, 1024);
+    else if (V + 3 <= 48 * 512) LIYAB_REGS(48, 512);
+    else if (V + 3 <= 72 * 512) LIYAB_REGS(72, 512);
+    else if (V + 3 <= 104 * 512) LIYAB_REGS(104, 512);
+    else if (V + 3 <= 128 * 512) LIYAB_REGS(128, 512);
     else sample_kernel<<<rows, S_THREADS, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out);
 #undef LIYAB_REGS
     return check_launch("sample");

@@ -550,6 +550,9 @@ def test_sampler_against_the_plain_sampler(ops, V):
     logits = rnd(14, V, scale=2.0, seed=11)
     logits[5, 100:140] = 3.0  # many ties at the top-k boundary
     logits[12, :] = 0.25  # all equal: ties everywhere
+    logits[3, 7:60:2] = 9.0  # ties above the top-k boundary: all kept
+    logits[4, 10:50] = 8.0  # ties at the top: the 5 of the lowest ids are kept
+    logits[13, 300:900] = 7.5  # more ties at the boundary than keys the one-wave pool would hold at the large vocabularies
     params = [(0.0, 0, 1.0), (1.0, 0, 1.0), (0.8, 0, 1.0), (0.8, 40, 0.95), (1.3, 5, 1.0), (0.7, 20, 1.0), (1.0, 0, 0.5),
               (1.0, 0, 0.05), (0.5, 1, 1.0), (2.0, 999, 0.9), (1.0, 40, 0.0), (0.8, 0, 0.999), (1.0, 64, 0.7), (0.9, 65, 0.9)]
     cpu = logits.cpu().numpy()
