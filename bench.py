@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|xl] [--layers L]
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -33,7 +33,10 @@ MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 SMALL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 12, "n_embd": 768, "n_head": 12,
          "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "layer_norm_epsilon": 1e-5,
          "activation_function": "gelu_new", "tie_word_embeddings": True}
-FULL_LAYERS = 12
+# GPT-2's other sizes, for --size: the layer sizes and, with them, the number of layers
+WEIGHT_SEEDS = {"small": 10, "medium": 20, "xl": 30}
+SIZES = {"small": {}, "medium": {"n_layer": 24, "n_embd": 1024, "n_head": 16, "n_inner": 4096},
+         "xl": {"n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400}}
 
 
 def weight_bytes(cfg, elt):
@@ -129,7 +132,8 @@ def main():
     ap.add_argument("--steps", type=int, default=504)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the configuration has, if needed")
+    ap.add_argument("--size", default="small", choices=sorted(SIZES), help="GPT-2 small's sizes (the default), medium's or XL's")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has, if needed")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
@@ -142,12 +146,15 @@ def main():
 
     from liyab_amd.weights import write_random_model
 
-    cfg = dict(SMALL, n_layer=args.layers)
+    cfg = dict(SMALL, **SIZES[args.size])
+    full_layers = cfg["n_layer"]
+    if args.layers:
+        cfg["n_layer"] = args.layers
     ctx = cfg["n_positions"]
     steps = max(1, min(args.steps, ctx - args.prompt - args.warmup))
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     with tempfile.TemporaryDirectory() as d:
-        write_random_model(d, cfg, 10, dtype="bfloat16" if short == "bf16" else "float32")
+        write_random_model(d, cfg, WEIGHT_SEEDS[args.size], dtype="bfloat16" if short == "bf16" else "float32")
         engine = make_engine(d, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), ctx)
         if args.prefill_only:
             ptps, pms = prefill_run(engine, cfg, [1024, 1024], repeat=20)
@@ -156,15 +163,15 @@ def main():
         tps, ms, bytes_per_step = decode_run(engine, cfg, args.batch, args.prompt, steps, args.warmup)
         achieved = bytes_per_step / (ms * 1e-3) / 1e9
         out = {
-            "metric": "decode tok/s (GPT-2 small sizes, batch 8, 512-token prompts decoding to 1024)",
+            "metric": f"decode tok/s (GPT-2 {args.size} sizes, batch {args.batch}, {args.prompt}-token prompts decoding to {ctx})",
             "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": short, "data": "synthetic",
-            "config": {"model": "gpt2-small-sizes-random-weights", "n_layer": cfg["n_layer"], "n_layer_full": FULL_LAYERS,
+            "config": {"model": f"gpt2-{args.size}-sizes-random-weights", "n_layer": cfg["n_layer"], "n_layer_full": full_layers,
                        "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": cfg["n_embd"] // cfg["n_head"],
                        "n_inner": cfg["n_inner"], "vocab_size": cfg["vocab_size"], "n_positions": cfg["n_positions"],
                        "global_batch": args.batch, "seq_len": ctx, "prompt_len": args.prompt, "page_size": 64,
-                       "weights_seed": 10, "ids_seed": 11, "parallelism": "single-gpu"},
+                       "weights_seed": WEIGHT_SEEDS[args.size], "ids_seed": 11, "parallelism": "single-gpu"},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4)},
         }
