@@ -11,6 +11,13 @@
 // global side when loading and again when reading. Rows past M or N are
 // clamped to the last valid row; their results are never stored. MFMA
 // operand layout and the fixed-order sum over k are those of gemm_mfma.hip.
+//
+// The product may be cut over K into parts (blockIdx.y), one plane of 32-bit
+// sums a part, the first plane also taking the bias and the rows the product
+// is added to (themselves a sum of planes): the planes together are then the
+// residual stream after the product, as the streaming kernel of few rows
+// leaves it (gemm_skinny.hip). A product with few output tiles and a long K
+// covers the chip that way.
 #include "common.h"
 #include "epilogue.h"
 
@@ -36,6 +43,16 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const f32x4& v) {
 }
 
 constexpr int DBK = 64;      // k per stage
+constexpr int kEpiParts = 5;  // this file's own epilogue: a plane of sums a part of K
+
+// A product cut over K: tiles of K a part, floats between the planes, and what the first plane adds.
+struct PartsParams {
+    int kt_per_part;
+    int64_t part_stride;
+    const float* base;  // rows the product is added to, a sum of n_base planes [M, N]; or null
+    int n_base;
+    int64_t base_stride;
+};
 
 // Where a row's 16-byte pieces sit within the row. LDS has 64 banks of 4 bytes: a 16-byte read
 // serves 16 lanes a cycle, which read 16 consecutive rows at one piece index. Rows are 128 bytes,
@@ -46,7 +63,7 @@ __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
-                    EpiParams epi, int vec_ok, int page_shift) {
+                    EpiParams epi, int vec_ok, int page_shift, PartsParams parts) {
     // WM x WN waves, each with (BM / WM) x (BN / WN) of the tile in blocks of 32 x 32
     constexpr int WAVES = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int STAGE = (BM + BN) * DBK;      // elements per stage: the tile of a, then the tile of w
@@ -95,7 +112,15 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    const int nk = K / DBK;
+    int nk = K / DBK;
+    if constexpr (EPI == kEpiParts) {
+        // this workgroup's part of K: tiles [kt0, kt0 + nk)
+        const int kt0 = blockIdx.y * parts.kt_per_part;
+        nk = min(nk - kt0, parts.kt_per_part);
+        a += static_cast<int64_t>(kt0) * DBK;
+        w += static_cast<int64_t>(kt0) * DBK;
+        if (blockIdx.y > 0) epi.bias = nullptr;  // the bias goes to the first plane only
+    }
     constexpr int AHEAD = DSTAGES - 1;  // tiles of K in flight or in use beside the one being multiplied
 #pragma unroll
     for (int p = 0; p < AHEAD; ++p)
@@ -238,6 +263,15 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                     b4[q] = epi.bias != nullptr ? *reinterpret_cast<const f32x4*>(epi.bias + nb + 8 * q) : f32x4{0.f, 0.f, 0.f, 0.f};
                     if constexpr (EPI == kEpiResidual)
                         r4[q] = *reinterpret_cast<const f32x4*>(epi.residual + static_cast<int64_t>(m) * epi.ldr + nb + 8 * q);
+                    if constexpr (EPI == kEpiParts) {
+                        // the first part adds the rows the product is added to, their planes in order
+                        r4[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+                        if (blockIdx.y == 0 && parts.base != nullptr) {
+                            const float* bp = parts.base + static_cast<int64_t>(m) * N + nb + 8 * q;
+                            r4[q] = *reinterpret_cast<const f32x4*>(bp);
+                            for (int p = 1; p < parts.n_base; ++p) r4[q] += *reinterpret_cast<const f32x4*>(bp + p * parts.base_stride);
+                        }
+                    }
                 }
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
@@ -247,6 +281,9 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                     for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e] + b4[q][e];
                     if constexpr (EPI == kEpiResidual) {
                         *reinterpret_cast<f32x4*>(epi.residual + static_cast<int64_t>(m) * epi.ldr + n) = v + r4[q];
+                    } else if constexpr (EPI == kEpiParts) {
+                        float* plane = static_cast<float*>(epi.out) + blockIdx.y * parts.part_stride;
+                        *reinterpret_cast<f32x4*>(plane + static_cast<int64_t>(m) * N + n) = v + r4[q];
                     } else if constexpr (EPI == kEpiQkvPaged) {
                         if (n < epi.q_dim) {
                             store4<OutT>(static_cast<OutT*>(epi.out) + static_cast<int64_t>(m) * epi.ldo + n, v);
@@ -280,7 +317,20 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int n = n0 + wn * (BN / WN) + j * 32 + 8 * (r / 4) + 4 * g + r % 4;
-                if (n < N) epilogue_store<OutT, EPI>(epi, m, n, acc[i][j][r]);
+                if constexpr (EPI == kEpiParts) {
+                    if (n < N) {
+                        float v = acc[i][j][r] + epilogue_bias(epi, n);
+                        if (blockIdx.y == 0 && parts.base != nullptr) {
+                            const float* bp = parts.base + static_cast<int64_t>(m) * N + n;
+                            float b = bp[0];
+                            for (int p = 1; p < parts.n_base; ++p) b += bp[p * parts.base_stride];
+                            v += b;
+                        }
+                        (static_cast<float*>(epi.out) + blockIdx.y * parts.part_stride)[static_cast<int64_t>(m) * N + n] = v;
+                    }
+                } else {
+                    if (n < N) epilogue_store<OutT, EPI>(epi, m, n, acc[i][j][r]);
+                }
             }
     }
 }
@@ -313,8 +363,27 @@ int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, in
     bool vec16 = vec && sizeof(OutT) == 2 && N % 8 == 0;
     if (EPI == kEpiQkvPaged) vec16 = vec16 && epi.ldo % 8 == 0 && epi.hd % 8 == 0 && epi.q_dim % 8 == 0;
     else if (EPI != kEpiResidual) vec16 = vec16 && epi.ldo % 8 == 0;
-    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec16 ? 2 : (vec ? 1 : 0), page_shift);
+    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec16 ? 2 : (vec ? 1 : 0), page_shift, PartsParams{});
     return check_launch("gemm_mfma_dl");
+}
+
+// The product cut over K into `kparts` parts (see the head of this file); epi carries the planes
+// (out, float32, rows of N) and the first plane's bias.
+template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2>
+int launch_dl_parts(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, int kparts, const EpiParams& epi,
+                    const PartsParams& parts, hipStream_t stream) {
+    const dim3 grid(((N + BN - 1) / BN) * ((M + BM - 1) / BM), kparts);
+    const size_t smem = static_cast<size_t>(DSTAGES) * (BM + BN) * DBK * sizeof(bf16_t);
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, float, kEpiParts, WM, WN>;
+    static bool ready = false;
+    if (!ready) {
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        ready = true;
+    }
+    auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec = N % 4 == 0 && al16(epi.bias) && al16(epi.out) && al16(parts.base) && parts.part_stride % 4 == 0 && parts.base_stride % 4 == 0;
+    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, -1, parts);
+    return check_launch("gemm_mfma_dl_parts");
 }
 
 template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2>
@@ -339,11 +408,10 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
 
 using namespace liyab;
 
-// tile: 1 = 128x128, 2 = 64x64, 3 = 128x64, 5 = 128x192, each three stages deep and four waves; 6 = 64x64
-// with four stages; with eight waves: 7 = 128x128 three stages, 8 = 128x128 two stages (deeper rings
-// measured slower: their LDS leaves one workgroup a compute unit, and 288 tiles then take two rounds), 9 = 128x64;
-// 13 = 128x128 two stages on four waves, 16 = 64x32 four stages on two waves (for one tile of rows)
-// (0 = chosen from the shape).
+// tile: 2 = 64x64 tiles, three stages deep, on four waves; 6 = the same with four stages; 8 = 128x128, two
+// stages, on eight waves; 16 = 64x32, four stages, on two waves (for one tile of rows); 0 = chosen from
+// the shape. (Measured and dropped: 128x128 on four waves, 128x64, 128x192, and deeper rings under
+// 128x128, whose LDS leaves one workgroup a compute unit, so that 288 tiles take two rounds.)
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
@@ -360,16 +428,50 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
     // 17.3 for 2,048 x 2,304 x 768, 18.0 against 22.6 for 2,048 x 3,072 x 768)
     if (tile == 0) tile = K >= 2048 ? 6 : (static_cast<long>(M) * N >= 2048L * 2048L ? 8 : 2);
     switch (tile) {
-        case 1: return launch_dl<128, 128, 3>(a, lda, w, M, N, K, epi, stream);
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
-        case 3: return launch_dl<128, 64, 3>(a, lda, w, M, N, K, epi, stream);
-        case 5: return launch_dl<128, 192, 3>(a, lda, w, M, N, K, epi, stream);
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
-        case 7: return launch_dl<128, 128, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
-        case 9: return launch_dl<128, 64, 3, 4, 2>(a, lda, w, M, N, K, epi, stream);
-        case 13: return launch_dl<128, 128, 2, 2, 2>(a, lda, w, M, N, K, epi, stream);
         case 16: return launch_dl<64, 32, 4, 2, 1>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
+}
+
+// The same product cut over K: parts[p * part_stride + m * N + n] = sum over the p-th of `kparts` parts
+// of K (whole tiles of 64) of a[m, k] w[n, k]. With `base` (n_base planes [M, N], base_stride floats
+// apart, not overlapping `parts`) the first plane also takes bias[n] and base[0] + base[1] + ...;
+// without it `bias` must be null. tile: 6 = 64x64 tiles, 16 = 64x32 (for one tile of rows).
+extern "C" int liyab_gemm_mfma_dl_parts(const void* a, int64_t lda, const void* w, int M, int N, int K, int kparts, int tile,
+                                        float* parts, int64_t part_stride, const float* bias, const float* base, int n_base,
+                                        int64_t base_stride, hipStream_t stream) {
+    LIYAB_REQUIRE(a && w && parts, "gemm: null operand");
+    LIYAB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma_dl_parts: bad sizes M=%d N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE(K % DBK == 0 && lda % 8 == 0 && lda >= K, "gemm_mfma_dl_parts: K %d must be a multiple of 64 and lda %lld of 8", K,
+                  static_cast<long long>(lda));
+    LIYAB_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0,
+                  "gemm_mfma_dl_parts: operands must be 16-byte aligned");
+    const int nk = K / DBK;
+    LIYAB_REQUIRE(kparts >= 1 && kparts <= 16 && (kparts - 1) * ((nk + kparts - 1) / kparts) < nk,
+                  "gemm_mfma_dl_parts: K = %d does not cut into %d parts of whole tiles of 64", K, kparts);
+    LIYAB_REQUIRE(kparts == 1 || part_stride >= static_cast<int64_t>(M) * N, "gemm_mfma_dl_parts: planes of %lld overlap",
+                  static_cast<long long>(part_stride));
+    LIYAB_REQUIRE(base != nullptr || bias == nullptr, "gemm_mfma_dl_parts: a bias needs the rows it is added to");
+    if (base != nullptr) {
+        LIYAB_REQUIRE(n_base >= 1 && n_base <= 16 && (n_base == 1 || base_stride >= static_cast<int64_t>(M) * N),
+                      "gemm_mfma_dl_parts: bad planes of rows to add to (%d, %lld apart)", n_base, static_cast<long long>(base_stride));
+        const float* base_end = base + (n_base - 1) * base_stride + static_cast<int64_t>(M) * N;
+        const float* parts_end = parts + (kparts - 1) * part_stride + static_cast<int64_t>(M) * N;
+        LIYAB_REQUIRE(base_end <= parts || parts_end <= base, "gemm_mfma_dl_parts: the rows to add to overlap the planes written");
+    }
+    EpiParams epi{};
+    epi.mode = kEpiNone;
+    epi.out_dtype = kF32;
+    epi.out = parts;
+    epi.ldo = N;
+    epi.bias = bias;
+    const PartsParams pp{(nk + kparts - 1) / kparts, part_stride, base, n_base, base_stride};
+    auto* pa = static_cast<const bf16_t*>(a);
+    auto* pw = static_cast<const bf16_t*>(w);
+    if (tile == 6) return launch_dl_parts<64, 64, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
+    if (tile == 16) return launch_dl_parts<64, 32, 4, 2, 1>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
+    return fail(1, "gemm_mfma_dl_parts: unknown tile %d (6 or 16)", tile);
 }

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "liyab_gemm_simple": [P, c_int, c_int64, P, c_int64, P, c_int, P, P, c_int64, c_int, c_int, c_int, c_int, P],
     "liyab_gemm_mfma": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_gemm_mfma_dl": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_mfma_dl_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_skinny": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_generic": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, P],

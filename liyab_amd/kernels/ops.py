@@ -425,6 +425,32 @@ def gemm_skinny_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *,
               planes.data_ptr(), planes.stride(0), _ptr(bias), bptr, n_base, bstride, _stream())
 
 
+def gemm_mfma_dl_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+                       base: Optional[torch.Tensor] = None, tile: int = 6) -> None:
+    """The tiled matrix-core product cut over K (K a multiple of 64), as `gemm_skinny_parts` for
+    any number of rows: planes float32 [parts, M, N]; with `base` the first plane also takes
+    `bias` and the rows of `base`. tile: 6 = 64 x 64 tiles, 16 = 64 x 32."""
+    lda = _rows(a, "a")
+    M, K = a.shape
+    _dev(w, "w")
+    _dev(planes, "planes")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_mfma_dl_parts: needs bfloat16 a [M, K] and contiguous w [N, K], got {tuple(a.shape)} {a.dtype}, {tuple(w.shape)} {w.dtype}")
+    N = w.shape[0]
+    if planes.dtype != torch.float32 or planes.dim() != 3 or tuple(planes.shape[1:]) != (M, N) or not planes.is_contiguous():
+        raise KernelError(f"gemm_mfma_dl_parts: planes must be contiguous float32 [parts, {M}, {N}], got {tuple(planes.shape)}")
+    bptr, n_base, bstride = None, 0, 0
+    if base is not None:
+        bptr, n_base, bstride, b_rows, b_d = _planes(base, "gemm_mfma_dl_parts: base")
+        if (b_rows, b_d) != (M, N):
+            raise KernelError(f"gemm_mfma_dl_parts: base must have rows [{M}, {N}], got {tuple(base.shape)}")
+        _f32vec(bias, "bias", N)
+    elif bias is not None:
+        raise KernelError("gemm_mfma_dl_parts: a bias needs the rows it is added to (base)")
+    _lib.call("liyab_gemm_mfma_dl_parts", a.data_ptr(), lda, w.data_ptr(), M, N, K, planes.shape[0], tile,
+              planes.data_ptr(), planes.stride(0), _ptr(bias), bptr, n_base, bstride, _stream())
+
+
 def gemm_att_parts(partials: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                    base: Optional[torch.Tensor] = None) -> None:
     """The product cut over K (as `gemm_skinny_parts`) whose first operand is attention's output
@@ -474,6 +500,19 @@ def k_parts(M: int, N: int, K: int) -> int:
     while parts < 4 and groups * parts * 2 <= 256 and units // (parts * 2) >= 3:
         parts *= 2
     return parts
+
+
+def tiled_k_parts(M: int, N: int, K: int) -> int:
+    """Into how many parts of K the tiled product of one tile of rows (33 to 64) is best cut when
+    it is added to the residual stream (1: not at all). With few output features the 64 x 32
+    tiles are few and each walks the whole of K; cut over K they cover the chip: alone, at 64
+    rows, 3,072 -> 768 takes 8.2 us whole (the streaming kernel) and 4.9 in 8 parts, 6,400 ->
+    1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: only the
+    longest inner dimensions gain, in 4 parts (us a step of 12 layers at 64 rows, whole and
+    cut: GPT-2 XL's sizes 1360 and 1300; medium's 929 and 951, small's 799 and 828: not there)."""
+    if not 32 < M <= 64 or K % 64 != 0 or K < 6144 or N > 2048:
+        return 1
+    return 4
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,

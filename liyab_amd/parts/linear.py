@@ -24,6 +24,7 @@ from .norms import Normed
 # 420 / 471, 16 rows 498 / 524, 24 rows 657 / 679, 32 rows 711 / 694, 64 rows 954 / 810).
 FOLD_NORM = True
 FOLD_NORM_ROWS = 24
+TILED_PARTS = True  # products of 33 to 64 rows that are added to the stream: tiled and cut over K (ops.tiled_k_parts)
 
 
 def _fuses(a, w: torch.Tensor, residual) -> bool:
@@ -72,6 +73,10 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     if (a.dtype != torch.bfloat16 and not in_splits) or w.dtype != torch.bfloat16 or M > 64:
         return None
     parts = ops.k_parts(M, w.shape[0], K)
+    tiled = False
+    if parts <= 1 and not in_splits and TILED_PARTS:
+        parts = ops.tiled_k_parts(M, w.shape[0], K)  # one tile of 33 to 64 rows: the tiled kernel, cut over K
+        tiled = parts > 1
     if parts <= 1:
         return None
     split = isinstance(stream, SplitStream)
@@ -81,6 +86,8 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
         return None  # the stream's planes are where these would go
     if in_splits:
         ops.gemm_att_parts(a, w, planes, bias=bias, base=base)
+    elif tiled:
+        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=16)
     else:
         ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
     return SplitStream(planes, stream.home if split else stream)

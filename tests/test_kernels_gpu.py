@@ -144,6 +144,36 @@ def test_gemm_skinny_parts(ops, M, N, K, parts):
         ops.gemm_skinny_parts(a, w, planes, base=planes[:1])
 
 
+@pytest.mark.parametrize("tile", [6, 16])
+@pytest.mark.parametrize("M,N,K,parts", [(64, 768, 3072, 4), (2048, 768, 3072, 2), (200, 100, 448, 3), (33, 1600, 6400, 4), (1, 40, 64, 1),
+                                         (130, 777, 1088, 5)])
+def test_gemm_tiled_parts(ops, tile, M, N, K, parts):
+    """The tiled product cut over K: plane p holds the sums over the p-th part of K (whole tiles
+    of 64); with rows to add to, the first plane also takes them and the bias."""
+    a, w = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16)
+    planes = torch.full((parts, M, N), float("nan"), device=DEV)
+    ops.gemm_mfma_dl_parts(a, w, planes, tile=tile)
+    part_k = (K // 64 + parts - 1) // parts * 64
+    for q in range(parts):
+        lo, hi = q * part_k, min(K, (q + 1) * part_k)
+        close(planes[q], a[:, lo:hi].double() @ w[:, lo:hi].double().t(), 1e-5, f"part {q}")
+    product = a.double() @ w.double().t()
+    bias = rnd(N, seed=7)
+    for n_base in (0, 3):
+        base = rnd(M, N, seed=8, scale=3.0) if n_base == 0 else rnd(n_base, M, N, seed=9, scale=3.0)
+        for with_bias in (True, False):
+            based = torch.full((parts, M, N), float("nan"), device=DEV)
+            ops.gemm_mfma_dl_parts(a, w, based, bias=bias if with_bias else None, base=base, tile=tile)
+            assert torch.equal(based[1:], planes[1:])
+            rows = base.double() if n_base == 0 else base.double().sum(0)
+            close(based[0], planes[0].double() + rows + (bias.double() if with_bias else 0), 1e-6, f"first plane over {n_base} planes of rows")
+            close(based.double().sum(0), product + rows + (bias.double() if with_bias else 0), 1e-5, "sum with rows")
+    with pytest.raises(Exception, match="parts"):
+        ops.gemm_mfma_dl_parts(a, w, torch.empty(K // 64 + 2, M, N, device=DEV), tile=tile)
+    with pytest.raises(Exception, match="overlap"):
+        ops.gemm_mfma_dl_parts(a, w, planes, base=planes[:1], tile=tile)
+
+
 def gemm_reference(a, w, bias, epilogue, residual=None):
     y = a.double() @ w.double().t()
     if bias is not None:
@@ -183,7 +213,7 @@ def test_gemm_float32(ops, M, N, K, epilogue):
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
-                                    "dl1", "dl2", "dl3", "dl5", "dl6", "dl7", "dl8", "dl9", "dl13", "dl16"])
+                                    "dl2", "dl6", "dl8", "dl16"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
                                                  (500, 300, 128), (129, 193, 192)])
@@ -573,7 +603,7 @@ def test_sampler_against_the_plain_sampler(ops, V):
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, params[r], got[r], want)
 
 
-@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl5", "auto"])
+@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "auto"])
 @pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
     """Queries to a dense buffer, keys and values straight into shuffled cache slots, against

@@ -247,6 +247,40 @@ def test_feed_forward_deferred(parts, reader, split_before, monkeypatch):
     core.close("f")
 
 
+@pytest.mark.parametrize("split_before", [False, True])
+def test_product_of_a_tile_of_rows_deferred_through_the_tiled_kernel(parts, split_before, monkeypatch):
+    """A product of 33 to 64 rows that is added to the stream, cut over K through the tiled
+    kernel (forced here: the rule takes only long inner dimensions): the stream comes back split,
+    its planes adding up to stream + a . W^T + bias, whether it was whole or split before."""
+    from liyab_amd.engine import StepItem
+    from liyab_amd.kernels import ops
+    from liyab_amd.parts.base import SplitStream
+    from liyab_amd.parts.linear import linear_deferred
+
+    p, dtype = parts
+    if dtype != "bfloat16":
+        pytest.skip("only the bfloat16 products are cut over K")
+    monkeypatch.setattr(ops, "tiled_k_parts", lambda M, N, K: 3)
+    core = p.core
+    core.open("f")
+    ctx, _ = core.step_fn.prepare([StepItem("f", [1] * 40, [])])
+    rng = np.random.default_rng(5)
+    a = rand(rng, 40, 320).to(DEV).to(torch.bfloat16)
+    w = rand(rng, 72, 320, scale=0.1).to(DEV).to(torch.bfloat16)
+    bias = rand(rng, 72).to(DEV)
+    residual = rand(rng, 40, 72).to(DEV)
+    stream = residual
+    if split_before:
+        half = rand(rng, 40, 72).to(DEV)
+        stream = SplitStream(torch.stack([residual - half, half]), torch.full_like(residual, float("nan")))
+    assert ops.k_parts(40, 72, 320) == 1
+    split = linear_deferred(a, w, bias, ctx, "tiled_parts_test", stream)
+    assert isinstance(split, SplitStream) and split.planes.shape == (3, 40, 72)
+    want = f64(residual.cpu()) + f64(a.float().cpu()) @ f64(w.float().cpu()).T + f64(bias.cpu())
+    assert tt.rel_err(split.settle().cpu().numpy(), want) < 1e-5
+    core.close("f")
+
+
 @pytest.mark.parametrize("geometry", [dict(H=5, Hkv=5, hd=16), dict(H=6, Hkv=2, hd=32, d=96), dict(H=3, Hkv=1, hd=48, d=64, window=13)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_mixer_alone(dtype, geometry):
