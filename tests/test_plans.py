@@ -1,0 +1,47 @@
+"""The shape rules that choose among kernels (pure functions of sizes): no GPU needed."""
+
+import pytest
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from liyab_amd.kernels import ops as o
+
+    return o
+
+
+def test_parts_of_k_are_whole_and_none_is_empty(ops):
+    """A product cut over K: every part holds whole units of 64 and at least one of them, for
+    every shape the rules answer for."""
+    for M in (1, 3, 8, 16, 17, 24, 32, 33, 48, 64, 65, 200):
+        for N in (16, 100, 768, 1024, 1600, 2304, 4800, 50257):
+            for K in (8, 64, 72, 192, 768, 1024, 1600, 3072, 4096, 6400, 8192):
+                units = (K + 63) // 64
+                for parts in (ops.k_parts(M, N, K), ops.tiled_k_parts(M, N, K)):
+                    assert 1 <= parts <= 16
+                    per = (units + parts - 1) // parts
+                    assert (parts - 1) * per < units, (M, N, K, parts)
+                if ops.k_parts(M, N, K) > 1:
+                    assert M <= 32 and K % 8 == 0
+                if ops.tiled_k_parts(M, N, K) > 1:
+                    assert 32 < M <= 64 and K % 64 == 0
+
+
+def test_attention_split_plan(ops):
+    """Decode attention in splits: powers of two up to 8, a split keeping 128 keys or more of the
+    longest context, workgroups of 4 waves; one split when the context is short."""
+    for n_tokens in (1, 2, 8, 9, 16):
+        for n_head in (1, 3, 12, 25):
+            for bucket in (256, 512, 1024, 2048, 8192):
+                splits, waves = ops.decode_split_plan(n_tokens, n_head, bucket)
+                assert splits in (1, 2, 4, 8) and waves == 4
+                assert splits == 1 or bucket // splits >= 128
+                assert ops.att_parts_takes(n_tokens, splits, 64)
+    assert ops.decode_split_plan(1, 12, 256)[0] == 2 and ops.decode_split_plan(1, 12, 1024)[0] == 8
+    assert ops.decode_split_plan(16, 12, 1024)[0] == 4
+
+
+def test_what_the_folded_norm_takes(ops):
+    assert ops.skinny_ln_takes(1, 64) and ops.skinny_ln_takes(32, 2048)
+    assert not ops.skinny_ln_takes(33, 768) and not ops.skinny_ln_takes(8, 2056) and not ops.skinny_ln_takes(8, 100)
+    assert ops.norm_takes_planes(768) and not ops.norm_takes_planes(777) and not ops.norm_takes_planes(4096)
