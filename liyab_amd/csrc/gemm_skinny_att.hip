@@ -60,7 +60,7 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
     // -- the first operand: four consecutive k of a token a thread, merged over the splits ----
     const int per = pk / 4, items = M * per;
     struct Item {
-        floatx4 acc[4];
+        floatx4 acc[MAX_SPLITS];
         floatx2 ml[MAX_SPLITS];
         const float* p;
         int m, kk, e;
@@ -77,8 +77,10 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
         x.p = att.partials + (static_cast<int64_t>(x.m) * att.n_head + head) * S * hd4;
 #pragma unroll
         for (int s = 0; s < MAX_SPLITS; ++s) x.ml[s] = *reinterpret_cast<const floatx2*>(x.p + min(s, S - 1) * hd4 + att.hd);
+        // every split's values are asked for here, ahead of the weights: asked for after them
+        // (loads are counted in order) a wait for a split would be a wait for the weights
 #pragma unroll
-        for (int s = 0; s < 4; ++s) x.acc[s] = *reinterpret_cast<const floatx4*>(x.p + min(s, S - 1) * hd4 + x.e);
+        for (int s = 0; s < MAX_SPLITS; ++s) x.acc[s] = *reinterpret_cast<const floatx4*>(x.p + min(s, S - 1) * hd4 + x.e);
         return x;
     };
     auto finish = [&](const Item& x) {
@@ -95,14 +97,7 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
         }
         floatx4 o = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int s = 0; s < 4; ++s) o += wgt[s] * x.acc[s];
-        if (S > 4) {
-            floatx4 more[4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) more[s] = *reinterpret_cast<const floatx4*>(x.p + min(4 + s, S - 1) * hd4 + x.e);
-#pragma unroll
-            for (int s = 0; s < 4; ++s) o += wgt[4 + s] * more[s];
-        }
+        for (int s = 0; s < MAX_SPLITS; ++s) o += wgt[s] * x.acc[s];  // a split past the last weighs nothing
         if (x.valid) {
             uint2 packed;
             packed.x = static_cast<uint32_t>(float_to_bf16(o[0] / sum)) | (static_cast<uint32_t>(float_to_bf16(o[1] / sum)) << 16);
