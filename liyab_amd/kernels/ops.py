@@ -702,12 +702,16 @@ def prefill_takes(hd: int) -> bool:
 
 def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
     """(splits of the keys, waves per workgroup), from measurements at 12 heads of 64: with many
-    (token, head) pairs a workgroup of 4 waves per pair is fastest; with few, 16 waves per pair,
+    (token, head) pairs a workgroup of 4 waves per pair is fastest, with a few hundred one of 8
+    (us a decode step at batch 24 / 32 / 40 with 4, 8 and 16 waves: 610 595 654 / 648 633 692 /
+    706 698 755; at batch 48 and more 4 waves win by a little); with few, 16 waves per pair,
     merged in LDS, beat cutting the keys across workgroups plus a merge kernel up to a few
     thousand keys; beyond that the keys are also split across workgroups."""
     pairs = max(1, n_tokens * n_head)
     if pairs >= 512 or context_bucket <= 256:
         return 1, 4
+    if pairs >= 256:
+        return 1, 8
     return max(1, min(context_bucket // 2048, 32)), 16
 
 
