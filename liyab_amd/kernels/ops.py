@@ -503,16 +503,30 @@ def k_parts(M: int, N: int, K: int) -> int:
 
 
 def tiled_k_parts(M: int, N: int, K: int) -> int:
-    """Into how many parts of K the tiled product of one tile of rows (33 to 64) is best cut when
-    it is added to the residual stream (1: not at all). With few output features the 64 x 32
-    tiles are few and each walks the whole of K; cut over K they cover the chip: alone, at 64
-    rows, 3,072 -> 768 takes 8.2 us whole (the streaming kernel) and 4.9 in 8 parts, 6,400 ->
+    """Into how many parts of K the tiled product of more than 32 rows is best cut when it is
+    added to the residual stream (1: not at all). Several tiles of rows, few output features and
+    a long K (a prompt's portion through the feed-forward's second product: 128 x 768 x 3,072 is
+    24 tiles of 64 x 64, each walking the whole of K in 18.7 us): cut until the tiles cover the
+    chip. One tile of rows (33 to 64): the 64 x 32 tiles are few and each walks the whole of K;
+    cut over K they cover the chip: alone, at 64 rows, 3,072 -> 768 takes 8.2 us whole (the streaming kernel) and 4.9 in 8 parts, 6,400 ->
     1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: only the
     longest inner dimensions gain, in 4 parts (us a step of 12 layers at 64 rows, whole and
     cut: GPT-2 XL's sizes 1360 and 1300; medium's 929 and 951, small's 799 and 828: not there)."""
-    if not 32 < M <= 64 or K % 64 != 0 or K < 6144 or N > 2048:
+    if K % 64 != 0 or M <= 32:
         return 1
-    return 4
+    if M <= 64:
+        return 4 if K >= 6144 and N <= 2048 else 1
+    # several tiles of rows (a prompt's portion): 64 x 64 tiles, cut until they cover the chip,
+    # a part keeping 256 of K or more
+    tiles = (M + 63) // 64 * ((N + 63) // 64)
+    nk = K // 64
+    parts = 1
+    while parts < TILED_MAX_PARTS and tiles * parts * 2 <= 256 and nk // (parts * 2) >= 4:
+        parts *= 2
+    return parts
+
+
+TILED_MAX_PARTS = 4  # (us a step of 128 / 256 / 512 tokens of one prompt with at most 1, 2, 4, 8 parts: 765 665 637 668 / 809 720 694 679 / 922 843 842 846)
 
 
 def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: Optional[torch.Tensor], eps: float,
@@ -696,6 +710,9 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
               n_head, hkv, hd, page, _stream())
 
 
+PREFILL_KSPLIT4_WORK = 256  # tiles x heads up to which four waves share a tile of 64 queries' keys
+
+
 def prefill_takes(hd: int) -> bool:
     return hd % 16 == 0 and 16 <= hd <= 128
 
@@ -766,7 +783,8 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         if host.n_attn_tiles:
             # with fewer workgroups than compute units, two waves share each query group's keys:
             # the longest tile's walk over its keys is then the kernel's critical path, and halves
-            ksplit = 2 if host.n_attn_tiles * n_head <= 256 else 1
+            work = host.n_attn_tiles * n_head
+            ksplit = (4 if host.attn_tile == 64 and hd <= 64 and work <= PREFILL_KSPLIT4_WORK else 2) if work <= 256 else 1
             attention_prefill(out, q, k_cache, v_cache, block_tables, ctx.attn_work, host.n_attn_tiles, n_head=n_head,
                               scale=scale, window=window, tile=host.attn_tile, ksplit=ksplit)
         if host.n_attn_single:

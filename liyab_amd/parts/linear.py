@@ -70,7 +70,7 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     a = a.tensor() if isinstance(a, Normed) else a
     in_splits = a.dim() == 4  # attention's output as its splits [tokens, heads, splits, head size + 4]
     M, K = (a.shape[0], a.shape[1] * (a.shape[3] - 4)) if in_splits else a.shape
-    if (a.dtype != torch.bfloat16 and not in_splits) or w.dtype != torch.bfloat16 or M > 64:
+    if (a.dtype != torch.bfloat16 and not in_splits) or w.dtype != torch.bfloat16:
         return None
     parts = ops.k_parts(M, w.shape[0], K)
     tiled = False
@@ -87,7 +87,7 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     if in_splits:
         ops.gemm_att_parts(a, w, planes, bias=bias, base=base)
     elif tiled:
-        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=16)
+        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=16 if M <= 64 else 6)
     else:
         ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
     return SplitStream(planes, stream.home if split else stream)
