@@ -1,4 +1,4 @@
-// Attention's output projection for steps of at most 16 tokens, cut over its inner
+// Attention's output projection for steps of at most 32 tokens, cut over its inner
 // dimension, reading attention's output as the decode kernel's splits leave it.
 //
 // With few tokens in flight a (token, head) pair's keys are cut into splits over several
@@ -41,6 +41,7 @@ struct BaseSum {
     int64_t stride;
 };
 
+template <int MT>  // tiles of 16 rows
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, int K, float* __restrict__ out, int part_k,
                       int64_t part_stride, const float* __restrict__ bias, BaseSum base) {
@@ -52,7 +53,7 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
     const int pk = k_end - k_begin, units = (pk + 63) / 64;
     const int ldx = pk + 8;
     bf16_t* xs = reinterpret_cast<bf16_t*>(smem);  // [M][pk + 8]
-    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][256]
+    float* red = reinterpret_cast<float*>(smem + ((static_cast<size_t>(M) * ldx * 2 + 15) / 16) * 16);  // [waves][MT][256]
     out += blockIdx.z * part_stride;
     const u32x4 zero = {0, 0, 0, 0};
     const int S = att.n_splits, hd4 = att.hd + 4;
@@ -124,8 +125,8 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
     };
     Frag wc[2][2];
     load_w(wave * 2, wc);
-    const int e_m = tid / 16, e_n = n0 + tid % 16;
-    const bool e_mine = tid < 256 && e_m < M && e_n < N;
+    const int e_m = 16 * (tid / 256) + (tid % 256) / 16, e_n = n0 + tid % 16;  // tile tid / 256 of rows
+    const bool e_mine = tid < MT * 256 && e_m < M && e_n < N;
     const bool based = base.planes != nullptr && blockIdx.z == 0;
     const float e_bias = (e_mine && based && bias != nullptr) ? bias[e_n] : 0.0f;
     float e_base[4];
@@ -145,17 +146,25 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
     lds_barrier();  // the weights may still be on their way
 
     // -- the product ---------------------------------------------------------------------
-    const bf16_t* arow = xs + min(i, M - 1) * ldx;
-    floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bf16_t* arow[MT];
+    floatx4 acc[MT];
+#pragma unroll
+    for (int r = 0; r < MT; ++r) {
+        arow[r] = xs + min(16 * r + i, M - 1) * ldx;
+        acc[r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     auto multiply = [&](int u0) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int kk = (u0 + p) * 64 + g * 8;  // within the part
-            Frag x0, x1;
-            x0.u = piece(arow, kk, pk);
-            x1.u = piece(arow, kk + 32, pk);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][0].v, x0.v, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][1].v, x1.v, acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < MT; ++r) {
+                Frag x0, x1;
+                x0.u = piece(arow[r], kk, pk);
+                x1.u = piece(arow[r], kk + 32, pk);
+                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][0].v, x0.v, acc[r], 0, 0, 0);
+                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[p][1].v, x1.v, acc[r], 0, 0, 0);
+            }
         }
     };
     int u0 = wave * 2;
@@ -170,14 +179,16 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
         }
     }
     multiply(u0);  // a wave past the end of the part holds zeros
-    // acc[r] = partial C^T[n = 4 g + r][m = i]; kept [m][n] per wave, added up in wave order
+    // acc[r][c] = partial C^T[n = 4 g + c][m = 16 r + i]; kept [tile][m][n] per wave, added up in wave order
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave * 256 + i * 16 + 4 * g + r] = acc[r];
+    for (int r = 0; r < MT; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) red[(wave * MT + r) * 256 + i * 16 + 4 * g + c] = acc[r][c];
     __syncthreads();
-    if (tid < 256) {
+    if (tid < MT * 256) {
         float v = 0.0f;
 #pragma unroll
-        for (int q = 0; q < WAVES; ++q) v += red[q * 256 + tid];
+        for (int q = 0; q < WAVES; ++q) v += red[q * MT * 256 + tid];
         if (e_mine) {
             if (based) {
                 // this plane = (sums + bias) + (base planes added up in their order)
@@ -202,14 +213,14 @@ using namespace liyab;
 // parts[p] = merged(partials) . w^T summed over the p-th of `kparts` parts of K = n_head * hd,
 // one plane [M, N] of 32-bit sums a part. partials [M][n_head][n_splits][hd + 4] float32 as
 // liyab_attention_decode leaves them with `leave_splits` (row m is token slot m); w [N, K]
-// bfloat16. M <= 16, n_splits <= 8, hd a multiple of 8. With `base` (n_base planes [M, N],
+// bfloat16. M <= 32, n_splits <= 8, hd a multiple of 8. With `base` (n_base planes [M, N],
 // base_stride floats apart, not overlapping `parts`) the first plane also takes bias[n] and the
 // rows base[0] + base[1] + ...; without it `bias` must be null.
 extern "C" int liyab_gemm_att_parts(const float* partials, int n_splits, int n_head, int hd, const void* w, int M, int N,
                                     int kparts, float* parts, int64_t part_stride, const float* bias, const float* base,
                                     int n_base, int64_t base_stride, hipStream_t stream) {
     LIYAB_REQUIRE(partials && w && parts, "gemm_att_parts: null operand");
-    LIYAB_REQUIRE(M >= 0 && M <= 16 && N > 0 && n_head > 0, "gemm_att_parts: bad sizes M=%d (at most 16) N=%d heads=%d", M, N, n_head);
+    LIYAB_REQUIRE(M >= 0 && M <= 32 && N > 0 && n_head > 0, "gemm_att_parts: bad sizes M=%d (at most 32) N=%d heads=%d", M, N, n_head);
     LIYAB_REQUIRE(hd >= 8 && hd <= 256 && hd % 8 == 0, "gemm_att_parts: head size %d is not a multiple of 8 in 8..256", hd);
     LIYAB_REQUIRE(n_splits >= 1 && n_splits <= att_proj::MAX_SPLITS, "gemm_att_parts: %d splits (1 to %d)", n_splits, att_proj::MAX_SPLITS);
     const int K = n_head * hd;
@@ -229,11 +240,14 @@ extern "C" int liyab_gemm_att_parts(const float* partials, int n_splits, int n_h
     }
     if (M == 0) return 0;
     const int part_k = (units + kparts - 1) / kparts * 64;
-    const size_t smem = ((static_cast<size_t>(M) * (part_k + 8) * 2 + 15) / 16) * 16 + att_proj::WAVES * 256 * sizeof(float);
+    const int mt = M <= 16 ? 1 : 2;
+    const size_t smem = ((static_cast<size_t>(M) * (part_k + 8) * 2 + 15) / 16) * 16 + att_proj::WAVES * mt * 256 * sizeof(float);
     LIYAB_REQUIRE(smem <= 64 * 1024, "gemm_att_parts: %d rows of a part of %d do not fit LDS", M, part_k);
     const dim3 grid((N + 15) / 16, 1, kparts);
-    att_proj::gemm_att_parts_kernel<<<grid, 64 * att_proj::WAVES, smem, stream>>>(
-        att_proj::Splits{partials, n_splits, n_head, hd}, static_cast<const bf16_t*>(w), M, N, K, parts, part_k, part_stride, bias,
-        att_proj::BaseSum{base, n_base, base_stride});
+    const att_proj::Splits att{partials, n_splits, n_head, hd};
+    const att_proj::BaseSum bs{base, n_base, base_stride};
+    auto* pw = static_cast<const bf16_t*>(w);
+    if (mt == 1) att_proj::gemm_att_parts_kernel<1><<<grid, 64 * att_proj::WAVES, smem, stream>>>(att, pw, M, N, K, parts, part_k, part_stride, bias, bs);
+    else att_proj::gemm_att_parts_kernel<2><<<grid, 64 * att_proj::WAVES, smem, stream>>>(att, pw, M, N, K, parts, part_k, part_stride, bias, bs);
     return check_launch("gemm_att_parts");
 }

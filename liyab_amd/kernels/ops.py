@@ -454,7 +454,7 @@ def gemm_mfma_dl_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *
 def gemm_att_parts(partials: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                    base: Optional[torch.Tensor] = None) -> None:
     """The product cut over K (as `gemm_skinny_parts`) whose first operand is attention's output
-    still in splits: partials float32 [M <= 16, heads, splits <= 8, head size + 4] as
+    still in splits: partials float32 [M <= 32, heads, splits <= 8, head size + 4] as
     `attention_decode(..., leave_splits=True)` leaves them, merged as they are loaded.
     w [N, heads * head size] bfloat16, planes float32 [parts, M, N]."""
     _dev(partials, "partials")
@@ -484,7 +484,7 @@ def gemm_att_parts(partials: torch.Tensor, w: torch.Tensor, planes: torch.Tensor
 
 
 def att_parts_takes(M: int, splits: int, hd: int) -> bool:
-    return 0 < M <= 16 and 1 <= splits <= 8 and hd % 8 == 0 and 8 <= hd <= 256
+    return 0 < M <= 32 and 1 <= splits <= 8 and hd % 8 == 0 and 8 <= hd <= 256
 
 
 def k_parts(M: int, N: int, K: int) -> int:
@@ -740,10 +740,16 @@ def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int):
     16 390 / 444 / 588. So: workgroups of 4 waves, 8 splits (4 from a hundred pairs on), a
     split keeping 128 keys or more of the longest context."""
     pairs = max(1, n_tokens * n_head)
+    most = 8 if pairs <= 96 else (4 if pairs <= SPLIT4_PAIRS else (2 if pairs <= SPLIT2_PAIRS else 1))
     splits = 1
-    while splits < (8 if pairs <= 96 else 4) and context_bucket // (2 * splits) >= 128:
+    while splits < most and context_bucket // (2 * splits) >= 128:
         splits *= 2
     return splits, 4
+
+
+# pairs up to which 4 and 2 splits are taken (beyond 16 tokens splits lost: us a step at batch 17 / 24 / 32
+# uncut 529 / 594 / 633, in 4 splits 568 / 630 / 708, in 2 splits 573 / 635 / 704)
+SPLIT4_PAIRS, SPLIT2_PAIRS = 192, 192
 
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

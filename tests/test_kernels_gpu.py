@@ -405,6 +405,7 @@ ATT_CASES = [
     ([100], [100], 2, 1, 128, 16),
     ([90, 31], [1, 1], 2, 2, 256, 16),
     ([50, 3], [4, 3], 3, 3, 80, 4),
+    ([300, 40, 90], [8, 8, 8], 4, 2, 64, 16),
 ]
 
 
@@ -438,7 +439,7 @@ def test_attention_decode(ops, case_id, splits, waves, window):
 
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("splits", [2, 4, 7, 8])
-@pytest.mark.parametrize("case_id", [0, 1, 3, 5, 6])
+@pytest.mark.parametrize("case_id", [0, 1, 2, 3, 5, 6, 7])
 def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window):
     """Attention that leaves each (token, head) pair's keys in splits, and the projection cut
     over its inner dimension that merges them as it loads them: the planes add up to rows +
@@ -469,7 +470,7 @@ def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window)
         for n_base in (None, 0, 2):
             base = None if n_base is None else (rnd(n, N, seed=8, scale=3.0) if n_base == 0 else rnd(n_base, n, N, seed=9, scale=3.0))
             planes = torch.full((parts, n, N), float("nan"), device=DEV)
-            if n > 16:
+            if n > 32:
                 with pytest.raises(Exception, match="outside"):
                     ops.gemm_att_parts(partials, w, planes, bias=bias if base is not None else None, base=base)
                 continue

@@ -30,7 +30,7 @@ def test_parts_of_k_are_whole_and_none_is_empty(ops):
 def test_attention_split_plan(ops):
     """Decode attention in splits: powers of two up to 8, a split keeping 128 keys or more of the
     longest context, workgroups of 4 waves; one split when the context is short."""
-    for n_tokens in (1, 2, 8, 9, 16):
+    for n_tokens in (1, 2, 8, 9, 16, 17, 32):
         for n_head in (1, 3, 12, 25):
             for bucket in (256, 512, 1024, 2048, 8192):
                 splits, waves = ops.decode_split_plan(n_tokens, n_head, bucket)
