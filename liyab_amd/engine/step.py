@@ -85,6 +85,7 @@ def attn_tile_for(q_lens) -> int:
     queries are twice as many, and four waves instead of two share each walk."""
     long_tokens = int(sum(int(q) for q in q_lens if q > DECODE_Q_LEN))
     return ATTN_TILE_FEW if long_tokens <= ATTN_FEW_TOKENS else ATTN_TILE
+GRAPH_AFTER_MIXED = 3  # eager runs of a shape with prompt portions before it is captured
 DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
 
 
@@ -103,7 +104,7 @@ class StepFunction:
     the shape: the ones in this package do."""
 
     def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0", use_graphs: bool = True,
-                 max_graphs: int = 64):
+                 max_graphs: int = 256):
         self.model = model
         self.manager = manager
         self.storage = storage
@@ -152,7 +153,9 @@ class StepFunction:
             self._graph_generation = self.workspace.generation
         key = (ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows, ctx.host.attention_mode, ctx.host.context_bucket,
                ctx.host.n_attn_tiles, ctx.host.attn_tile, ctx.host.n_attn_single)
-        entry = self._graphs.get(key)
+        entry = self._graphs.pop(key, None)
+        if entry is not None:
+            self._graphs[key] = entry  # back in as the most recently used (a dict keeps insertion order)
         if isinstance(entry, tuple):
             entry[0].replay()
             self.graph_replays += 1
@@ -160,8 +163,18 @@ class StepFunction:
         if entry is None:
             # first sight: run eagerly, which also sizes every workspace buffer for this shape
             if len(self._graphs) >= self.max_graphs:
-                self._graphs.pop(next(iter(self._graphs)))
+                # make room: a shape seen once and never again before a captured graph, the least
+                # recently used of either (a serving loop sees many one-off mixes of portions and
+                # decoded tokens between its recurring decode-only shapes)
+                victim = next((k for k, v in self._graphs.items() if not isinstance(v, tuple)), None)
+                self._graphs.pop(victim if victim is not None else next(iter(self._graphs)))
             self._graphs[key] = 1
+            return self.model.forward(ctx, self.storage)
+        # A decode-only shape comes back step after step: captured at its second sight. A mix of
+        # prompt portions and decoded tokens mostly does not, and a capture costs about two eager
+        # runs: captured only once it has shown that it recurs.
+        if entry < (1 if ctx.host.attention_mode == "decode" else GRAPH_AFTER_MIXED):
+            self._graphs[key] = entry + 1
             return self.model.forward(ctx, self.storage)
         before = self.workspace.generation
         graph = torch.cuda.CUDAGraph()
