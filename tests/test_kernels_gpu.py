@@ -664,3 +664,44 @@ def test_folded_norm_with_the_paged_qkv_epilogue(ops, M, H, Hkv, hd, K, page):
         else:
             close(g, t, 8e-3, what)
     assert (got[0] == 0).sum() == (want[0] == 0).sum()  # nothing written outside the tokens' slots
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_drawn_shapes_of_the_folded_and_the_cut_products(ops, seed):
+    """Shapes drawn at random (rows, widths that are multiples of 8 only, any number of output
+    features, planes up to 16, rows to add to in up to 9 planes): the folded norm against norm +
+    product, the cut products against the whole product."""
+    import random
+
+    rng = random.Random(seed)
+    for _ in range(12):
+        M = rng.choice([1, 2, 7, 8, 9, 16, 17, 31, 32])
+        K, N, P = 8 * rng.randint(1, 256), rng.randint(1, 700), rng.choice([1, 1, 2, 4, 5, 16])
+        planes = rnd(P, M, K, scale=2.0, seed=rng.randint(0, 99))
+        planes[0] += 0.5
+        x = planes if P > 1 else planes[0]
+        lw, lb = rnd(K, seed=5) + 1.0, rnd(K, seed=6)
+        w, bias = rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_skinny_ln(x, lw, lb, 1e-5, w, bias, out=out, epilogue=ops.EPI_GELU_TANH, wide=rng.choice([0, 1]) if M <= 16 else 0)
+        normed = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+        ops.layernorm(normed, x, lw, lb, 1e-5)
+        two = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.gemm(normed, w, bias, out=two, epilogue=ops.EPI_GELU_TANH)
+        close(out, two, 1e-2, f"folded norm M={M} K={K} N={N} planes={P}")
+    for _ in range(12):
+        M, K, N = rng.choice([1, 5, 16, 33, 64]), 8 * rng.randint(8, 400), rng.randint(1, 300)
+        units = (K + 63) // 64
+        parts = rng.randint(1, min(8, units))
+        if (parts - 1) * ((units + parts - 1) // parts) >= units:
+            parts = 1
+        a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+        base = rnd(rng.choice([1, 2, 4, 5, 9]), M, N, seed=3)
+        want = a.double() @ w.double().t() + bias.double() + base.double().sum(0)
+        planes = torch.full((parts, M, N), float("nan"), device=DEV)
+        ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
+        close(planes.double().sum(0), want, 1e-5, f"streaming product in parts M={M} K={K} N={N} parts={parts}")
+        if K % 64 == 0 and parts <= K // 64 and (parts - 1) * ((K // 64 + parts - 1) // parts) < K // 64:
+            planes = torch.full((parts, M, N), float("nan"), device=DEV)
+            ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=rng.choice([6, 16]))
+            close(planes.double().sum(0), want, 1e-5, f"tiled product in parts M={M} K={K} N={N} parts={parts}")
