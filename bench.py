@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|xl] [--layers L]
+    python bench.py --sequences 1,2,4,8 [-n 128]     # together against in turns, and whether replies are the same
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -126,6 +127,40 @@ def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
     return n / best, best * 1e3
 
 
+def sequences_run(engine, cfg, counts, prompt_len, n_new, seed=13):
+    """Several sequences generated together against the same sequences one after the other, as
+    the reference's liyab-seq-bench reports them (tools/liyab_seq_bench.cpp:1-32): total tokens
+    a second both ways, the gain, and whether every reply equals its reply alone. Greedy, and
+    with a seeded temperature."""
+    import numpy as np
+    import torch
+
+    from liyab_amd import SamplingParams
+
+    rng = np.random.default_rng(seed)
+    engine.stop_at_eos = False
+    out = []
+    for count in counts:
+        prompts = [rng.integers(0, cfg["vocab_size"], prompt_len).tolist() for _ in range(count)]
+        for name, make in (("greedy", lambda i: SamplingParams(temperature=0.0, max_tokens=n_new)),
+                           ("temperature 0.8", lambda i: SamplingParams(temperature=0.8, top_k=40, top_p=0.95, seed=100 + i, max_tokens=n_new))):
+            for _ in range(2):  # the second run replays captured graphs
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                together = engine.generate(prompts, [make(i) for i in range(count)])
+                torch.cuda.synchronize()
+                t_together = time.perf_counter() - t0
+                t0 = time.perf_counter()
+                alone = [engine.generate([p], [make(i)])[0] for i, p in enumerate(prompts)]
+                torch.cuda.synchronize()
+                t_turns = time.perf_counter() - t0
+            total = sum(len(r.tokens) for r in together)
+            out.append({"sequences": count, "sampling": name, "together_tok_s": round(total / t_together, 1),
+                        "in_turns_tok_s": round(total / t_turns, 1), "gain": round(t_turns / t_together, 2),
+                        "same": all(a.tokens == b.tokens for a, b in zip(together, alone))})
+    return {"metric": "sequences together against in turns", "prompt_len": prompt_len, "new_tokens": n_new, "runs": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +173,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill of 2,048 tokens (for profiling)")
+    ap.add_argument("--sequences", default="", help="e.g. 1,2,4: that many sequences together against one after the other "
+                    "(the reference's liyab-seq-bench): tokens a second both ways and whether every reply equals its reply alone")
+    ap.add_argument("-n", type=int, default=128, help="tokens generated per sequence with --sequences")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -156,6 +194,9 @@ def main():
     with tempfile.TemporaryDirectory() as d:
         write_random_model(d, cfg, WEIGHT_SEEDS[args.size], dtype="bfloat16" if short == "bf16" else "float32")
         engine = make_engine(d, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), ctx)
+        if args.sequences:
+            print(json.dumps(sequences_run(engine, cfg, [int(x) for x in args.sequences.split(",")], args.prompt, args.n)))
+            return 0
         if args.prefill_only:
             ptps, pms = prefill_run(engine, cfg, [1024, 1024], repeat=20)
             print(json.dumps({"prefill": {"value": round(ptps, 1), "tokens": 2048, "ms": round(pms, 4)}}))
