@@ -64,14 +64,19 @@ class Workspace:
 
     def __init__(self, device):
         self.device = torch.device(device)
-        self._bufs: Dict[str, torch.Tensor] = {}
+        self._bufs: Dict[tuple, torch.Tensor] = {}
+        self._views: Dict[tuple, tuple] = {}  # the last view handed out under a name: (shape, tensor)
         self.generation = 0  # counts reallocations: captured graphs hold the old addresses
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        key = (name, dtype)
+        shape = tuple(shape)
+        hit = self._views.get(key)
+        if hit is not None and hit[0] == shape:
+            return hit[1]  # the same view as last time: most calls of a decode loop
         n = 1
         for s in shape:
             n *= int(s)
-        key = f"{name}/{dtype}"
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
             cap = max(n, 1)
@@ -80,7 +85,9 @@ class Workspace:
             buf = torch.empty(cap, dtype=dtype, device=self.device)
             self.generation += 1
             self._bufs[key] = buf
-        return buf[:n].view(*shape)
+        view = buf[:n].view(*shape)
+        self._views[key] = (shape, view)
+        return view
 
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
