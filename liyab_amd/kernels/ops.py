@@ -336,6 +336,13 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, t
 EPI_QKV_PAGED = 4
 
 
+class _Rows:
+    """What `_epilogue` reads of a first operand that is no tensor: its rows and its dtype."""
+
+    def __init__(self, rows: int, dtype: torch.dtype):
+        self.shape, self.dtype = (rows, 0), dtype
+
+
 def _epilogue(a, w, bias, out, residual, epilogue, kv):
     """Checks the epilogue's operands against [M, N] and fills the launchers' struct."""
     M, N = a.shape[0], w.shape[0]
@@ -545,8 +552,7 @@ def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: 
         raise KernelError("gemm_skinny_ln: the residual epilogue is not taken")
     _f32vec(ln_weight, "norm weight", K)
     _f32vec(ln_bias, "norm bias", K)
-    fake_a = torch.empty((M, 0), dtype=torch.bfloat16, device="meta")  # shapes only, for the epilogue's checks
-    e = _epilogue(fake_a, w, bias, out, None, epilogue, kv)
+    e = _epilogue(_Rows(M, torch.bfloat16), w, bias, out, None, epilogue, kv)
     e.exact = 0
     _lib.call("liyab_gemm_skinny_ln", ptr, n_parts, stride, _ptr(ln_weight), _ptr(ln_bias), float(eps),
               w.data_ptr(), M, w.shape[0], K, wide, ctypes.byref(e), _stream())
