@@ -96,6 +96,7 @@ def main(argv=None) -> int:
         engine = Engine(model_dir, dtype=args.dtype, device=args.device, page_size=args.page_size,
                         num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
                         max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk, ctx=args.ctx)
+        engine.warmup()  # kernels' code loaded here, not inside the first turn's time to first token
     except LiyabError as e:
         print(f"liyab-cli: {e}", file=sys.stderr)
         return 1

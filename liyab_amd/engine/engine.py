@@ -75,6 +75,24 @@ class Engine:
         self._host_tokens = [None, None]
         self._turn = 0
 
+    def warmup(self) -> None:
+        """Runs a short prompt and a few decoded tokens of a request of its own and drops it: the
+        first launch of a kernel loads its code, which would otherwise count into the first
+        request's time to first token."""
+        rid = ("warmup", id(self))
+        n = max(1, min(9, self.core.model.max_positions - 4))
+        self.core.open(rid)
+        try:
+            logits = self.core.step([StepItem(rid, [0] * n, [n - 1])])
+            for _ in range(3):  # eager, then captured, then replayed
+                self.sampler.sample(logits, [SamplingParams(temperature=0.0)], [1], [0])
+                self.sampler.sample(logits, [SamplingParams(seed=1)], [1], [0])
+                if self.core.manager.length(rid) + 1 >= self.core.model.max_positions:
+                    break
+                logits = self.core.step([StepItem(rid, [0], [0])])
+        finally:
+            self.core.close(rid)
+
     # -- plumbing ---------------------------------------------------------------
     def _reset_slot(self, rid: Hashable) -> None:
         if self.core.storage.states:
