@@ -223,6 +223,9 @@ def test_greedy_generation_through_the_entry_point(name, dtype, model_dirs, plai
     engine = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=40, max_num_seqs=4, max_batched_tokens=64,
                     prefill_chunk=5 if name == "A" else 48)
     engine.stop_at_eos = False
+    if name == "B":  # a warm-up beforehand leaves nothing behind
+        engine.warmup()
+        assert engine.core.manager.pages_in_use() == 0
     results = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new))
     for prompt, res in zip(prompts, results):
         want_n = min(n_new, cfg["n_positions"] - len(prompt) + 1)
