@@ -65,9 +65,11 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     bf16_t* const Vb = Kb + 2 * STAGE;                     // [2][VSTAGE]
     __shared__ __attribute__((aligned(16))) bf16_t Os[QG][32 * LDK];
 
-    const int* wk = work + 4 * blockIdx.x;
+    // heads vary fastest: the work list has the longest tiles first, and workgroups start in the
+    // grid's order, so that every head's longest tile starts before anybody's short one
+    const int* wk = work + 4 * blockIdx.y;
     const int seq = wk[0], row0 = wk[1], pos0 = wk[2], nq = wk[3];
-    const int h = blockIdx.y;
+    const int h = blockIdx.x;
     const int hkv = h / (n_head / n_kv_head);
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int qg = wave % QG, ks = wave / QG;
@@ -321,7 +323,7 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
         if ((1 << b) == page_size) page_shift = b;
-    dim3 grid(n_tiles, n_head);
+    dim3 grid(n_head, n_tiles);
     auto* o = static_cast<bf16_t*>(out);
     auto* pq = static_cast<const bf16_t*>(q);
     auto* pk = static_cast<const bf16_t*>(kc);
