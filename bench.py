@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|xl] [--layers L]
     python bench.py --sequences 1,2,4,8 [-n 128]     # together against in turns, and whether replies are the same
+    python bench.py --prefill-tokens 512,2048,8192   # prefill tokens a second per length
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -173,6 +174,8 @@ def main():
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill of 2,048 tokens (for profiling)")
+    ap.add_argument("--prefill-tokens", default="", help="e.g. 512,2048,8192: best-of-5 prefill tokens a second per length, "
+                    "in prompts of up to 1,024 tokens (the reference's liyab-bench --prefill --tokens)")
     ap.add_argument("--sequences", default="", help="e.g. 1,2,4: that many sequences together against one after the other "
                     "(the reference's liyab-seq-bench): tokens a second both ways and whether every reply equals its reply alone")
     ap.add_argument("-n", type=int, default=128, help="tokens generated per sequence with --sequences")
@@ -193,7 +196,20 @@ def main():
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     with tempfile.TemporaryDirectory() as d:
         write_random_model(d, cfg, WEIGHT_SEEDS[args.size], dtype="bfloat16" if short == "bf16" else "float32")
-        engine = make_engine(d, args.dtype, max(args.batch, 64 if not args.no_points else args.batch), ctx)
+        slots = max(args.batch, 64 if not args.no_points else args.batch)
+        if args.prefill_tokens:
+            slots = max(slots, max(-(-int(x) // ctx) for x in args.prefill_tokens.split(",")))
+        engine = make_engine(d, args.dtype, slots, ctx)
+        if args.prefill_tokens:
+            runs = []
+            for total in [int(x) for x in args.prefill_tokens.split(",")]:
+                lens = [ctx] * (total // ctx) + ([total % ctx] if total % ctx else [])
+                ptps, pms = prefill_run(engine, cfg, lens)
+                flops = prefill_flops(cfg, lens, len(lens))
+                runs.append({"tokens": total, "prompts": len(lens), "value": round(ptps, 1), "ms": round(pms, 4),
+                             "frac": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)})
+            print(json.dumps({"metric": f"prefill tok/s (GPT-2 {args.size} sizes)", "dtype": short, "runs": runs}))
+            return 0
         if args.sequences:
             print(json.dumps(sequences_run(engine, cfg, [int(x) for x in args.sequences.split(",")], args.prompt, args.n)))
             return 0
