@@ -45,3 +45,16 @@ def test_what_the_folded_norm_takes(ops):
     assert ops.skinny_ln_takes(1, 64) and ops.skinny_ln_takes(32, 2048)
     assert not ops.skinny_ln_takes(33, 768) and not ops.skinny_ln_takes(8, 2056) and not ops.skinny_ln_takes(8, 100)
     assert ops.norm_takes_planes(768) and not ops.norm_takes_planes(777) and not ops.norm_takes_planes(4096)
+
+
+def test_attention_tile_of_a_step():
+    """Steps whose long portions hold few tokens take query tiles of 64, others of 128; short
+    portions (taken token by token) do not count."""
+    from liyab_amd.engine import step
+
+    assert step.attn_tile_for([1, 1, 1]) == step.ATTN_TILE_FEW
+    assert step.attn_tile_for([256, 1, 8]) == step.ATTN_TILE_FEW
+    assert step.attn_tile_for([1024]) == step.ATTN_TILE_FEW
+    assert step.attn_tile_for([1024, 9]) == step.ATTN_TILE
+    assert step.attn_tile_for([1024, 1024]) == step.ATTN_TILE
+    assert step.attn_tile_for([1024] + [8] * 40) == step.ATTN_TILE_FEW
