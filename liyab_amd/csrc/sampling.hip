@@ -325,7 +325,11 @@ __device__ __forceinline__ int block_count(int v, int* red) {
     return t;
 }
 
-template <int EPT, int THREADS>
+// PLAIN: no row asks for top-k or top-p (the caller's word): every logit is kept, and what serves
+// the cuts is not compiled in, which leaves the registers to the row (the full kernel spills some
+// of the 104 keys a thread holds at GPT-2's vocabulary, and every pass over them then waits for
+// scratch memory).
+template <int EPT, int THREADS, bool PLAIN>
 __global__ void __launch_bounds__(THREADS)
 sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t ld, int V,
                         const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -406,7 +410,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     const float lmax = key_value(kmax), inv_t = 1.4426950408889634f / T;  // exponentials are taken in base 2
     const int k = top_k != nullptr ? top_k[r] : 0;
     const float tp = top_p != nullptr ? top_p[r] : 1.0f;
-    const bool use_k = k > 0 && k < V, use_p = tp < 1.0f;
+    const bool use_k = !PLAIN && k > 0 && k < V, use_p = !PLAIN && tp < 1.0f;
     const unsigned long long lanes_below = (1ull << lane) - 1ull;
 
     // Which of this thread's ids are kept, as bits: key > t, or key == t and among the first
@@ -453,6 +457,10 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         }
     };
 
+    uint32_t bits[(EPT + 31) / 32];
+    // is id j of this thread kept? (PLAIN: every element of the row is)
+    auto is_kept = [&](int j) { return PLAIN ? keys[j] != 0u : ((bits[j / 32] >> (j % 32)) & 1u) != 0u; };
+    if constexpr (!PLAIN) {
     // ---- one wave among at most 64 candidates in cand_key / cand_id: nucleus cut and draw ----
     auto wave_finish = [&]() {
         const int n = n_cand;  // = k
@@ -609,7 +617,6 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         ties_k = k - block_count<WAVES>(c, redi);
     }
 
-    uint32_t bits[(EPT + 31) / 32];
     if (use_k && k <= kWaveCandidates) {
         // ---- few candidates (the pool overflowed): gathered, then one wave does the rest ----
         kept_bits(tau_k, ties_k, bits);
@@ -676,12 +683,14 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         ties = need < avail ? need : avail;
     }
 
+        kept_bits(tau, ties, bits);
+    }
+
     // ---- inverse CDF over ascending ids among the kept ----
-    kept_bits(tau, ties, bits);
     unsigned long long mine = 0;
 #pragma unroll
     for (int j = 0; j < EPT; ++j)
-        if (bits[j / 32] >> (j % 32) & 1u) mine += fixed_mass(again(keys[j]), lmax, inv_t);
+        if (is_kept(j)) mine += fixed_mass(again(keys[j]), lmax, inv_t);
     // the wave where the walk ends, from the waves' masses in order; then that wave alone walks
     // its ids in their order: group by group, a scan over the lanes' four ids each
     const unsigned long long wave_mass = wave_sum_u64(mine);
@@ -713,7 +722,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const int j = 4 * (g0 + b) + e;
-                            if (bits[j / 32] >> (j % 32) & 1u) tot[b] += fixed_mass(again(keys[j]), lmax, inv_t);
+                            if (is_kept(j)) tot[b] += fixed_mass(again(keys[j]), lmax, inv_t);
                         }
                     }
                 }
@@ -745,7 +754,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int j = 4 * g + e;
-                    q[e] = (bits[j / 32] >> (j % 32) & 1u) ? fixed_mass(again(keys[j]), lmax, inv_t) : 0ull;
+                    q[e] = is_kept(j) ? fixed_mass(again(keys[j]), lmax, inv_t) : 0ull;
                     q4 += q[e];
                 }
                 unsigned long long inc = q4;
@@ -862,8 +871,13 @@ extern "C" int liyab_sample(int* out, const float* logits, int64_t ld, int rows,
     LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d", rows, V);
     if (rows == 0) return 0;
     LIYAB_REQUIRE(scatter_index == nullptr || scatter_out != nullptr, "sample: a scatter index needs a target");
+    const bool plain = top_k == nullptr && top_p == nullptr;  // no row cuts its candidates
     // the row in registers where it fits; the general kernel beyond
-#define LIYAB_REGS(E, T) sample_registers_kernel<E, T><<<rows, T, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out)
+#define LIYAB_REGS(E, T)                                                                                                              \
+    do {                                                                                                                              \
+        if (plain) sample_registers_kernel<E, T, true><<<rows, T, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out); \
+        else sample_registers_kernel<E, T, false><<<rows, T, 0, stream>>>(out, logits, ld, V, temperature, top_k, top_p, uniform, scatter_index, scatter_out); \
+    } while (0)
     // (3 more ids than the row has: a row may start up to 3 entries past a multiple of 16 bytes)
     if (V + 3 <= 8 * 1024) LIYAB_REGS(8, 1024);
     else if (V + 3 <= 16 * 1024) LIYAB_REGS(16, 1024);

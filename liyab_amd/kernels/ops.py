@@ -316,21 +316,26 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, scatter=None) -> None:
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, uniform: torch.Tensor, scatter=None) -> None:
-    """Per-row sampling; temperature/top_p float32 [rows], top_k int32 [rows], uniform float64 [rows] in [0, 1)."""
+    """Per-row sampling; temperature/top_p float32 [rows], top_k int32 [rows], uniform float64 [rows] in [0, 1).
+    top_k and top_p may both be None when no row cuts its candidates: a shorter kernel runs then."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
     if logits.dtype != torch.float32:
         raise KernelError("sample: logits must be float32")
     _i32(out, "out", rows)
     _f32vec(temperature, "temperature", rows)
-    _f32vec(top_p, "top_p", rows)
-    _i32(top_k, "top_k", rows)
+    if (top_k is None) != (top_p is None):
+        raise KernelError("sample: top_k and top_p are given together or not at all")
+    if top_k is not None:
+        _f32vec(top_p, "top_p", rows)
+        _i32(top_k, "top_k", rows)
     _dev(uniform, "uniform")
     if uniform.dtype != torch.float64 or uniform.numel() != rows or not uniform.is_contiguous():
         raise KernelError("sample: uniform must be contiguous float64 [rows]")
     si, so = _scatter(scatter, rows)
     _lib.call("liyab_sample", out.data_ptr(), logits.data_ptr(), ld, rows, V, temperature.data_ptr(),
-              top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(), si, so, _stream())
+              0 if top_k is None else top_k.data_ptr(), 0 if top_p is None else top_p.data_ptr(),
+              uniform.data_ptr(), si, so, _stream())
 
 
 EPI_QKV_PAGED = 4

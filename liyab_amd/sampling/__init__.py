@@ -115,8 +115,9 @@ class Sampler:
             if self._events[i] is None:
                 self._events[i] = torch.cuda.Event()
             self._events[i].record()
-            ops.sample(out, logits, self._temp[:rows], self._topk[:rows], self._topp[:rows], self._u[:rows],
-                       scatter=scatter)
+            cuts = any(p.top_k > 0 or p.top_p < 1.0 for p in params)
+            ops.sample(out, logits, self._temp[:rows], self._topk[:rows] if cuts else None,
+                       self._topp[:rows] if cuts else None, self._u[:rows], scatter=scatter)
         return out
 
     def sample(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int]) -> List[int]:

@@ -604,6 +604,36 @@ def test_sampler_against_the_plain_sampler(ops, V):
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, params[r], got[r], want)
 
 
+@pytest.mark.parametrize("V", [1000, 50257, 70001])
+def test_sampler_without_cuts(ops, V):
+    """Temperature alone, called without top-k and top-p: the shorter kernel draws what the
+    plain sampler draws, also from a row of ties and beside a greedy row."""
+    import plain_gpt2 as plain
+
+    temps = [1.0, 0.8, 0.0, 1.7, 0.3, 1.0, 0.05]
+    logits = rnd(len(temps), V, scale=2.0, seed=13)
+    logits[5, :] = -1.5  # all equal
+    logits[3, 40:90] = 6.0
+    cpu = logits.cpu().numpy()
+    with pytest.raises(ops.KernelError):
+        ops.sample(torch.empty(len(temps), dtype=torch.int32, device=DEV), logits,
+                   torch.tensor(temps, dtype=torch.float32, device=DEV), None,
+                   torch.ones(len(temps), dtype=torch.float32, device=DEV),
+                   torch.zeros(len(temps), dtype=torch.float64, device=DEV))
+    for trial in range(8):
+        u = [plain.uniform(23 + trial, r) for r in range(len(temps))]
+        out = torch.empty(len(temps), dtype=torch.int32, device=DEV)
+        ops.sample(out, logits, torch.tensor(temps, dtype=torch.float32, device=DEV), None, None,
+                   torch.tensor(u, dtype=torch.float64, device=DEV))
+        got = out.tolist()
+        for r, T in enumerate(temps):
+            probs = plain.probabilities(cpu[r], T, 0, 1.0)
+            want = plain.sample(probs, u[r])
+            if got[r] != want:
+                cdf = np.cumsum(probs)
+                assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, T, got[r], want)
+
+
 @pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "auto"])
 @pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
