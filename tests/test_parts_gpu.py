@@ -1,6 +1,6 @@
 """Each part alone against its plain formula, and the generality of the layer plan: a toy
-mixer with state of its own, defined here, is registered, built and stepped without touching
-the framework's files; a layer reads another layer's cache; the run order names a layer twice
+mixer with state of its own, a feed-forward that routes and a position encoding without a
+table, defined here, are registered, built and stepped without touching the framework's files; a layer reads another layer's cache; the run order names a layer twice
 (needs the GPU)."""
 
 import math
@@ -468,6 +468,160 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
         tt.check_against_plain(got, reqs, ref, tol, f"toy {name} {dtype}")
         core.manager.check()
         assert all(core.manager.pages_in_use(g.index) == 0 for g in groups)
+
+
+# ---------------------------------------------------------------------------
+# more toy parts: a feed-forward with routing and a position encoding without a table
+# ---------------------------------------------------------------------------
+class RoutedSpec:
+    kind = "toy_routed"
+
+    def __init__(self, width, inner, n_experts, top, prefix):
+        self.width, self.inner, self.n_experts, self.top, self.prefix = width, inner, n_experts, top, prefix
+
+
+class RoutedFFN:
+    """Router logits h . Wr^T in float32; the `top` largest experts of a token (ties to the lower
+    index), a softmax over those; each expert an ungated tanh-GELU feed-forward without biases.
+    A test's toy in torch: the framework's files know nothing of routing."""
+
+    def __init__(self, spec, store, dtype):
+        from liyab_amd.config import TensorSource
+
+        self.top, self.dtype = spec.top, dtype
+        self.router = store.fetch(TensorSource(spec.prefix + ".router"), (spec.n_experts, spec.width), "matrix")
+        self.up = [store.fetch(TensorSource(f"{spec.prefix}.{e}.up"), (spec.inner, spec.width), "matrix") for e in range(spec.n_experts)]
+        self.down = [store.fetch(TensorSource(f"{spec.prefix}.{e}.down"), (spec.width, spec.inner), "matrix") for e in range(spec.n_experts)]
+
+    def forward(self, h, ctx, residual):
+        from liyab_amd.parts import as_tensor
+
+        h = as_tensor(h).float()
+        logits = h @ self.router.float().t()
+        top = torch.topk(logits, self.top, dim=1, sorted=True)  # equal logits do not occur with these weights
+        gates = torch.softmax(top.values, dim=1)
+        out = torch.zeros_like(h)
+        for e in range(len(self.up)):
+            rows, which = (top.indices == e).nonzero(as_tuple=True)
+            if rows.numel():
+                m = torch.nn.functional.gelu(h[rows] @ self.up[e].float().t(), approximate="tanh") @ self.down[e].float().t()
+                out.index_add_(0, rows, m * gates[rows, which].unsqueeze(1))
+        residual += out
+
+
+class SinusoidSpec:
+    kind = "toy_sinusoid"
+
+    def __init__(self, width, base):
+        self.width, self.base = width, base
+
+
+class SinusoidPositions:
+    """x[t, 2i] += sin(pos_t / base^(2i / d)), x[t, 2i + 1] += cos(the same): computed from the
+    positions of the step's tokens, no table and no limit to the context of its own."""
+
+    where = "residual"
+
+    def __init__(self, spec, store, dtype):
+        self.width, self.base = spec.width, spec.base
+
+    def fused_table(self):
+        return None  # nothing the embedding kernel could add in its pass
+
+    def add(self, ctx, x):
+        i = torch.arange(0, self.width, 2, device=x.device, dtype=torch.float64)
+        angle = ctx.positions.double().unsqueeze(1) / self.base ** (i / self.width)
+        x[:, 0::2] += angle.sin().to(x.dtype)
+        x[:, 1::2] += angle.cos().to(x.dtype)
+
+
+def routed_model(dtype):
+    """Layer 0: attention (3 heads of 16) + routed feed-forward (top 2 of 5 experts); layer 1:
+    attention on 1 key/value head + dense feed-forward. Positions by sinusoids."""
+    from liyab_amd.config import HeadSpec, LayerSpec, ModelPlan, OrderEntry, TokenEmbeddingSpec
+    from liyab_amd.parts import register_ffn, register_position
+
+    register_ffn("toy_routed", RoutedFFN)
+    register_position("toy_sinusoid", SinusoidPositions)
+    d, V, P, eps, E, F = 48, 157, 200, 1e-6, 5, 40
+    rng = np.random.default_rng(29)
+    layers = [
+        LayerSpec(attention_spec("a0", d, 3, 3, 16, 0.25), RoutedSpec(d, F, E, 2, "r0"), norm_spec("n0a", d, eps), norm_spec("n0b", d, eps)),
+        LayerSpec(attention_spec("a1", d, 2, 1, 32, 0.15), ffn_spec("f1", d, 72, "gelu_erf"), norm_spec("n1a", d, eps), norm_spec("n1b", d, eps)),
+    ]
+    tw = {"emb": rand(rng, V, d, scale=0.5), **norm_tensors(rng, "nf", d), "r0.router": rand(rng, E, d, scale=0.5),
+          **attention_tensors(rng, "a0", d, 3, 3, 16), **attention_tensors(rng, "a1", d, 2, 1, 32), **ffn_tensors(rng, "f1", d, 72)}
+    for e in range(E):
+        tw[f"r0.{e}.up"] = rand(rng, F, d, scale=0.2)
+        tw[f"r0.{e}.down"] = rand(rng, d, F, scale=0.2)
+    for name in ("n0a", "n0b", "n1a", "n1b"):
+        tw.update(norm_tensors(rng, name, d))
+    if dtype == "bfloat16":
+        tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tw.items()}
+    plan = ModelPlan(architecture="toy_routed", width=d, vocab_size=V, max_positions=P,
+                     embedding=TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": T("emb")}),
+                     residual_position=SinusoidSpec(d, 50.0), layers=layers, order=[OrderEntry(0), OrderEntry(1)],
+                     final_norm=norm_spec("nf", d, eps), head=HeadSpec("lm_head", d, V, 1.0, {"weight": T("emb")}))
+    return plan, tw, dict(d=d, V=V, eps=eps, E=E)
+
+
+def routed_plain(tw, info, ids):
+    d, eps, E = info["d"], info["eps"], info["E"]
+    pos = np.arange(len(ids), dtype=np.float64)[:, None]
+    angle = pos / 50.0 ** (np.arange(0, d, 2, dtype=np.float64) / d)
+    x = f64(tw["emb"])[ids].copy()
+    x[:, 0::2] += np.sin(angle)
+    x[:, 1::2] += np.cos(angle)
+    a, _ = plain_attention(plain_norm(x, tw, "n0a", eps), tw, "a0", 3, 3, 16, 0.25)
+    x = x + a
+    h = plain_norm(x, tw, "n0b", eps)
+    logits = h @ f64(tw["r0.router"]).T
+    out = np.zeros_like(h)
+    margins = []
+    for t in range(len(ids)):
+        order = np.argsort(-logits[t], kind="stable")
+        chosen = order[:2]
+        margins.append(logits[t, order[1]] - logits[t, order[2]])
+        g = np.exp(logits[t, chosen] - logits[t, chosen].max())
+        g /= g.sum()
+        for gate, e in zip(g, chosen):
+            out[t] += gate * (plain.gelu_tanh(h[t] @ f64(tw[f"r0.{e}.up"]).T) @ f64(tw[f"r0.{e}.down"]).T)
+    x = x + out
+    a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 2, 1, 32, 0.15)
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_erf")
+    return plain_norm(x, tw, "nf", eps) @ f64(tw["emb"]).T, np.array(margins)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_routing_and_computed_positions(dtype):
+    """A feed-forward that routes and a position encoding without a table, both defined here,
+    are registered, built and stepped beside the framework's attention, norms and dense
+    feed-forward, under every way of cutting the work."""
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = routed_model(dtype)
+    reqs = {f"r{i}": tt.random_tokens(40 + i, n, info["V"]) for i, n in enumerate([33, 150, 2, 77])}
+    ref, used = {}, set()
+    for rid, toks in reqs.items():
+        ref[rid], margins = routed_plain(tw, info, toks)
+        if dtype == "bfloat16":
+            # a token whose second and third experts are nearly tied may be routed otherwise in
+            # reduced precision: such a request is cut before that token
+            close = np.nonzero(margins < 0.05)[0]
+            if close.size:
+                reqs[rid] = toks[:max(2, int(close[0]))]
+                ref[rid] = ref[rid][:len(reqs[rid])]
+    assert sum(len(t) for t in reqs.values()) > 60
+    tol = TOL[dtype]
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=5))):
+        core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4,
+                                    use_graphs=False)
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, tol, f"routed toy {name} {dtype}")
+        core.manager.check()
+        assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
 
 class BareNorm:
