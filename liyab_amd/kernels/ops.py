@@ -514,6 +514,11 @@ def k_parts(M: int, N: int, K: int) -> int:
     return parts
 
 
+def skinny_parts_takes(M: int, N: int, K: int) -> bool:
+    """Whether `gemm_skinny_parts` takes this shape and is the kernel `gemm` would choose for it."""
+    return 0 < M <= 64 and K % 8 == 0 and N <= 8192 and not (M > 32 and K % 64 == 0 and N >= (2048 if M > 48 else 4097))
+
+
 def tiled_k_parts(M: int, N: int, K: int) -> int:
     """Into how many parts of K the tiled product of more than 32 rows is best cut when it is
     added to the residual stream (1: not at all). Several tiles of rows, few output features and

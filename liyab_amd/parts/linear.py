@@ -77,9 +77,14 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     if parts <= 1 and not in_splits and TILED_PARTS:
         parts = ops.tiled_k_parts(M, w.shape[0], K)  # one tile of 33 to 64 rows: the tiled kernel, cut over K
         tiled = parts > 1
-    if parts <= 1:
-        return None
     split = isinstance(stream, SplitStream)
+    if parts <= 1:
+        # not worth cutting; but a stream that arrives split is taken as it is by the streaming
+        # kernel's epilogue (one plane written: the sum of the stream's planes, the bias and the
+        # product), where settling it first would be a kernel of its own
+        if not (split and not in_splits and ops.skinny_parts_takes(M, w.shape[0], K)):
+            return None
+        parts = 1
     base = stream.planes if split else stream
     planes = ctx.workspace.get(name, (parts, M, w.shape[0]), torch.float32)
     if _overlap(planes, base):

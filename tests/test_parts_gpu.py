@@ -281,6 +281,42 @@ def test_product_of_a_tile_of_rows_deferred_through_the_tiled_kernel(parts, spli
     core.close("f")
 
 
+@pytest.mark.parametrize("rows,n_planes", [(40, 3), (64, 1), (7, 2)])
+def test_product_that_is_not_cut_takes_a_split_stream(parts, rows, n_planes, monkeypatch):
+    """A product of few rows that is not worth cutting over K, added to a stream that arrives
+    split: the streaming kernel adds the stream's planes in its epilogue and leaves one plane
+    (the stream's own tensor stays stale, no pass to settle it first); a whole stream is left to
+    the caller as before."""
+    from liyab_amd.engine import StepItem
+    from liyab_amd.kernels import ops
+    from liyab_amd.parts.base import SplitStream
+    from liyab_amd.parts.linear import linear_deferred
+
+    p, dtype = parts
+    if dtype != "bfloat16":
+        pytest.skip("only the bfloat16 products take planes")
+    monkeypatch.setattr(ops, "k_parts", lambda M, N, K: 1)
+    core = p.core
+    core.open("f")
+    ctx, _ = core.step_fn.prepare([StepItem("f", [1] * rows, [])])
+    rng = np.random.default_rng(6)
+    a = rand(rng, rows, 200).to(DEV).to(torch.bfloat16)
+    w = rand(rng, 88, 200, scale=0.1).to(DEV).to(torch.bfloat16)
+    bias = rand(rng, 88).to(DEV)
+    residual = rand(rng, rows, 88).to(DEV)
+    assert linear_deferred(a, w, bias, ctx, "uncut_test", residual) is None  # a whole stream: the caller's plain product
+    planes = torch.stack([rand(rng, rows, 88).to(DEV) for _ in range(n_planes)])
+    planes[0] += residual - planes.sum(dim=0)
+    home = torch.full_like(residual, float("nan"))
+    split = linear_deferred(a, w, bias, ctx, "uncut_test", SplitStream(planes, home))
+    assert isinstance(split, SplitStream) and split.planes.shape == (1, rows, 88) and split.home is home
+    assert torch.isnan(home).all()
+    want = f64(residual.cpu()) + f64(a.float().cpu()) @ f64(w.float().cpu()).T + f64(bias.cpu())
+    assert tt.rel_err(split.planes[0].cpu().numpy(), want) < 1e-5
+    assert tt.rel_err(split.settle().cpu().numpy(), want) < 1e-5
+    core.close("f")
+
+
 @pytest.mark.parametrize("geometry", [dict(H=5, Hkv=5, hd=16), dict(H=6, Hkv=2, hd=32, d=96), dict(H=3, Hkv=1, hd=48, d=64, window=13)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_mixer_alone(dtype, geometry):
