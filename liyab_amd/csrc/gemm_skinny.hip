@@ -341,5 +341,7 @@ extern "C" int liyab_gemm_skinny_parts(const void* a, int64_t lda, const void* w
     epi.out = parts;
     epi.ldo = N;
     epi.bias = bias;
-    return skinny_dispatch(a, lda, w, M, N, K, ksplit, 0, 1, epi, BaseSum{base, n_base, base_stride}, stream, kparts, part_stride);
+    // cut over K: 16 rows a workgroup (the parts cover the chip); whole: as the plain product chooses
+    return skinny_dispatch(a, lda, w, M, N, K, ksplit, 0, kparts > 1 ? 1 : 0, epi, BaseSum{base, n_base, base_stride}, stream, kparts,
+                           part_stride);
 }
