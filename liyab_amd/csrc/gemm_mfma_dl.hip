@@ -60,44 +60,55 @@ struct PartsParams {
 // 8 different pieces: the piece index is XORed with (row / 2) % 8.
 __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
-__global__ void __launch_bounds__(64 * WM * WN)
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1>
+__global__ void __launch_bounds__(64 * WM * WN * WK)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
                     EpiParams epi, int vec_ok, int page_shift, PartsParams parts) {
-    // WM x WN waves, each with (BM / WM) x (BN / WN) of the tile in blocks of 32 x 32
-    constexpr int WAVES = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int STAGE = (BM + BN) * DBK;      // elements per stage: the tile of a, then the tile of w
-    constexpr int A_LOADS = BM / 8 / WAVES, W_LOADS = BN / 8 / WAVES;  // wave-loads (8 rows each) per wave and stage
+    // WK groups of WM x WN waves, each wave with (BM / WM) x (BN / WN) of the tile in blocks of 32 x 32.
+    // A stage holds WK consecutive units of 64 k, one a group: the groups walk K side by side (a
+    // tile of few rows has few products a unit, and its walk is a chain of waits: load, barrier,
+    // fragments, products; WK of them run at once), and their sums are added at the end in the
+    // groups' order.
+    constexpr int GROUP = WM * WN, WAVES = GROUP * WK, TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int UNIT = (BM + BN) * DBK;       // elements of one unit of 64 k: the tile of a, then the tile of w
+    constexpr int STAGE = WK * UNIT;            // elements per stage
+    constexpr int A_LOADS = BM / 8 / GROUP, W_LOADS = BN / 8 / GROUP;  // wave-loads (8 rows each) per wave and stage
     static_assert(TM >= 1 && TN >= 1 && A_LOADS >= 1 && W_LOADS >= 1, "tile too small for its waves");
     extern __shared__ __attribute__((aligned(1024))) bf16_t lds[];
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int wm = wave / WN, wn = wave % WN;
+    const int wk = wave / GROUP, wg = wave % GROUP;
+    const int wm = wg / WN, wn = wg % WN;
     // Workgroups go to the 8 XCDs round-robin, each XCD with an L2 of its own. Tile t of the
     // row-major tile order goes to the XCD that holds the tiles around it, so that an XCD's
     // tiles share a few row blocks of `a` and its L2 holds them beside all of `w`.
     const int tiles_n = (N + BN - 1) / BN, n_tiles = tiles_n * ((M + BM - 1) / BM);
     const int xcd = blockIdx.x % 8, base = n_tiles / 8, rem = n_tiles % 8;
     const int tile_id = xcd * base + min(xcd, rem) + blockIdx.x / 8;
-    const int m0 = (tile_id / tiles_n) * BM, n0 = (tile_id % tiles_n) * BN;
+    int m0 = (tile_id / tiles_n) * BM;
+    const int n0 = (tile_id % tiles_n) * BN;
     const int li = lane % 32, g = lane / 32;
 
     // this lane's part in a wave-load: row lane / 8 of the 8, LDS piece position lane % 8
     const int lrow = lane / 8, lpos = lane % 8;
+    // a group's waves load their group's unit of the stage; a unit past the end of K is the last
+    // one again (loaded and not multiplied: every wave asks for as many loads a stage as the
+    // waits below count on)
+    int units = K / DBK;  // units of 64 k this workgroup walks
     auto issue = [&](int kt, int stage) {
-        const int k0 = kt * DBK;
-        bf16_t* sa = lds + stage * STAGE;
+        const int k0 = min(kt * WK + wk, units - 1) * DBK;
+        bf16_t* sa = lds + stage * STAGE + wk * UNIT;
         bf16_t* sw = sa + BM * DBK;
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) {
-            const int r0 = (wave * A_LOADS + i) * 8, row = r0 + lrow;
+            const int r0 = (wg * A_LOADS + i) * 8, row = r0 + lrow;
             const int c = lpos ^ swizzle(row);
             const bf16_t* src = a + static_cast<int64_t>(min(m0 + row, M - 1)) * lda + k0 + c * 8;
             __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sa + r0 * DBK), 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) {
-            const int r0 = (wave * W_LOADS + i) * 8, row = r0 + lrow;
+            const int r0 = (wg * W_LOADS + i) * 8, row = r0 + lrow;
             const int c = lpos ^ swizzle(row);
             const bf16_t* src = w + static_cast<int64_t>(min(n0 + row, N - 1)) * K + k0 + c * 8;
             __builtin_amdgcn_global_load_lds(src, (lds_void_ptr)(sw + r0 * DBK), 16, 0, 0);
@@ -112,15 +123,15 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    int nk = K / DBK;
     if constexpr (EPI == kEpiParts) {
-        // this workgroup's part of K: tiles [kt0, kt0 + nk)
+        // this workgroup's part of K: units [kt0, kt0 + units)
         const int kt0 = blockIdx.y * parts.kt_per_part;
-        nk = min(nk - kt0, parts.kt_per_part);
+        units = min(units - kt0, parts.kt_per_part);
         a += static_cast<int64_t>(kt0) * DBK;
         w += static_cast<int64_t>(kt0) * DBK;
         if (blockIdx.y > 0) epi.bias = nullptr;  // the bias goes to the first plane only
     }
+    const int nk = (units + WK - 1) / WK;  // stages walked
     constexpr int AHEAD = DSTAGES - 1;  // tiles of K in flight or in use beside the one being multiplied
 #pragma unroll
     for (int p = 0; p < AHEAD; ++p)
@@ -129,7 +140,13 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         // tile kt must have landed: the loads of the tiles after it may still be in flight (a
         // wave's loads complete in order, A_LOADS + W_LOADS a tile)
         const int later = min(nk - 1 - kt, AHEAD - 1);
-        if (later >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (A_LOADS + W_LOADS)) : "memory");
+        constexpr int PER_TILE = A_LOADS + W_LOADS;
+        static_assert((AHEAD - 1) * PER_TILE <= 63, "the counter of loads in flight has six bits");
+        if (later >= 7) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD > 7 ? 7 * PER_TILE : 0) : "memory");
+        else if (later == 6) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD > 6 ? 6 * PER_TILE : 0) : "memory");
+        else if (later == 5) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD > 5 ? 5 * PER_TILE : 0) : "memory");
+        else if (later == 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD > 4 ? 4 * PER_TILE : 0) : "memory");
+        else if (later == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD > 3 ? 3 * PER_TILE : 0) : "memory");
         else if (later == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (A_LOADS + W_LOADS)) : "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(A_LOADS + W_LOADS) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -137,8 +154,9 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         // barrier: __syncthreads() would also wait for the loads still meant to be in flight.
         __builtin_amdgcn_s_barrier();
         if (kt + AHEAD < nk) issue(kt + AHEAD, (kt + AHEAD) % DSTAGES);  // into the stage tile kt - 1 used
-        const bf16_t* sa = lds + (kt % DSTAGES) * STAGE;
+        const bf16_t* sa = lds + (kt % DSTAGES) * STAGE + wk * UNIT;
         const bf16_t* sw = sa + BM * DBK;
+        if (WK > 1 && kt * WK + wk >= units) continue;  // this group's unit is past the end of K (the last stage only)
         // fragments of slab ks + 1 are read from LDS while slab ks multiplies
         bf16x8 fa[2][TM], fw[2][TN];
         auto read_frags = [&](int ks, int buf) {
@@ -163,6 +181,38 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0);
+        }
+    }
+    if constexpr (WK > 1) {
+        // the groups' sums, added in the groups' order by the first group, which alone stores:
+        // the others go through the epilogue as a tile below the last row
+        constexpr int PER_WAVE = TM * TN * 16 * 64;
+        static_assert((WK - 1) * GROUP * PER_WAVE * 4 <= DSTAGES * STAGE * 2, "the groups' sums must fit the operand stages");
+        float* red = reinterpret_cast<float*>(lds);
+        __syncthreads();  // everyone is done reading the last operand stage
+        if (wk > 0) {
+            float* mine = red + ((wk - 1) * GROUP + wg) * PER_WAVE + lane;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mine[((i * TN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (wk == 0) {
+#pragma unroll
+            for (int q = 1; q < WK; ++q) {
+                const float* theirs = red + ((q - 1) * GROUP + wg) * PER_WAVE + lane;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] += theirs[((i * TN + j) * 16 + r) * 64];
+            }
+        } else {
+            m0 = M;
         }
     }
     // The products were taken transposed (w's fragment as the first operand), so a lane holds one
@@ -335,11 +385,11 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     }
 }
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2>
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1>
 int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     const int grid = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
-    const size_t smem = static_cast<size_t>(DSTAGES) * (BM + BN) * DBK * sizeof(bf16_t);
-    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN>;
+    const size_t smem = static_cast<size_t>(DSTAGES) * WK * (BM + BN) * DBK * sizeof(bf16_t);
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN, WK>;
     static bool ready = false;  // once per instantiation, outside any stream capture's first use
     if (!ready) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
@@ -363,18 +413,18 @@ int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, in
     bool vec16 = vec && sizeof(OutT) == 2 && N % 8 == 0;
     if (EPI == kEpiQkvPaged) vec16 = vec16 && epi.ldo % 8 == 0 && epi.hd % 8 == 0 && epi.q_dim % 8 == 0;
     else if (EPI != kEpiResidual) vec16 = vec16 && epi.ldo % 8 == 0;
-    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec16 ? 2 : (vec ? 1 : 0), page_shift, PartsParams{});
+    kern<<<grid, 64 * WM * WN * WK, smem, stream>>>(a, lda, w, M, N, K, epi, vec16 ? 2 : (vec ? 1 : 0), page_shift, PartsParams{});
     return check_launch("gemm_mfma_dl");
 }
 
 // The product cut over K into `kparts` parts (see the head of this file); epi carries the planes
 // (out, float32, rows of N) and the first plane's bias.
-template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2>
+template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2, int WK = 1>
 int launch_dl_parts(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, int kparts, const EpiParams& epi,
                     const PartsParams& parts, hipStream_t stream) {
     const dim3 grid(((N + BN - 1) / BN) * ((M + BM - 1) / BM), kparts);
-    const size_t smem = static_cast<size_t>(DSTAGES) * (BM + BN) * DBK * sizeof(bf16_t);
-    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, float, kEpiParts, WM, WN>;
+    const size_t smem = static_cast<size_t>(DSTAGES) * WK * (BM + BN) * DBK * sizeof(bf16_t);
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, float, kEpiParts, WM, WN, WK>;
     static bool ready = false;
     if (!ready) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
@@ -382,25 +432,25 @@ int launch_dl_parts(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N,
     }
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     const bool vec = N % 4 == 0 && al16(epi.bias) && al16(epi.out) && al16(parts.base) && parts.part_stride % 4 == 0 && parts.base_stride % 4 == 0;
-    kern<<<grid, 64 * WM * WN, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, -1, parts);
+    kern<<<grid, 64 * WM * WN * WK, smem, stream>>>(a, lda, w, M, N, K, epi, vec ? 1 : 0, -1, parts);
     return check_launch("gemm_mfma_dl_parts");
 }
 
-template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2>
+template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2, int WK = 1>
 int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
-    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
     if (epi.out_dtype == kF32) {
-        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
-        return launch_dl_as<BM, BN, DSTAGES, float, -1, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        return launch_dl_as<BM, BN, DSTAGES, float, -1, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
     }
     switch (epi.mode) {
-        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
-        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1, WM, WN>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
     }
 }
 
@@ -409,7 +459,10 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
 using namespace liyab;
 
 // tile: 2 = 64x64 tiles, three stages deep, on four waves; 6 = the same with four stages; 8 = 128x128, two
-// stages, on eight waves; 16 = 64x32, four stages, on two waves (for one tile of rows); 0 = chosen from
+// stages, on eight waves; 16 = 64x32 on four groups of two waves that walk K side by side, three stages of
+// four units (for one tile of rows: 8.2 us for 64 x 4,800 x 1,600 where two waves walking K alone, four
+// stages deep, took 10.3; deeper rings for those took longer, 11.1 with eight stages: the walk waits on
+// its own chain of load, barrier, fragments and products, not on the loads in flight); 0 = chosen from
 // the shape. (Measured and dropped: 128x128 on four waves, 128x64, 128x192, and deeper rings under
 // 128x128, whose LDS leaves one workgroup a compute unit, so that 288 tiles take two rounds.)
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
@@ -431,7 +484,7 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
-        case 16: return launch_dl<64, 32, 4, 2, 1>(a, lda, w, M, N, K, epi, stream);
+        case 16: return launch_dl<64, 32, 3, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }
@@ -472,6 +525,6 @@ extern "C" int liyab_gemm_mfma_dl_parts(const void* a, int64_t lda, const void* 
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
     if (tile == 6) return launch_dl_parts<64, 64, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
-    if (tile == 16) return launch_dl_parts<64, 32, 4, 2, 1>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
+    if (tile == 16) return launch_dl_parts<64, 32, 3, 2, 1, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
     return fail(1, "gemm_mfma_dl_parts: unknown tile %d (6 or 16)", tile);
 }

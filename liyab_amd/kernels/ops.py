@@ -516,7 +516,7 @@ def k_parts(M: int, N: int, K: int) -> int:
 
 def skinny_parts_takes(M: int, N: int, K: int) -> bool:
     """Whether `gemm_skinny_parts` takes this shape and is the kernel `gemm` would choose for it."""
-    return 0 < M <= 64 and K % 8 == 0 and N <= 8192 and not (M > 32 and K % 64 == 0 and N >= (2048 if M > 48 else 4097))
+    return 0 < M <= 64 and K % 8 == 0 and N <= 8192 and not (M > 32 and K % 64 == 0 and N >= 2048)
 
 
 def tiled_k_parts(M: int, N: int, K: int) -> int:
@@ -624,10 +624,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             # a vocabulary's worth of output features: large tiles re-read the tokens least
             # (16 rows: 22.5 against 25.1 us for 768 -> 50,257; 64 rows: 27.9 against 32.9)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=8)
-        elif M > 32 and M <= 64 and a.shape[1] % 64 == 0 and N >= (2048 if M > 48 else 4097):
-            # one tile of 64 rows and many output features: 64 x 32 tiles share the tokens' rows
-            # through LDS where the streaming kernel's workgroups each read them again (64 rows:
-            # 6.2 against 7.6 us for 768 -> 2,304, 10.3 against 18.3 for 1,600 -> 4,800)
+        elif M > 32 and M <= 64 and a.shape[1] % 64 == 0 and N >= 2048:
+            # one tile of 33 to 64 rows and many output features: 64 x 32 tiles share the tokens'
+            # rows through LDS where the streaming kernel's workgroups each read them again (40
+            # rows: 5.2 against 6.4 us for 768 -> 2,304, 8.0 against 10.4 for 1,600 -> 4,800; the
+            # products back to the model's width, with fewer tiles, stay with the streaming kernel)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=16)
         elif M <= 16 or (M <= 64 and N <= 8192):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled

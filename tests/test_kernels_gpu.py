@@ -634,7 +634,7 @@ def test_sampler_without_cuts(ops, V):
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, T, got[r], want)
 
 
-@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "auto"])
+@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "dl16", "auto"])
 @pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
     """Queries to a dense buffer, keys and values straight into shuffled cache slots, against
