@@ -526,13 +526,13 @@ def tiled_k_parts(M: int, N: int, K: int) -> int:
     24 tiles of 64 x 64, each walking the whole of K in 18.7 us): cut until the tiles cover the
     chip. One tile of rows (33 to 64): the 64 x 32 tiles are few and each walks the whole of K;
     cut over K they cover the chip: alone, at 64 rows, 3,072 -> 768 takes 8.2 us whole (the streaming kernel) and 4.9 in 8 parts, 6,400 ->
-    1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: only the
-    longest inner dimensions gain, in 4 parts (us a step of 12 layers at 64 rows, whole and
-    cut: GPT-2 XL's sizes 1360 and 1300; medium's 929 and 951, small's 799 and 828: not there)."""
+    1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: inner
+    dimensions from 3,072 gain, in 4 parts (ms a step at 64 rows, whole and cut: GPT-2 small's
+    sizes 0.806 and 0.797, medium's 1.767 and 1.715; XL's 5.19 and 4.90)."""
     if K % 64 != 0 or M <= 32:
         return 1
     if M <= 64:
-        return 4 if K >= 6144 and N <= 2048 else 1
+        return 4 if K >= 3072 and N <= 2048 else 1
     # several tiles of rows (a prompt's portion): 64 x 64 tiles, cut until they cover the chip,
     # a part keeping 256 of K or more
     tiles = (M + 63) // 64 * ((N + 63) // 64)
