@@ -624,13 +624,17 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             # a vocabulary's worth of output features: large tiles re-read the tokens least
             # (16 rows: 22.5 against 25.1 us for 768 -> 50,257; 64 rows: 27.9 against 32.9)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=8)
-        elif (M > 32 or (M > 16 and N * a.shape[1] >= 6 << 20)) and M <= 64 and a.shape[1] % 64 == 0 and N >= 2048:
+        elif ((M > 32 or (M > 16 and N * a.shape[1] >= 6 << 20)) and a.shape[1] % 64 == 0 and N >= 2048
+              and (M + 63) // 64 * ((N + 31) // 32) <= compute_units()):
             # one tile of 33 to 64 rows and many output features: 64 x 32 tiles share the tokens'
             # rows through LDS where the streaming kernel's workgroups each read them again (40
             # rows: 5.2 against 6.4 us for 768 -> 2,304, 8.0 against 10.4 for 1,600 -> 4,800; the
             # products back to the model's width, with fewer tiles, stay with the streaming kernel);
             # the largest matrices already from 17 rows (32 rows, weights cold from HBM: 8.9
-            # against 12.5 us for 1,600 -> 4,800, but 6.6 against 6.1 for 1,024 -> 3,072)
+            # against 12.5 us for 1,600 -> 4,800, but 6.6 against 6.1 for 1,024 -> 3,072); more
+            # tiles of rows as long as every tile has a compute unit of its own (the stages fill
+            # a unit's LDS; 128 rows: 6.1 against 7.7 us for 768 -> 2,304 in 64 x 64 tiles; with
+            # more tiles than units, 400 rows: 10.7 against 8.0)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=16)
         elif M <= 16 or (M <= 64 and N <= 8192):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
