@@ -57,15 +57,32 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
 }
 
+// Sums and maxima over the 64 lanes of a wave, the same bits in every lane. Within a row of 16
+// lanes the partners come through the lanes' own data path (DPP: neighbours in a quad, the other
+// pair of the quad, the other quad of eight, the other eight of the row: a few cycles each);
+// the four rows' results are then read as scalars and combined. An exchange through the LDS
+// crossbar (__shfl_xor) takes about a hundred cycles to come back, six of them in a row a
+// reduction: a norm's two sums were a microsecond of its kernel.
+template <int CTRL>
+__device__ __forceinline__ float lanes_dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_of(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    v += lanes_dpp<0xB1>(v);   // quad_perm [1, 0, 3, 2]: lane ^ 1
+    v += lanes_dpp<0x4E>(v);   // quad_perm [2, 3, 0, 1]: lane ^ 2
+    v += lanes_dpp<0x141>(v);  // row_half_mirror: the other quad of eight (every lane of a quad holds the same)
+    v += lanes_dpp<0x140>(v);  // row_mirror: the other eight of the row
+    return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    v = fmaxf(v, lanes_dpp<0xB1>(v));
+    v = fmaxf(v, lanes_dpp<0x4E>(v));
+    v = fmaxf(v, lanes_dpp<0x141>(v));
+    v = fmaxf(v, lanes_dpp<0x140>(v));
+    return fmaxf(fmaxf(lane_of(v, 0), lane_of(v, 16)), fmaxf(lane_of(v, 32), lane_of(v, 48)));
 }
 
 }  // namespace liyab
