@@ -6,6 +6,7 @@
 // No launcher allocates device memory: callers pass outputs and workspaces.
 #pragma once
 
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -76,6 +77,43 @@ __device__ __forceinline__ float wave_sum(float v) {
     v += lanes_dpp<0x141>(v);  // row_half_mirror: the other quad of eight (every lane of a quad holds the same)
     v += lanes_dpp<0x140>(v);  // row_mirror: the other eight of the row
     return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
+}
+// The largest value of the wave and the lowest index that holds it (every lane gets both):
+// the same steps, a pair at a time. KeyT is float or uint32_t.
+template <typename KeyT>
+__device__ __forceinline__ void wave_argmax(KeyT& bv, int& bi) {
+    auto take = [&](KeyT ov, int oi) {
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    };
+    auto step = [&](auto ctrl) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        uint32_t bits;
+        __builtin_memcpy(&bits, &bv, 4);
+        const uint32_t ob = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(bits), CTRL, 0xf, 0xf, false));
+        const int oi = __builtin_amdgcn_update_dpp(0, bi, CTRL, 0xf, 0xf, false);
+        KeyT ov;
+        __builtin_memcpy(&ov, &ob, 4);
+        take(ov, oi);
+    };
+    step(std::integral_constant<int, 0xB1>{});
+    step(std::integral_constant<int, 0x4E>{});
+    step(std::integral_constant<int, 0x141>{});
+    step(std::integral_constant<int, 0x140>{});
+    // the four rows' pairs, read as scalars
+    uint32_t bits;
+    __builtin_memcpy(&bits, &bv, 4);
+    KeyT rv[4];
+    int ri[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t b = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(bits), 16 * q));
+        __builtin_memcpy(&rv[q], &b, 4);
+        ri[q] = __builtin_amdgcn_readlane(bi, 16 * q);
+    }
+    bv = rv[0];
+    bi = ri[0];
+#pragma unroll
+    for (int q = 1; q < 4; ++q) take(rv[q], ri[q]);
 }
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, lanes_dpp<0xB1>(v));

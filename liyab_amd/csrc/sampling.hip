@@ -71,12 +71,7 @@ __device__ __forceinline__ void block_argmax(const float* row, int V, float& bes
         const float v = row[i];
         if (v > bv) { bv = v; bi = i; }  // strict: an equal later id does not replace
     }
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, kWave);
-        const int oi = __shfl_xor(bi, off, kWave);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    wave_argmax(bv, bi);
     __syncthreads();
     if (threadIdx.x % kWave == 0) { redv[threadIdx.x / kWave] = bv; redi[threadIdx.x / kWave] = bi; }
     __syncthreads();
@@ -292,13 +287,18 @@ __device__ __forceinline__ unsigned long long lane_value64(unsigned long long v,
     return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), off, kWave);
-        const uint32_t hi = __shfl_xor(static_cast<uint32_t>(v >> 32), off, kWave);
+    // within rows of 16 lanes through DPP, the rows' sums as scalars (integer sums: any order gives the same)
+    auto step = [&](auto ctrl) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(v)), CTRL, 0xf, 0xf, false));
+        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(v >> 32)), CTRL, 0xf, 0xf, false));
         v += (static_cast<unsigned long long>(hi) << 32) | lo;
-    }
-    return v;
+    };
+    step(std::integral_constant<int, 0xB1>{});
+    step(std::integral_constant<int, 0x4E>{});
+    step(std::integral_constant<int, 0x141>{});
+    step(std::integral_constant<int, 0x140>{});
+    return (lane_value64(v, 0) + lane_value64(v, 16)) + (lane_value64(v, 32) + lane_value64(v, 48));
 }
 
 // Sums over a workgroup of WAVES waves, exact; every thread gets the result. `red`: WAVES values.
@@ -385,12 +385,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     for (int j = 0; j < EPT; ++j)
         if (keys[j] > kmax) { kmax = keys[j]; imax = id_of(j); }
     thread_max[tid] = kmax;
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const uint32_t ok = __shfl_xor(kmax, off, kWave);
-        const int oi = __shfl_xor(imax, off, kWave);
-        if (ok > kmax || (ok == kmax && oi < imax)) { kmax = ok; imax = oi; }
-    }
+    wave_argmax(kmax, imax);
     if (lane == 0) { redk[wave] = kmax; redi[wave] = imax; }
     if (tid == 0) { result = -1; n_cand = 0; n_pool = 0; }
     __syncthreads();
@@ -808,12 +803,7 @@ argmax_partial_kernel(float* __restrict__ pv, int* __restrict__ pi, const float*
         const float v = row[i];
         if (v > bv) { bv = v; bi = i; }
     }
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, kWave);
-        const int oi = __shfl_xor(bi, off, kWave);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    wave_argmax(bv, bi);
     if (threadIdx.x % kWave == 0) { redv[threadIdx.x / kWave] = bv; redi[threadIdx.x / kWave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -830,12 +820,7 @@ argmax_final_kernel(int* __restrict__ out, const float* __restrict__ pv, const i
     const int r = blockIdx.x;
     float bv = pv[r * AM_CHUNKS + threadIdx.x];
     int bi = pi[r * AM_CHUNKS + threadIdx.x];
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, kWave);
-        const int oi = __shfl_xor(bi, off, kWave);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    wave_argmax(bv, bi);
     if (threadIdx.x == 0) {
         const int token = bi == 0x7fffffff ? 0 : bi;
         out[r] = token;
