@@ -115,8 +115,7 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
             float d = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) d = fmaf(kf[e], qf[e], d);
-#pragma unroll
-            for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, 64);
+            d = group_sum<LPK>(d);  // over the lanes that share the key
             s[u] = valid[u] ? d * scale : -INFINITY;
             m_new = fmaxf(m_new, s[u]);
         }

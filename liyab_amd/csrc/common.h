@@ -71,6 +71,18 @@ __device__ __forceinline__ float lanes_dpp(float v) {
 __device__ __forceinline__ float lane_of(float v, int lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
+// The sum over each group of LANES consecutive lanes (a power of two up to 32), in every lane of
+// the group; the partners' order is that of v += lane ^ 1, ^ 2, ^ 4, ^ 8.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(LANES == 1 || LANES == 2 || LANES == 4 || LANES == 8 || LANES == 16 || LANES == 32, "a power of two up to 32");
+    if constexpr (LANES > 1) v += lanes_dpp<0xB1>(v);
+    if constexpr (LANES > 2) v += lanes_dpp<0x4E>(v);
+    if constexpr (LANES > 4) v += lanes_dpp<0x141>(v);
+    if constexpr (LANES > 8) v += lanes_dpp<0x140>(v);
+    if constexpr (LANES > 16) v += __shfl_xor(v, 16, kWave);  // the next row of 16: no path but the crossbar
+    return v;
+}
 __device__ __forceinline__ float wave_sum(float v) {
     v += lanes_dpp<0xB1>(v);   // quad_perm [1, 0, 3, 2]: lane ^ 1
     v += lanes_dpp<0x4E>(v);   // quad_perm [2, 3, 0, 1]: lane ^ 2
