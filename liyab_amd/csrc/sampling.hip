@@ -16,6 +16,9 @@
 // draws the same tokens alone or in any batch. One workgroup per row; every
 // count and sum is reduced in a fixed order.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 namespace liyab {
 
@@ -844,6 +847,57 @@ extern "C" int liyab_argmax(int* out, const float* logits, int64_t ld, int rows,
     argmax_partial_kernel<<<dim3(rows, AM_CHUNKS), 256, 0, stream>>>(scratch_v, scratch_i, logits, ld, V);
     if (int rc = check_launch("argmax_partial")) return rc;
     argmax_final_kernel<<<rows, 64, 0, stream>>>(out, scratch_v, scratch_i, scatter_index, scatter_out);
+    return check_launch("argmax_final");
+}
+
+// The scratch of liyab_argmax_static: 64 values, then 64 ids, for each of up to
+// LIYAB_ARGMAX_STATIC_MAX_ROWS rows. In host code this name is a stand-in for the symbol, not a
+// device address: the address is asked for once a device (each GPU holds its own copy) and only
+// that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[LIYAB_ARGMAX_STATIC_MAX_ROWS * AM_CHUNKS * (sizeof(float) + sizeof(int))];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};  // the array's address on each device, once looked up
+
+// The array's address on the current device (nullptr after fail(...)).
+void* scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { fail(2, "argmax_static: hipGetDevice: %s", hipGetErrorString(e)); return nullptr; }
+    if (dev < 0 || dev >= kMaxDevices) { fail(1, "argmax_static: device %d is beyond the %d this library keeps track of", dev, kMaxDevices); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            fail(2, "argmax_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int liyab_argmax_static_init(void) { return scratch_of_current_device() != nullptr ? 0 : 2; }
+
+extern "C" int liyab_argmax_static(int* out, const float* logits, int64_t ld, int rows, int V, const int* scatter_index,
+                                   int* scatter_out, hipStream_t stream) {
+    LIYAB_REQUIRE(out && logits, "argmax_static: null pointer");
+    LIYAB_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax_static: bad sizes rows=%d V=%d", rows, V);
+    LIYAB_REQUIRE(rows <= LIYAB_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows; the library's own scratch holds %d (use liyab_argmax with a workspace beyond)",
+                  rows, LIYAB_ARGMAX_STATIC_MAX_ROWS);
+    LIYAB_REQUIRE(scatter_index == nullptr || scatter_out != nullptr, "argmax_static: a scatter index needs a target");
+    if (rows == 0) return 0;
+    void* ptr = scratch_of_current_device();
+    if (ptr == nullptr) return 2;
+    float* pv = static_cast<float*>(ptr);
+    int* pi = reinterpret_cast<int*>(pv + static_cast<size_t>(LIYAB_ARGMAX_STATIC_MAX_ROWS) * AM_CHUNKS);
+    argmax_partial_kernel<<<dim3(rows, AM_CHUNKS), 256, 0, stream>>>(pv, pi, logits, ld, V);
+    if (int rc = check_launch("argmax_partial")) return rc;
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(out, pv, pi, scatter_index, scatter_out);
     return check_launch("argmax_final");
 }
 

@@ -58,6 +58,8 @@ _SIGNATURES = {
     "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
+    "liyab_argmax_static_init": [],
+    "liyab_argmax_static": [P, P, c_int64, c_int, c_int, P, P, P],
     "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P, P, P],
 }
 
