@@ -29,7 +29,7 @@ def _ids(text: str):
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="liyab-cli", description="Generate tokens with a GPT-2 model folder on one MI355X.")
+    ap = argparse.ArgumentParser(prog="liyab-cli", description="Generate tokens with a model folder (config.json + model.safetensors) on one MI355X.")
     ap.add_argument("-m", "--model", help="model folder (config.json + model.safetensors)")
     ap.add_argument("-p", "--prompt", "--prompt-ids", dest="prompt", help="prompt as token ids, e.g. 5,17,3")
     ap.add_argument("--prompt-file", help="file holding the prompt's token ids")

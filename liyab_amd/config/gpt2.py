@@ -22,6 +22,7 @@ from .plan import (
     AttentionSpec,
     DenseFFNSpec,
     HeadSpec,
+    Init,
     LayerSpec,
     ModelPlan,
     NormSpec,
@@ -157,6 +158,13 @@ class GPT2Config:
     def plan(self) -> ModelPlan:
         d, F, V = self.n_embd, self.n_inner, self.vocab_size
         eps = self.layer_norm_epsilon
+        # What the random-weights mode draws: embeddings and the products into a layer N(0, 0.02), the
+        # two products back to the stream N(0, 0.02 / sqrt(2 n_layer)), biases N(0, 0.02), norm weights
+        # 1 + N(0, 0.05) and norm biases N(0, 0.02). Norm weights away from 1 and biases away from 0
+        # make a norm or a bias applied in the wrong place visible (tools/reference_trace.py:424-437
+        # argues the same for its own random checkpoints).
+        wide, bias = Init(0.02), Init(0.02)
+        back = Init(0.02 / math.sqrt(2.0 * self.n_layer))
 
         def norm(prefix: str) -> NormSpec:
             return NormSpec(
@@ -164,8 +172,8 @@ class GPT2Config:
                 width=d,
                 eps=eps,
                 tensors={
-                    "weight": TensorSource(prefix + ".weight"),
-                    "bias": TensorSource(prefix + ".bias"),
+                    "weight": TensorSource(prefix + ".weight", init=Init(0.05, 1.0)),
+                    "bias": TensorSource(prefix + ".bias", init=bias),
                 },
             )
 
@@ -181,10 +189,10 @@ class GPT2Config:
                 scale=self.attention_scale(i),
                 window=0,
                 tensors={
-                    "qkv_weight": TensorSource(p + ".attn.c_attn.weight", layout="in_out"),
-                    "qkv_bias": TensorSource(p + ".attn.c_attn.bias"),
-                    "out_weight": TensorSource(p + ".attn.c_proj.weight", layout="in_out"),
-                    "out_bias": TensorSource(p + ".attn.c_proj.bias"),
+                    "qkv_weight": TensorSource(p + ".attn.c_attn.weight", layout="in_out", init=wide),
+                    "qkv_bias": TensorSource(p + ".attn.c_attn.bias", init=bias),
+                    "out_weight": TensorSource(p + ".attn.c_proj.weight", layout="in_out", init=back),
+                    "out_bias": TensorSource(p + ".attn.c_proj.bias", init=bias),
                 },
             )
             ffn = DenseFFNSpec(
@@ -193,10 +201,10 @@ class GPT2Config:
                 inner=F,
                 activation=_ACTIVATIONS[self.activation_function],
                 tensors={
-                    "up_weight": TensorSource(p + ".mlp.c_fc.weight", layout="in_out"),
-                    "up_bias": TensorSource(p + ".mlp.c_fc.bias"),
-                    "down_weight": TensorSource(p + ".mlp.c_proj.weight", layout="in_out"),
-                    "down_bias": TensorSource(p + ".mlp.c_proj.bias"),
+                    "up_weight": TensorSource(p + ".mlp.c_fc.weight", layout="in_out", init=wide),
+                    "up_bias": TensorSource(p + ".mlp.c_fc.bias", init=bias),
+                    "down_weight": TensorSource(p + ".mlp.c_proj.weight", layout="in_out", init=back),
+                    "down_bias": TensorSource(p + ".mlp.c_proj.bias", init=bias),
                 },
             )
             layers.append(
@@ -216,14 +224,14 @@ class GPT2Config:
                 vocab_size=V,
                 width=d,
                 scale=1.0,
-                tensors={"table": TensorSource("wte.weight")},
+                tensors={"table": TensorSource("wte.weight", init=wide)},
             ),
             residual_position=PositionSpec(
                 kind="learned_positions",
                 where="residual",
                 max_positions=self.n_positions,
                 width=d,
-                tensors={"table": TensorSource("wpe.weight")},
+                tensors={"table": TensorSource("wpe.weight", init=wide)},
             ),
             layers=layers,
             order=[OrderEntry(layer=i) for i in range(self.n_layer)],
@@ -233,7 +241,7 @@ class GPT2Config:
                 width=d,
                 vocab_size=V,
                 logit_scale=1.0,
-                tensors={"weight": TensorSource(head_weight), "bias": TensorSource("lm_head.bias", required=False)},
+                tensors={"weight": TensorSource(head_weight, init=wide), "bias": TensorSource("lm_head.bias", required=False)},
             ),
             ignorable=tuple(ignorable),
             name_prefixes=("", "transformer."),

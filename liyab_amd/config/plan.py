@@ -20,6 +20,14 @@ from typing import Any, Optional, Sequence
 
 
 @dataclass(frozen=True)
+class Init:
+    """How the random-weights mode draws a tensor: N(mean, std)."""
+
+    std: float
+    mean: float = 0.0
+
+
+@dataclass(frozen=True)
 class TensorSource:
     """Where a part's tensor lives in the weights file.
 
@@ -27,11 +35,14 @@ class TensorSource:
     (the reference's and this engine's working layout: `y = x . W^T`,
     `include/liyab/backend.h:35`), "in_out" = row per input feature (GPT-2's
     four projection matrices). The loader brings every matrix to "out_in".
+    `init` is the distribution the random-weights mode draws the tensor from
+    (None: N(0, 0.02)).
     """
 
     name: str
     layout: str = "out_in"
     required: bool = True
+    init: Optional[Init] = None
 
 
 @dataclass(frozen=True)
@@ -53,8 +64,9 @@ class TokenEmbeddingSpec:
 
 @dataclass(frozen=True)
 class PositionSpec:
-    """A position encoding. `where` = "residual" (added to the embeddings,
-    as learned positions are) or "mixer" (applied to queries and keys)."""
+    """A position encoding. `where` = "residual" (added to the embeddings, as learned
+    positions are: the model's `residual_position`) or "mixer" (applied to queries and keys
+    inside a mixer: that mixer's `position` field; the part then has `rotate(q, k, ctx)`)."""
 
     kind: str  # "learned_positions" | "none"
     where: str
@@ -73,6 +85,9 @@ class AttentionSpec:
     scale: float  # multiplies q.k before the softmax
     window: int  # 0 = every earlier position
     tensors: dict = field(default_factory=dict)  # qkv_weight, qkv_bias, out_weight, out_bias
+    # a position encoding that acts on queries and keys (a spec with a `kind` of the position
+    # registry and where = "mixer"), applied after the projection and before keys go to the cache
+    position: Any = None
 
 
 @dataclass(frozen=True)

@@ -132,7 +132,7 @@ int liyab_sched_finish(void* h, int id) { return static_cast<SchedulerHandle*>(h
 // what: 0 state, 1 computed, 2 pending, 3 generated, 4 preemptions, 5 slot
 int liyab_sched_get(void* h, int id, int what) {
     const auto& s = static_cast<SchedulerHandle*>(h)->sched;
-    if (id < 0 || id >= s.n_requests()) return -1;
+    if (id < 0) return -1;
     switch (what) {
         case 0: return s.state(id);
         case 1: return s.computed(id);

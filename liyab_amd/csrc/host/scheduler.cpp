@@ -29,14 +29,15 @@ Status Scheduler::add(int n_prompt, int max_tokens, int* id, std::string* err) {
     Request r;
     r.n_prompt = n_prompt;
     r.max_tokens = max_tokens;
-    *id = static_cast<int>(reqs_.size());
-    reqs_.push_back(r);
+    *id = next_id_++;
+    reqs_.emplace(*id, r);
     waiting_.push_back(*id);
     return kOk;
 }
 
 bool Scheduler::draining(int id) const {
-    const Request& r = reqs_[id];
+    if (find(id) == nullptr) return false;
+    const Request& r = req(id);
     return r.pending > 0 && (r.n_generated + r.pending >= r.max_tokens || r.n_tokens() > m_->max_positions());
 }
 
@@ -47,13 +48,13 @@ bool Scheduler::pressure() const {
     // a portion of c tokens takes at most ceil(c / page) + 1 new pages of a group
     long long bound = 0;
     for (int id : running_) {
-        const int count = std::min(reqs_[id].remaining(), prefill_chunk_);
+        const int count = std::min(req(id).remaining(), prefill_chunk_);
         if (count > 0) bound += (count + page - 1) / page + 1;
     }
     if (bound <= free) return false;
     std::vector<int> need(static_cast<size_t>(G), 0), extra(static_cast<size_t>(G));
     for (int id : running_) {
-        const Request& r = reqs_[id];
+        const Request& r = req(id);
         const int count = std::min(r.remaining(), prefill_chunk_);
         if (count <= 0) continue;
         m_->pages_needed(r.slot, r.computed + count, extra.data());
@@ -65,7 +66,7 @@ bool Scheduler::pressure() const {
 }
 
 Status Scheduler::preempt(int id, std::string* err) {
-    Request& r = reqs_[id];
+    Request& r = req(id);
     if (r.pending > 0)
         return fail(err, kInternal, "a request with a pending token cannot be preempted: read the tokens first");
     if (Status s = m_->close(r.slot, err)) return s;
@@ -94,7 +95,7 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
     int free = min_free();  // read again whenever a request is preempted
     auto fits = [&](const Request& r, int count) { return need + extra_pages(r, count) <= free; };
     auto take = [&](int id, int count) {
-        Request& r = reqs_[id];
+        Request& r = req(id);
         need += extra_pages(r, count);
         batch->push_back({id, r.slot, r.computed, count, r.computed + count == r.n_tokens() ? 1 : 0});
         budget -= count;
@@ -105,11 +106,11 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
     for (int pass = 0; pass < 2; ++pass)
         for (int id : running_) {
             if (draining(id)) continue;
-            const int rem = reqs_[id].remaining();
+            const int rem = req(id).remaining();
             if ((pass == 0 && rem == 1) || (pass == 1 && rem > 1)) order.push_back(id);
         }
     for (int id : order) {
-        Request& r = reqs_[id];
+        Request& r = req(id);
         if (r.state != kRunning || budget <= 0) continue;
         int count = std::min({r.remaining(), prefill_chunk_, budget});
         while (!fits(r, count)) {
@@ -122,7 +123,7 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
             }
             for (size_t i = 0; i < batch->size();) {
                 if ((*batch)[i].id == victim) {
-                    need -= extra_pages(reqs_[victim], (*batch)[i].count);
+                    need -= extra_pages(req(victim), (*batch)[i].count);
                     budget += (*batch)[i].count;
                     batch->erase(batch->begin() + static_cast<long>(i));
                 } else {
@@ -138,7 +139,7 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
     // admission, first come first served
     while (!waiting_.empty() && static_cast<int>(running_.size()) < max_num_seqs_ && budget > 0) {
         const int id = waiting_.front();
-        Request& r = reqs_[id];
+        Request& r = req(id);
         const int count = std::min({r.remaining(), prefill_chunk_, budget});
         const int pages = (count + m_->page_size() - 1) / m_->page_size();
         if (m_->free_slots() == 0 || need + pages > free) break;
@@ -151,14 +152,14 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
     }
     if (batch->empty() && has_unfinished()) {
         bool any_pending = false;
-        for (int id : running_) any_pending = any_pending || reqs_[id].pending > 0;
+        for (int id : running_) any_pending = any_pending || req(id).pending > 0;
         if (!any_pending)
             return fail(err, kOutOfPages, "no request can make progress: the page pool is too small for any of them");
     }
     stats_.steps += 1;
     for (const Scheduled& s : *batch) {
         stats_.batched_tokens += s.count;
-        if (s.count == 1 && s.wants_logits && reqs_[s.id].n_generated > 0) stats_.decode_tokens += 1;
+        if (s.count == 1 && s.wants_logits && req(s.id).n_generated > 0) stats_.decode_tokens += 1;
     }
     stats_.prefill_tokens = stats_.batched_tokens - stats_.decode_tokens;
     return kOk;
@@ -166,15 +167,15 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
 
 void Scheduler::advance(const Scheduled* batch, int n) {
     for (int i = 0; i < n; ++i) {
-        Request& r = reqs_[batch[i].id];
+        Request& r = req(batch[i].id);
         r.computed += batch[i].count;
         if (batch[i].wants_logits) r.pending += 1;
     }
 }
 
 int Scheduler::token(int id, bool is_stop_token) {
-    Request& r = reqs_[id];
-    if (r.state == kFinished) return kAlreadyFinished;
+    if (find(id) == nullptr) return kAlreadyFinished;
+    Request& r = req(id);
     r.pending -= 1;
     r.n_generated += 1;
     int reason = kGoesOn;
@@ -186,7 +187,8 @@ int Scheduler::token(int id, bool is_stop_token) {
 }
 
 Status Scheduler::finish(int id, std::string* err) {
-    Request& r = reqs_[id];
+    if (find(id) == nullptr) return kOk;  // finished before
+    Request& r = req(id);
     if (r.state == kRunning) {
         if (Status s = m_->close(r.slot, err)) return s;
         running_.erase(std::find(running_.begin(), running_.end(), id));
@@ -194,8 +196,7 @@ Status Scheduler::finish(int id, std::string* err) {
     } else if (r.state == kWaiting) {
         waiting_.erase(std::find(waiting_.begin(), waiting_.end(), id));
     }
-    r.state = kFinished;
-    r.pending = 0;
+    reqs_.erase(id);
     return kOk;
 }
 

@@ -26,6 +26,7 @@
 
 #include <deque>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "cache_manager.h"
@@ -70,13 +71,15 @@ public:
     // Ends a request for any other reason (callback, cancel); gives back what it holds.
     Status finish(int id, std::string* err);
 
-    int state(int id) const { return reqs_[id].state; }
-    int computed(int id) const { return reqs_[id].computed; }
-    int pending(int id) const { return reqs_[id].pending; }
-    int n_generated(int id) const { return reqs_[id].n_generated; }
-    int preemptions(int id) const { return reqs_[id].preemptions; }
-    int slot(int id) const { return reqs_[id].slot; }
-    int n_requests() const { return static_cast<int>(reqs_.size()); }
+    // A finished request is forgotten (ids are never given out twice): it reads as finished,
+    // holding nothing.
+    int state(int id) const { const Request* r = find(id); return r ? r->state : kFinished; }
+    int computed(int id) const { const Request* r = find(id); return r ? r->computed : 0; }
+    int pending(int id) const { const Request* r = find(id); return r ? r->pending : 0; }
+    int n_generated(int id) const { const Request* r = find(id); return r ? r->n_generated : 0; }
+    int preemptions(int id) const { const Request* r = find(id); return r ? r->preemptions : 0; }
+    int slot(int id) const { const Request* r = find(id); return r ? r->slot : -1; }
+    int n_requests() const { return static_cast<int>(reqs_.size()); }  // the unfinished ones
     const std::vector<int>& running() const { return running_; }
     const std::deque<int>& waiting() const { return waiting_; }
     const SchedulerStats& stats() const { return stats_; }
@@ -96,10 +99,17 @@ private:
         return (r.computed + count + p - 1) / p - (r.computed + p - 1) / p;
     }
     Status preempt(int id, std::string* err);
+    const Request* find(int id) const {
+        auto it = reqs_.find(id);
+        return it == reqs_.end() ? nullptr : &it->second;
+    }
+    Request& req(int id) { return reqs_.at(id); }
+    const Request& req(int id) const { return reqs_.at(id); }
 
     CacheManager* m_;
     int max_num_seqs_, max_batched_tokens_, prefill_chunk_;
-    std::vector<Request> reqs_;
+    std::unordered_map<int, Request> reqs_;  // waiting and running requests by id; a finished one is erased
+    int next_id_ = 0;
     std::deque<int> waiting_;
     std::vector<int> running_;  // in order of admission
     SchedulerStats stats_{};

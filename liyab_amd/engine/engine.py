@@ -46,11 +46,15 @@ class GenerationResult:
 
 
 class Engine:
-    def __init__(self, model: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
+    def __init__(self, model: Optional[str] = None, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_num_seqs: int = 64,
                  max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None,
-                 overlap: bool = True):
-        """`model`: a folder with config.json and model.safetensors. `ctx`: the
+                 overlap: bool = True, use_graphs: bool = True, core: Optional[EngineCore] = None):
+        """`model`: a folder with config.json and model.safetensors; or `core`: an `EngineCore`
+        built elsewhere (`EngineCore.from_plan` for a model made of a plan and tensors), whose
+        own dtype, pages and graph setting then hold. `use_graphs`: replay recurring step shapes
+        as captured HIP graphs (a part that decides on the host from a step's values, not from
+        its shape, needs this off). `ctx`: the
         context length (default: the model's). `prefill_chunk`: the longest
         portion of a prompt in one step (the reference's 256,
         src/core/engine.cpp:2863-2864). `num_pages` / `max_tokens` size the
@@ -58,8 +62,14 @@ class Engine:
         this step's tokens (decoding requests take their last token from a table on the
         device); finishing by an end token is then seen one step late and that step's work
         for the request is dropped. Tokens are the same either way."""
-        self.core = EngineCore(model, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
-                               max_tokens=max_tokens, max_requests=max_num_seqs, context_length=ctx)
+        if core is not None:
+            if model is not None:
+                raise InvalidArgument("give a model folder or a built core, not both")
+            self.core = core
+        else:
+            self.core = EngineCore(model, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
+                                   max_tokens=max_tokens, max_requests=max_num_seqs, context_length=ctx,
+                                   use_graphs=use_graphs)
         self.scheduler = Scheduler(self.core.manager, max_num_seqs=max_num_seqs,
                                    max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
                                    eos_token_id=self.core.model.plan.eos_token_id, on_open=self._reset_slot)
@@ -119,6 +129,8 @@ class Engine:
         r = Request(rid=rid, prompt=prompt, params=params, seed=params.resolved_seed())
         self.scheduler.add(r)
         self._requests[rid] = r
+        self._t_first.pop(rid, None)  # an id used before starts its clocks again
+        self._t_end.pop(rid, None)
         self._t_start[rid] = time.perf_counter()
         return rid
 
@@ -206,6 +218,13 @@ class Engine:
         if r is not None and r.state != "finished":
             self.scheduler.finish(r, "cancelled")  # a step in flight may still hold it: its result is dropped
 
+    def release(self, rid: Hashable) -> None:
+        """Forgets a finished request (its tokens and clocks); `result(rid)` is gone after it."""
+        r = self._requests.get(rid)
+        if r is not None and r.state == "finished":
+            for table in (self._requests, self._t_start, self._t_first, self._t_end):
+                table.pop(rid, None)
+
     def result(self, rid: Hashable) -> GenerationResult:
         r = self._requests[rid]
         end = time.perf_counter()
@@ -245,4 +264,6 @@ class Engine:
             self.step(on_token)
         self.flush(on_token)
         results = [self.result(r) for r in rids]
+        for r in rids:
+            self.release(r)
         return results[0] if single else results

@@ -260,6 +260,7 @@ class Scheduler:
         r.state = FINISHED
         r.pending = 0
         r.finish_reason = reason
+        self._by_sid.pop(r.sid, None)  # the native side has forgotten it too; ids are never given out twice
 
     def finish(self, r: Request, reason: str) -> None:
         if r.state != FINISHED:

@@ -775,6 +775,14 @@ def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int):
 SPLIT4_PAIRS, SPLIT2_PAIRS = 192, 192
 
 
+ATTENTION_MAX_HEAD_DIM = 256  # what the attention kernels take (attention_generic.hip, attention_decode.hip)
+
+
+def attention_takes(head_dim: int) -> bool:
+    """Whether some attention kernel of the library takes this head size, in either precision."""
+    return 0 < head_dim <= ATTENTION_MAX_HEAD_DIM
+
+
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0,
               splits_ok: bool = False) -> Optional[torch.Tensor]:

@@ -8,10 +8,11 @@ import torch
 
 from ..cache.pages import KVSpec
 from ..cache.storage import LayerCache
+from ..errors import Unsupported
 from ..kernels import ops
 from .base import StepContext, settled
 from .linear import linear, linear_deferred, paged_qkv_takes
-from .registry import register_mixer
+from .registry import build_part, register_mixer
 
 
 class Attention:
@@ -24,7 +25,11 @@ class Attention:
     softmax and weighted values over positions [0, pos] or the last `window`
     (:2162-2453); out = att . Wo^T + bo added into the residual (:3139-3140,
     :5647). Head counts, head size, scale and window are the spec's; queries
-    may outnumber key/value heads by a whole factor."""
+    may outnumber key/value heads by a whole factor. A position encoding of the
+    spec's (`spec.position`, a part of the position registry with `rotate(q, k,
+    ctx)`) acts on the step's queries and keys in place between the projection
+    and the cache write, where the reference applies its rotary encoding
+    (:3113-3116); GPT-2 has none."""
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.spec = spec
@@ -33,6 +38,10 @@ class Attention:
         self.n_head, self.n_kv_head, self.head_dim = spec.n_head, spec.n_kv_head, spec.head_dim
         if self.n_head % self.n_kv_head != 0:
             raise ValueError(f"{self.n_head} query heads are no multiple of {self.n_kv_head} key/value heads")
+        if not ops.attention_takes(self.head_dim):
+            # said when the model is built, not at its first step
+            raise Unsupported(f"attention: heads of {self.head_dim} are not supported (the kernels take head sizes up to "
+                              f"{ops.ATTENTION_MAX_HEAD_DIM})")
         self.scale = float(spec.scale)
         self.window = int(spec.window)
         self.q_dim = self.n_head * self.head_dim
@@ -43,6 +52,10 @@ class Attention:
         self.qkv_bias = store.fetch(t["qkv_bias"], (qkv_out,), "vector") if "qkv_bias" in t else None
         self.out_weight = store.fetch(t["out_weight"], (self.width, self.q_dim), "matrix")
         self.out_bias = store.fetch(t["out_bias"], (self.width,), "vector") if "out_bias" in t else None
+        pos = getattr(spec, "position", None)
+        self.position = build_part("position", pos, store, dtype) if pos is not None else None
+        if self.position is not None and getattr(self.position, "where", None) != "mixer":
+            raise ValueError(f"position encoding '{pos.kind}' does not act inside a mixer (where = 'mixer')")
 
     def cache_spec(self) -> Optional[KVSpec]:
         return KVSpec(self.n_kv_head, self.head_dim, self.window)
@@ -61,13 +74,16 @@ class Attention:
         n = h.shape[0]
         ws = ctx.workspace
         group = ctx.groups[cache.group]
-        if writes_cache and paged_qkv_takes(self.dtype, self.width):
+        if writes_cache and self.position is None and paged_qkv_takes(self.dtype, self.width):
             # the projection's epilogue puts keys and values straight into their pages
             q = ws.get("q", (n, self.q_dim), self.dtype)
             linear(h, self.qkv_weight, self.qkv_bias, out=q, kv=(cache.k, cache.v, group.slots, self.q_dim))
         else:
             q = ws.get("qkv", (n, self.q_dim + 2 * self.kv_dim), self.dtype)
             linear(h, self.qkv_weight, self.qkv_bias, out=q)
+            if self.position is not None:
+                # queries and keys of this step's tokens, rotated where they lie, before a key is stored
+                self.position.rotate(q[:, :self.q_dim], q[:, self.q_dim:self.q_dim + self.kv_dim], ctx)
             if writes_cache:
                 ops.kv_write(cache.k, cache.v, q, self.q_dim, self.q_dim + self.kv_dim, group.slots)
         att = ws.get("att", (n, self.q_dim), self.dtype)

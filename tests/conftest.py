@@ -34,12 +34,29 @@ CONFIG_C = {
 }
 CONFIGS = {"A": (CONFIG_A, 0), "B": (CONFIG_B, 2), "C": (CONFIG_C, 5)}
 
-# tolerances, relative to the largest |logit| of the compared row; fixed, never widened to pass
-TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+# Tolerances, relative to the largest |logit| of the compared row; fixed, never widened to pass.
+# A test session prints the largest error each family of checks saw (pytest_terminal_summary below).
+# float32: the engine's families show 0.5e-6 to 3.2e-6 (the largest at GPT-2 XL's layer sizes).
+# bfloat16, GPT-2 models with the benchmark's weight distributions: 2.6e-3 to 6.4e-3 (the largest at
+# XL's layer sizes again); the tolerance is twice that largest. It was 2e-2 before the errors were on record.
+TOL = {"float32": 1e-5, "bfloat16": 1.3e-2}
+# The toy models of test_parts_gpu.py draw weights five to ten times as large and run torch arithmetic
+# of their own between the framework's kernels (values rounded to bfloat16 twice): 7.8e-3 to 1.27e-2.
+TOL_TOY = {"float32": 1e-5, "bfloat16": 2e-2}
 
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu)")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The largest relative error each family of logit checks saw, beside its tolerance."""
+    import trace_tools
+
+    if trace_tools.WORST:
+        terminalreporter.write_line("largest relative error of the engine's logits against the plain implementation:")
+        for (family, tol), worst in sorted(trace_tools.WORST.items(), key=lambda kv: (kv[0][1], kv[0][0])):
+            terminalreporter.write_line(f"  {family:<24} tolerance {tol:.0e}  worst {worst:.3e}  ({worst / tol:.2f} of it)")
 
 
 @pytest.fixture(scope="session")

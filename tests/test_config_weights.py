@@ -12,7 +12,7 @@ from conftest import CONFIG_A, CONFIG_B
 from liyab_amd import InvalidModel, Unsupported
 from liyab_amd.config import GPT2Config, config_from_dict, find_architecture, load_config, supported_architectures
 from liyab_amd.models.decoder import DecoderModel
-from liyab_amd.weights import SafetensorsFile, WeightStore, random_gpt2_tensors, write_random_model, write_safetensors
+from liyab_amd.weights import SafetensorsFile, WeightStore, random_tensors, write_random_model, write_safetensors
 
 
 def test_config_reads_every_key():
@@ -129,7 +129,7 @@ def _build(tensors, cfg=CONFIG_A, dtype=torch.float32):
 
 def test_weights_load_by_name_with_dtypes_and_layouts():
     cfg = config_from_dict(dict(CONFIG_A))
-    t = random_gpt2_tensors(cfg, 0)
+    t = random_tensors(cfg, 0)
     t["h.0.attn.bias"] = torch.ones(1, 1, 8, 8)  # buffers a checkpoint may carry: ignored
     t["h.1.attn.masked_bias"] = torch.tensor(-1e4)
     t["lm_head.weight"] = t["wte.weight"]
@@ -139,10 +139,10 @@ def test_weights_load_by_name_with_dtypes_and_layouts():
     assert torch.equal(att.qkv_weight, t["h.0.attn.c_attn.weight"].t().to(torch.bfloat16))
     assert att.qkv_bias.dtype == torch.float32 and m.blocks[1].norm_ffn.weight.dtype == torch.float32
     assert m.head.weight.data_ptr() == m.embedding.table.data_ptr()  # tied: resident once
-    m32 = _build({("transformer." + k): v for k, v in random_gpt2_tensors(cfg, 0).items()})  # prefixed names
+    m32 = _build({("transformer." + k): v for k, v in random_tensors(cfg, 0).items()})  # prefixed names
     assert m32.blocks[0].ffn.up_weight.dtype == torch.float32 and m32.blocks[0].ffn.up_weight.shape == (256, 64)
     # a file stored in bfloat16 runs on the 32-bit path too (exact upcast)
-    bf = {k: (v.to(torch.bfloat16) if v.dim() == 2 else v) for k, v in random_gpt2_tensors(cfg, 0).items()}
+    bf = {k: (v.to(torch.bfloat16) if v.dim() == 2 else v) for k, v in random_tensors(cfg, 0).items()}
     m3 = _build(bf)
     assert m3.embedding.table.dtype == torch.float32
     assert torch.equal(m3.embedding.table, bf["wte.weight"].float())
@@ -150,7 +150,7 @@ def test_weights_load_by_name_with_dtypes_and_layouts():
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes():
     cfg = config_from_dict(dict(CONFIG_A))
-    t = random_gpt2_tensors(cfg, 0)
+    t = random_tensors(cfg, 0)
     del t["h.1.ln_2.bias"], t["wpe.weight"]
     t["h.0.mlp.c_fc.weight"] = torch.zeros(256, 64)  # stored [out, in]: the wrong way round
     t["ln_f.weight"] = torch.zeros(65)
@@ -168,7 +168,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes():
 
 def test_untied_head_needs_its_tensor():
     cfg = config_from_dict(dict(CONFIG_A, tie_word_embeddings=False))
-    t = random_gpt2_tensors(cfg, 0)
+    t = random_tensors(cfg, 0)
     m = _build(t, cfg=dict(CONFIG_A, tie_word_embeddings=False))
     assert m.head.weight.data_ptr() != m.embedding.table.data_ptr()
     del t["lm_head.weight"]
@@ -192,3 +192,73 @@ def test_random_weights_mode_writes_a_folder(tmp_path):
     w = f1.tensor("h.1.mlp.c_fc.weight").double()
     assert abs(w.std().item() - 0.02) < 2e-3 and abs(f1.tensor("h.0.ln_1.weight").mean().item() - 1.0) < 0.05
     assert abs(f1.tensor("h.1.attn.c_proj.weight").double().std().item() - 0.02 / (2 * 3) ** 0.5) < 1e-3
+
+
+def test_random_weights_come_from_the_plan_not_from_an_architecture():
+    """A plan nobody has registered as an architecture, with a part of its own: the
+    random-weights mode draws exactly what its parts ask for, each tensor from the rule the
+    plan gives with its name, in the layout the plan says the file holds; and a tensor's
+    values depend on the seed and its name only."""
+    from liyab_amd.config.plan import (HeadSpec, Init, LayerSpec, ModelPlan, NormSpec, OrderEntry, TensorSource,
+                                       TokenEmbeddingSpec)
+    from liyab_amd.parts.registry import register_mixer
+
+    class Gate:  # a mixer that scales the stream by a learned vector and keeps nothing
+        def __init__(self, spec, store, dtype):
+            self.scale = store.fetch(spec.tensors["scale"], (spec.width,), "vector")
+            self.mix = store.fetch(spec.tensors["mix"], (spec.width, 7), "matrix")
+            self.extra = store.fetch(spec.tensors["extra"], (3,), "vector")  # optional, absent
+
+        def cache_spec(self): return None
+        def state_spec(self): return None
+
+    register_mixer("test_gate", Gate)
+
+    class GateSpec:
+        kind = "test_gate"
+
+        def __init__(self, layer, width):
+            self.width = width
+            self.tensors = {"scale": TensorSource(f"l.{layer}.scale", init=Init(0.5, 3.0)),
+                            "mix": TensorSource(f"l.{layer}.mix", layout="in_out"),
+                            "extra": TensorSource(f"l.{layer}.extra", required=False)}
+
+    def toy(n_layer, d=12, V=40):
+        emb = TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": TensorSource("emb", init=Init(1.0))})
+        layers = [LayerSpec(mixer=GateSpec(i, d), ffn=None, norm_mixer=None, norm_ffn=None) for i in range(n_layer)]
+        return ModelPlan(architecture="toy", width=d, vocab_size=V, max_positions=64, embedding=emb, residual_position=None,
+                         layers=layers, order=[OrderEntry(i) for i in range(n_layer)],
+                         final_norm=NormSpec("layernorm", d, 1e-5, {"weight": TensorSource("out_norm.w", init=Init(0.05, 1.0))}),
+                         head=HeadSpec("lm_head", d, V, 1.0, {"weight": TensorSource("emb")}))
+
+    t2, t3 = random_tensors(toy(2), 9), random_tensors(toy(3), 9)
+    assert sorted(t2) == ["emb", "l.0.mix", "l.0.scale", "l.1.mix", "l.1.scale", "out_norm.w"]
+    assert t2["l.0.mix"].shape == (7, 12)  # stored [in, out], as the plan says
+    assert abs(t2["l.1.scale"].mean().item() - 3.0) < 0.6 and abs(t2["emb"].std().item() - 1.0) < 0.15
+    assert abs(t2["l.0.mix"].std().item() - 0.02) < 0.01  # no rule given: N(0, 0.02)
+    for k in t2:
+        assert torch.equal(t2[k], t3[k])  # another layer changes none of the others
+    assert not torch.equal(t2["l.0.scale"], random_tensors(toy(2), 10)["l.0.scale"])
+    assert not torch.equal(t2["l.0.scale"], t2["l.1.scale"])
+
+
+def test_the_four_projection_matrices_share_one_stored_layout():
+    """GPT-2's checkpoints hold c_attn, attn.c_proj, c_fc and mlp.c_proj under one rule: the
+    reference's converter treats exactly these four suffixes in one branch
+    (docs/validation/models-stage1/converter-classic.patch:14-20). Three of them show by their
+    shapes which way round they are stored ([in, out]: c_attn is [d, 3d]); the square attn.c_proj
+    cannot, and follows the rule of the other three. The loader refuses each of the three
+    unambiguous ones when it is stored the other way round."""
+    cfg = config_from_dict(dict(CONFIG_B))
+    plan = cfg.plan()
+    for layer in plan.layers:
+        layouts = {layer.mixer.tensors["qkv_weight"].layout, layer.mixer.tensors["out_weight"].layout,
+                   layer.ffn.tensors["up_weight"].layout, layer.ffn.tensors["down_weight"].layout}
+        assert layouts == {"in_out"}
+    for name, shape in (("h.0.attn.c_attn.weight", [96, 288]), ("h.1.mlp.c_fc.weight", [96, 320]),
+                        ("h.2.mlp.c_proj.weight", [320, 96])):
+        t = random_tensors(cfg, 1)
+        assert list(t[name].shape) == shape
+        t[name] = t[name].t().contiguous()
+        with pytest.raises(InvalidModel, match=name.replace(".", r"\.")):
+            _build(t, cfg=CONFIG_B)

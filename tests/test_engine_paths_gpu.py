@@ -1,0 +1,253 @@
+"""Paths of the engine that a plain run of prompts does not reach (needs the GPU): a pool so
+small that requests are preempted and recomputed, HIP graphs replayed and compared with eager
+runs of the same steps, geometries that take the kernels' fallbacks in bfloat16, a head of its
+own (untied), and sizes refused when a model is built."""
+
+import numpy as np
+import pytest
+
+import plain_gpt2 as plain
+import trace_tools as tt
+from conftest import CONFIGS, TOL
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+
+def _near_argmax(ref_row, token, tol):
+    ref_row = np.asarray(ref_row, dtype=np.float64)
+    return ref_row[token] >= ref_row.max() - tol * np.abs(ref_row).max()
+
+
+# ---------------------------------------------------------------------------
+# preemption and recomputation on the device
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("overlap", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_preempted_requests_are_recomputed_to_the_same_tokens(dtype, overlap, model_dirs, plain_models):
+    """Three prompts of 30 tokens that each grow to 74 positions (5 pages of 16) in a pool of 8
+    pages: they cannot all stay, so the latest admitted is preempted, its pages go to the others
+    and it is recomputed from its prompt plus what it had generated, through pages other
+    requests have used. Greedy and seeded: the tokens are those of each request alone (in
+    32-bit also the plain implementation's), whatever was preempted when."""
+    from liyab_amd import Engine, SamplingParams
+
+    name = "B"
+    cfg, _ = CONFIGS[name]
+    config, tensors = plain_models[name]
+    weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+    V = cfg["vocab_size"]
+    prompts = [tt.random_tokens(900 + i, 30, V) for i in range(3)]
+    for sp in (SamplingParams(temperature=0.0, max_tokens=45),
+               SamplingParams(temperature=0.8, top_k=0, top_p=1.0, seed=4, max_tokens=45)):
+        tight = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=8, max_num_seqs=3, max_batched_tokens=64,
+                       prefill_chunk=32, overlap=overlap)
+        tight.stop_at_eos = False
+        for c in tight.core.storage.layers.values():  # free pages hold NaN
+            c.k.fill_(float("nan"))
+            c.v.fill_(float("nan"))
+        together = tight.generate(prompts, sp)
+        stats = tight.scheduler.stats
+        assert stats.preemptions >= 1, "the pool held every request: nothing was preempted"
+        assert sum(r.stats.preemptions for r in together) == stats.preemptions
+        assert tight.core.manager.pages_in_use() == 0
+        tight.core.manager.check()
+        assert tight.core.step_fn.graph_replays > 0
+        roomy = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=64, max_num_seqs=3, max_batched_tokens=64,
+                       prefill_chunk=32, overlap=overlap)
+        roomy.stop_at_eos = False
+        alone = [roomy.generate(p, sp) for p in prompts]
+        assert roomy.scheduler.stats.preemptions == 0
+        for prompt, a, b in zip(prompts, together, alone):
+            assert len(a.tokens) == 45 and a.finish_reason == "length"
+            if dtype == "float32":
+                assert a.tokens == b.tokens
+                if sp.temperature == 0.0:
+                    assert a.tokens == plain.generate_greedy(config, tensors, prompt, 45)
+            elif sp.temperature == 0.0:
+                # bfloat16: each token is the plain implementation's choice given the tokens before it,
+                # within the tolerance (a recomputed prompt goes through other kernels than single tokens)
+                ref = plain.forward(config, weights, prompt + a.tokens[:-1])
+                for i, t in enumerate(a.tokens):
+                    assert _near_argmax(ref[len(prompt) - 1 + i], t, TOL[dtype]), f"token {i}"
+
+
+# ---------------------------------------------------------------------------
+# HIP graphs: replays happen, and give what eager runs give
+# ---------------------------------------------------------------------------
+def _graph_schedule(V, P):
+    """Steps that bring the same shapes again and again with different contents: a decode shape
+    (two requests, one token each) many times, across a context bucket's edge (256); and a
+    mixed shape of 500 tokens cut (300, 200) and (270, 230), which fall into the same tiles and
+    the same bucket, five times and more."""
+    assert P >= 600
+    steps = []
+    a = tt.random_tokens(1, 300, V)
+    b = tt.random_tokens(2, 300, V)
+    # two requests that decode from 250 to 262: the bucket changes from 256 to 512 on the way
+    steps.append({"entries": [("a", a[:250], [249]), ("b", b[:250], [0, 249])], "end": []})
+    for i in range(250, 262):
+        steps.append({"entries": [("a", a[i:i + 1], [0]), ("b", b[i:i + 1], [0])], "end": ["a", "b"] if i == 261 else []})
+    # the mixed shape, each time with other tokens and another cut
+    for i in range(7):
+        x = tt.random_tokens(10 + i, 300, V)
+        y = tt.random_tokens(30 + i, 300, V)
+        nx, ny = (300, 200) if i % 2 == 0 else (270, 230)
+        steps.append({"entries": [(f"x{i}", x[:nx], [0, nx - 1]), (f"y{i}", y[:ny], [ny - 1])], "end": [f"x{i}", f"y{i}"]})
+    # a decode shape of three requests beside, so that a small table of graphs has to drop one
+    c = tt.random_tokens(3, 40, V)
+    steps.append({"entries": [("a2", a[:20], []), ("b2", b[:20], []), ("c2", c[:20], [])], "end": []})
+    for i in range(20, 26):
+        steps.append({"entries": [("a2", a[i:i + 1], [0]), ("b2", b[i:i + 1], [0]), ("c2", c[i:i + 1], [0])], "end": []})
+    for i in range(26, 32):  # back to two: its graph may have been dropped meanwhile, and is captured again
+        steps.append({"entries": [("a2", a[i:i + 1], [0]), ("b2", b[i:i + 1], [0])], "end": []})
+    steps[-1]["end"] = ["a2", "b2", "c2"]
+    return steps
+
+
+def _run_steps(core, steps):
+    from liyab_amd.engine import StepItem
+
+    out = []
+    for st in steps:
+        items = []
+        for rid, toks, want in st["entries"]:
+            if not core.is_open(rid):
+                core.open(rid)
+            items.append(StepItem(rid, toks, want))
+        logits = core.step(items)
+        out.append(None if logits is None else logits.float().cpu().numpy().copy())
+        for rid in st["end"]:
+            core.close(rid)
+    return out
+
+
+@pytest.mark.parametrize("max_graphs", [256, 2])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replayed_graphs_give_the_eager_logits(dtype, max_graphs, model_dirs):
+    """The same steps through an engine that captures and replays HIP graphs and through one that
+    launches every kernel itself: the same bits at every step. Shapes recur with other contents
+    (other tokens, other cuts into requests, a context past a bucket's edge), so a kernel argument
+    that a graph had baked in where it should have come from the step's metadata would show.
+    With room for two graphs only, shapes are dropped and captured again in between."""
+    from liyab_amd.engine import EngineCore
+
+    name = "C"
+    cfg, _ = CONFIGS[name]
+    steps = _graph_schedule(cfg["vocab_size"], cfg["n_positions"])
+    eager = EngineCore(model_dirs[name], dtype=dtype, page_size=16, max_tokens=2048, max_requests=8, use_graphs=False)
+    want = _run_steps(eager, steps)
+    assert eager.step_fn.graph_replays == 0
+    graphs = EngineCore(model_dirs[name], dtype=dtype, page_size=16, max_tokens=2048, max_requests=8, use_graphs=True)
+    graphs.step_fn.max_graphs = max_graphs
+    got = _run_steps(graphs, steps)
+    fn = graphs.step_fn
+    captured = [k for k, v in fn._graphs.items() if isinstance(v, tuple)]
+    assert fn.graph_replays >= (15 if max_graphs > 2 else 8), fn.graph_replays
+    if max_graphs > 2:
+        assert any(k[3] == "decode" for k in captured) and any(k[3] == "prefill" for k in captured), captured
+    else:
+        assert len(fn._graphs) <= 2
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert (g is None) == (w is None)
+        if g is not None:
+            assert np.array_equal(g, w), f"step {i} ({[(r, len(t)) for r, t, _ in steps[i]['entries']]}): replayed and eager logits differ"
+    graphs.manager.check()
+    assert graphs.manager.pages_in_use() == 0
+
+
+# ---------------------------------------------------------------------------
+# geometries that take the kernels' fallbacks in bfloat16; a head of its own
+# ---------------------------------------------------------------------------
+FALLBACKS = {
+    # width 60 = 3 heads of 20: no multiple of 8, so in bfloat16 neither the matrix-core products nor
+    # the paged QKV epilogue nor the fast attention take it (plain product + kv_write + plain attention)
+    "w60_h20": dict(n_layer=2, n_embd=60, n_head=3, n_inner=100, vocab_size=333, n_positions=200),
+    # width 44 = 4 heads of 11
+    "w44_h11": dict(n_layer=1, n_embd=44, n_head=4, n_inner=50, vocab_size=97, n_positions=160,
+                    activation_function="gelu", scale_attn_by_inverse_layer_idx=True),
+    # heads of 40 (8 x odd): matrix cores for the products, the decode kernel, no tiled prefill attention
+    "w120_h40": dict(n_layer=2, n_embd=120, n_head=3, n_inner=90, vocab_size=500, n_positions=300),
+    # heads of 24 in a width of 72, an untied head and eps 1e-6
+    "w72_h24_untied": dict(n_layer=2, n_embd=72, n_head=3, n_inner=64, vocab_size=211, n_positions=180,
+                           tie_word_embeddings=False, layer_norm_epsilon=1e-6),
+    # an untied head at sizes every fast kernel takes
+    "w64_untied": dict(n_layer=2, n_embd=64, n_head=2, n_inner=256, vocab_size=1031, n_positions=256,
+                       tie_word_embeddings=False),
+}
+
+
+@pytest.mark.parametrize("name", list(FALLBACKS))
+def test_fallback_geometries_whole_and_mixed(name, tmp_path):
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new", **FALLBACKS[name]}
+    seed = 700 + list(FALLBACKS).index(name)
+    write_random_model(str(tmp_path), cfg, seed)
+    config, tensors = plain.read_model(str(tmp_path))
+    if not cfg.get("tie_word_embeddings", True):
+        assert "lm_head.weight" in tensors and not np.array_equal(tensors["lm_head.weight"], tensors["wte.weight"])
+    P, V = cfg["n_positions"], cfg["vocab_size"]
+    reqs = {f"f{i}": tt.random_tokens(seed * 10 + i, n, V) for i, n in enumerate([P, 37, 3, 101])}
+    for dtype in DTYPES:
+        weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+        refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+        for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=seed, decode_tail=7)),
+                             ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48, 2)))):
+            core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=8)
+            for c in core.storage.layers.values():
+                c.k.fill_(float("nan"))
+                c.v.fill_(float("nan"))
+            got = tt.run_schedule(core, steps)
+            tt.check_against_plain(got, reqs, refs, TOL[dtype], f"{name} {label} {dtype}", family=f"fallback:{name}")
+            core.manager.check()
+            assert core.manager.pages_in_use() == 0
+            del core
+
+
+def test_untied_head_is_the_heads_own_matrix(tmp_path):
+    """With tie_word_embeddings false the logits come from lm_head.weight: they equal the plain
+    implementation's with its own head and are far from what the embedding table as head gives."""
+    from liyab_amd.engine import EngineCore, StepItem
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], **FALLBACKS["w64_untied"]}
+    write_random_model(str(tmp_path), cfg, 5)
+    config, tensors = plain.read_model(str(tmp_path))
+    toks = tt.random_tokens(8, 50, cfg["vocab_size"])
+    core = EngineCore(str(tmp_path), dtype="float32", page_size=16, max_tokens=64)
+    core.open("r")
+    got = core.step([StepItem("r", toks, list(range(50)))]).cpu().numpy()
+    assert tt.rel_err(got, plain.forward(config, tensors, toks)) <= TOL["float32"]
+    tied = dict(config, tie_word_embeddings=True)
+    assert tt.rel_err(got, plain.forward(tied, tensors, toks)) > 1e-2  # the embedding table is not the head
+
+
+def test_head_sizes_the_kernels_cannot_take_are_refused_at_load(tmp_path):
+    """One head of 272: no attention kernel takes it, and the model says so when it is built
+    (from a folder, and already when the random-weights mode builds it), not at its first step."""
+    import json
+
+    import torch
+
+    from liyab_amd import Unsupported
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model, write_safetensors
+
+    d, F, V, P = 272, 16, 20, 16
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 1, "n_embd": d, "n_head": 1, "n_inner": F, "vocab_size": V,
+           "n_positions": P}
+    with pytest.raises(Unsupported, match="272"):
+        write_random_model(str(tmp_path / "drawn"), cfg, 1)
+    shapes = {"wte.weight": (V, d), "wpe.weight": (P, d), "ln_f.weight": (d,), "ln_f.bias": (d,), "h.0.ln_1.weight": (d,),
+              "h.0.ln_1.bias": (d,), "h.0.ln_2.weight": (d,), "h.0.ln_2.bias": (d,), "h.0.attn.c_attn.weight": (d, 3 * d),
+              "h.0.attn.c_attn.bias": (3 * d,), "h.0.attn.c_proj.weight": (d, d), "h.0.attn.c_proj.bias": (d,),
+              "h.0.mlp.c_fc.weight": (d, F), "h.0.mlp.c_fc.bias": (F,), "h.0.mlp.c_proj.weight": (F, d), "h.0.mlp.c_proj.bias": (d,)}
+    folder = tmp_path / "written"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    write_safetensors(str(folder / "model.safetensors"), {k: torch.zeros(s) for k, s in shapes.items()}, {})
+    with pytest.raises(Unsupported, match="272"):
+        EngineCore(str(folder), dtype="float32", page_size=16, max_tokens=64)

@@ -11,7 +11,7 @@ import torch
 
 import plain_gpt2 as plain
 import trace_tools as tt
-from conftest import TOL
+from conftest import TOL, TOL_TOY
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -80,10 +80,13 @@ def f64(t):
 # ---------------------------------------------------------------------------
 # plain formulas for the toy models (whole sequences, float64)
 # ---------------------------------------------------------------------------
-def plain_attention(h, tw, prefix, H, Hkv, hd, scale, window=0, kv_from=None):
-    """QKV with [out, in] weights, grouped heads, optional window; `kv_from` = (k, v) of another layer."""
+def plain_attention(h, tw, prefix, H, Hkv, hd, scale, window=0, kv_from=None, rotate=None):
+    """QKV with [out, in] weights, grouped heads, optional window; `kv_from` = (k, v) of another
+    layer; `rotate(x, heads)` acts on queries and keys before any score."""
     qkv = h @ f64(tw[prefix + ".qkv.w"]).T + f64(tw[prefix + ".qkv.b"])
     q, k, v = qkv[:, :H * hd], qkv[:, H * hd:(H + Hkv) * hd], qkv[:, (H + Hkv) * hd:]
+    if rotate is not None:
+        q, k = rotate(q, H), rotate(k, Hkv)
     if kv_from is not None:
         k, v = kv_from
     rep = H // Hkv
@@ -491,7 +494,7 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
     plan, tw, info = toy_model(dtype)
     reqs = {f"t{i}": tt.random_tokens(90 + i, n, info["V"]) for i, n in enumerate([37, 90, 5, 128, 61])}
     ref = {rid: toy_plain(tw, info, toks) for rid, toks in reqs.items()}
-    tol = TOL[dtype]
+    tol = TOL_TOY[dtype]
     for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48))),
                         ("mixed", tt.schedule_mixed(reqs, seed=3))):
         core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4,
@@ -649,13 +652,124 @@ def test_toy_architecture_with_routing_and_computed_positions(dtype):
                 reqs[rid] = toks[:max(2, int(close[0]))]
                 ref[rid] = ref[rid][:len(reqs[rid])]
     assert sum(len(t) for t in reqs.values()) > 60
-    tol = TOL[dtype]
+    tol = TOL_TOY[dtype]
     for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3))),
                         ("mixed", tt.schedule_mixed(reqs, seed=5))):
         core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4,
                                     use_graphs=False)
         got = tt.run_schedule(core, steps)
         tt.check_against_plain(got, reqs, ref, tol, f"routed toy {name} {dtype}")
+        core.manager.check()
+        assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
+
+
+# ---------------------------------------------------------------------------
+# a toy position encoding that acts on queries and keys inside attention
+# ---------------------------------------------------------------------------
+class TurnSpec:
+    kind = "toy_turn"
+    where = "mixer"
+
+    def __init__(self, head_dim, base):
+        self.head_dim, self.base = head_dim, base
+
+
+class TurnPositions:
+    """Turns each pair (x[2i], x[2i + 1]) of a head by the angle pos * base^(-2i / head size): a
+    test's toy in torch. It acts on the step's queries and keys where they lie, between the
+    projection and the cache write, from the positions in the step's metadata."""
+
+    where = "mixer"
+
+    def __init__(self, spec, store, dtype):
+        self.head_dim, self.base = spec.head_dim, spec.base
+
+    def rotate(self, q, k, ctx):
+        hd = self.head_dim
+        i = torch.arange(0, hd, 2, device=q.device, dtype=torch.float64)
+        angle = ctx.positions.double().unsqueeze(1) * self.base ** (-i / hd)  # [tokens, pairs]
+        cos, sin = angle.cos().float()[:, None, :], angle.sin().float()[:, None, :]
+        for x in (q, k):
+            v = x.float().reshape(x.shape[0], -1, hd // 2, 2)
+            a, b = v[..., 0], v[..., 1]
+            x.copy_(torch.stack((a * cos - b * sin, a * sin + b * cos), dim=-1).reshape(x.shape[0], -1).to(x.dtype))
+
+
+def plain_turn(x, heads, hd, base, first=0):
+    """The same turn over a whole sequence whose first token stands at position `first`."""
+    T_ = x.shape[0]
+    angle = (first + np.arange(T_, dtype=np.float64))[:, None] * base ** (-np.arange(0, hd, 2, dtype=np.float64) / hd)
+    v = x.reshape(T_, heads, hd // 2, 2)
+    a, b = v[..., 0], v[..., 1]
+    c, s_ = np.cos(angle)[:, None, :], np.sin(angle)[:, None, :]
+    return np.stack((a * c - b * s_, a * s_ + b * c), axis=-1).reshape(T_, heads * hd)
+
+
+def turned_model(dtype):
+    """Two attention layers whose queries and keys are turned by position and no other position
+    encoding: layer 0 four query heads on two key/value heads of 32, layer 1 three heads of 16
+    with a window of 20 and another base."""
+    import dataclasses
+
+    from liyab_amd.config import HeadSpec, LayerSpec, ModelPlan, OrderEntry, TokenEmbeddingSpec
+    from liyab_amd.parts import register_position
+
+    register_position("toy_turn", TurnPositions)
+    d, V, P, eps = 64, 190, 180, 1e-5
+    rng = np.random.default_rng(41)
+    a0 = dataclasses.replace(attention_spec("a0", d, 4, 2, 32, 0.2), position=TurnSpec(32, 100.0))
+    a1 = dataclasses.replace(attention_spec("a1", d, 3, 3, 16, 0.3, window=20), position=TurnSpec(16, 10000.0))
+    layers = [LayerSpec(a0, ffn_spec("f0", d, 96, "gelu_tanh"), norm_spec("n0a", d, eps), norm_spec("n0b", d, eps)),
+              LayerSpec(a1, ffn_spec("f1", d, 80, "gelu_erf"), norm_spec("n1a", d, eps), norm_spec("n1b", d, eps))]
+    tw = {"emb": rand(rng, V, d, scale=0.5), **norm_tensors(rng, "nf", d), **attention_tensors(rng, "a0", d, 4, 2, 32),
+          **attention_tensors(rng, "a1", d, 3, 3, 16), **ffn_tensors(rng, "f0", d, 96), **ffn_tensors(rng, "f1", d, 80)}
+    for name in ("n0a", "n0b", "n1a", "n1b"):
+        tw.update(norm_tensors(rng, name, d))
+    if dtype == "bfloat16":
+        tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tw.items()}
+    plan = ModelPlan(architecture="toy_turned", width=d, vocab_size=V, max_positions=P,
+                     embedding=TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": T("emb")}),
+                     residual_position=None, layers=layers, order=[OrderEntry(0), OrderEntry(1)],
+                     final_norm=norm_spec("nf", d, eps), head=HeadSpec("lm_head", d, V, 1.0, {"weight": T("emb")}))
+    return plan, tw, dict(d=d, V=V, eps=eps)
+
+
+def turned_plain(tw, info, ids, first=0, turn=True):
+    eps = info["eps"]
+    rot = (lambda hd, base: (lambda x, heads: plain_turn(x, heads, hd, base, first))) if turn else (lambda hd, base: None)
+    x = f64(tw["emb"])[ids]
+    a, _ = plain_attention(plain_norm(x, tw, "n0a", eps), tw, "a0", 4, 2, 32, 0.2, rotate=rot(32, 100.0))
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n0b", eps), tw, "f0", "gelu_tanh")
+    a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 3, 3, 16, 0.3, window=20, rotate=rot(16, 10000.0))
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_erf")
+    return plain_norm(x, tw, "nf", eps) @ f64(tw["emb"]).T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_position_encoding_inside_attention(dtype):
+    """A position encoding that turns queries and keys, defined here, is given to the framework's
+    attention as a field of its spec: it is built from the position registry and applied between
+    the projection and the cache write, so a portion's keys are stored turned and later steps
+    find them so. The plain formula is pinned first: only distances count (all positions moved by
+    41 give the same logits), and without the turn the logits differ (the model has no other
+    position encoding, so the turn is what tells positions apart)."""
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = turned_model(dtype)
+    probe = tt.random_tokens(7, 50, info["V"])
+    base = turned_plain(tw, info, probe)
+    assert tt.rel_err(turned_plain(tw, info, probe, first=41), base) < 1e-9
+    assert tt.rel_err(turned_plain(tw, info, probe, turn=False), base) > 1e-2
+    reqs = {f"p{i}": tt.random_tokens(50 + i, n, info["V"]) for i, n in enumerate([45, 180, 3, 99])}
+    ref = {rid: turned_plain(tw, info, toks) for rid, toks in reqs.items()}
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3, 40))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=8))):
+        core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        assert all(b.mixer.position is not None for b in core.model.blocks)
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, TOL_TOY[dtype], f"turned toy {name} {dtype}", family="toy:turned")
         core.manager.check()
         assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
@@ -723,7 +837,7 @@ def test_split_streams_reach_parts_that_cannot_take_them(monkeypatch):
         core = EngineCore.from_plan(plan, tw, dtype="bfloat16", page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4,
                                     use_graphs=False)
         got = tt.run_schedule(core, steps)
-        tt.check_against_plain(got, reqs, ref, TOL["bfloat16"], f"toy with forced cuts, {name}")
+        tt.check_against_plain(got, reqs, ref, TOL_TOY["bfloat16"], f"toy with forced cuts, {name}")
         core.manager.check()
     assert 2 in cut and 1 in cut  # both ways were taken
 
