@@ -81,14 +81,19 @@ int liyab_cm_peak_in_use(void* h, int g) { return static_cast<CacheManager*>(h)-
 int liyab_cm_check(void* h) { return static_cast<CacheManager*>(h)->check(&g_error); }
 
 // -- a step's metadata --------------------------------------------------------------
-int liyab_step_shape(void* h, int n_seqs, const int* slots, const int* q_lens, const int* want_counts, int decode_q_len,
-                     int attn_tile, StepShape* out) {
-    return step_shape(*static_cast<CacheManager*>(h), n_seqs, slots, q_lens, want_counts, decode_q_len, attn_tile, out, &g_error);
+int liyab_step_shape(void* h, int n_seqs, const int* slots, const int* q_lens, const int* want_counts, StepShape* out) {
+    return step_shape(*static_cast<CacheManager*>(h), n_seqs, slots, q_lens, want_counts, out, &g_error);
 }
 int liyab_step_fill(void* h, const StepShape* shape, const int* slots, const int* q_lens, const int64_t* tokens,
-                    const int* want_counts, const int* wants, int vocab_size, int decode_q_len, int attn_tile, int32_t* block) {
-    return step_fill(*static_cast<CacheManager*>(h), *shape, slots, q_lens, tokens, want_counts, wants, vocab_size, decode_q_len,
-                     attn_tile, block, &g_error);
+                    const int* want_counts, const int* wants, int vocab_size, int32_t* block) {
+    return step_fill(*static_cast<CacheManager*>(h), *shape, slots, q_lens, tokens, want_counts, wants, vocab_size, block, &g_error);
+}
+// attention's own words of a step (step_meta.h): counts[0] tiles, counts[1] single rows
+void liyab_attn_counts(int n_seqs, const int* q_lens, int decode_q_len, int attn_tile, int* counts) {
+    attn_counts(n_seqs, q_lens, decode_q_len, attn_tile, &counts[0], &counts[1]);
+}
+void liyab_attn_fill(int n_seqs, const int* q_lens, const int* first_pos, int decode_q_len, int attn_tile, int32_t* words) {
+    attn_fill(n_seqs, q_lens, first_pos, decode_q_len, attn_tile, words);
 }
 
 // -- the scheduler --------------------------------------------------------------------

@@ -11,7 +11,7 @@ static Status fail(std::string* err, Status s, const std::string& msg) {
 }
 
 Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int* q_lens, const int* want_counts,
-                  int decode_q_len, int attn_tile, StepShape* out, std::string* err) {
+                  StepShape* out, std::string* err) {
     if (n_seqs <= 0) return fail(err, kInvalidArgument, "a step needs at least one item");
     if (m.n_groups() > kMaxGroups) return fail(err, kInvalidArgument, "more cache groups than a step's metadata holds");
     StepShape s{};
@@ -25,13 +25,6 @@ Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int
         s.n_logit_rows += want_counts[i];
         s.max_q_len = std::max(s.max_q_len, q_lens[i]);
         s.max_context = std::max(s.max_context, m.length(slots[i]) + q_lens[i]);
-    }
-    s.mode = s.max_q_len <= decode_q_len ? 0 : 1;
-    if (s.mode == 1) {
-        for (int i = 0; i < n_seqs; ++i) {
-            if (q_lens[i] <= decode_q_len) s.n_single += q_lens[i];
-            else s.n_tiles += (q_lens[i] + attn_tile - 1) / attn_tile;
-        }
     }
     int cur = 0;
     auto place = [&cur](int size) {
@@ -48,8 +41,6 @@ Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int
     s.off_state_slots = place(S);
     s.off_logit_rows = place(std::max(R, 1));
     s.off_logit_slots = place(std::max(R, 1));
-    s.off_attn_work = place(std::max(4 * s.n_tiles, 1));
-    s.off_attn_single = place(std::max(s.n_single, 1));
     for (int g = 0; g < s.n_groups; ++g) {
         s.off_block_tables[g] = place(S * s.max_blocks);
         s.off_slots[g] = place(N);
@@ -60,8 +51,7 @@ Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int
 }
 
 Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, const int* q_lens, const int64_t* tokens,
-                 const int* want_counts, const int* wants, int vocab_size, int decode_q_len, int attn_tile, int32_t* block,
-                 std::string* err) {
+                 const int* want_counts, const int* wants, int vocab_size, int32_t* block, std::string* err) {
     const int S = s.n_seqs, page = m.page_size(), W = s.max_blocks;
     int32_t* tok = block + s.off_token_ids;
     int32_t* pos = block + s.off_positions;
@@ -71,16 +61,7 @@ Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, co
     int32_t* row_slots = block + s.off_logit_slots;
     rows[0] = 0;
     row_slots[0] = 0;
-    block[s.off_attn_work] = 0;
-    block[s.off_attn_single] = 0;
-
-    struct Tile {
-        int seq, row, pos, count;
-    };
-    std::vector<Tile> tiles;
-    tiles.reserve(static_cast<size_t>(s.n_tiles));
-    int32_t* single = block + s.off_attn_single;
-    int n_single = 0, row0 = 0, r = 0;
+    int row0 = 0, r = 0;
     for (int i = 0; i < S; ++i) {
         const int first = m.length(slots[i]), n = q_lens[i];
         starts[i] = row0;
@@ -100,26 +81,9 @@ Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, co
             rows[r] = row0 + wants[r];
             row_slots[r] = slots[i];
         }
-        if (s.mode == 1) {
-            if (n <= decode_q_len) {
-                for (int j = 0; j < n; ++j) single[n_single++] = row0 + j;
-            } else {
-                for (int t0 = 0; t0 < n; t0 += attn_tile) tiles.push_back({i, row0 + t0, first + t0, std::min(attn_tile, n - t0)});
-            }
-        }
         row0 += n;
     }
     starts[S] = row0;
-    // a tile's work grows with its last position: the longest first, so that the short ones
-    // fill the gaps at the end
-    std::stable_sort(tiles.begin(), tiles.end(), [](const Tile& a, const Tile& b) { return a.pos + a.count > b.pos + b.count; });
-    int32_t* work = block + s.off_attn_work;
-    for (size_t t = 0; t < tiles.size(); ++t) {
-        work[4 * t] = tiles[t].seq;
-        work[4 * t + 1] = tiles[t].row;
-        work[4 * t + 2] = tiles[t].pos;
-        work[4 * t + 3] = tiles[t].count;
-    }
     for (int g = 0; g < s.n_groups; ++g) {
         int32_t* bt = block + s.off_block_tables[g];
         int32_t* sl = block + s.off_slots[g];
@@ -137,6 +101,49 @@ Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, co
         }
     }
     return kOk;
+}
+
+void attn_counts(int n_seqs, const int* q_lens, int decode_q_len, int attn_tile, int* n_tiles, int* n_single) {
+    int tiles = 0, single = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        if (q_lens[i] <= decode_q_len) single += q_lens[i];
+        else tiles += (q_lens[i] + attn_tile - 1) / attn_tile;
+    }
+    *n_tiles = tiles;
+    *n_single = single;
+}
+
+void attn_fill(int n_seqs, const int* q_lens, const int* first_pos, int decode_q_len, int attn_tile, int32_t* words) {
+    struct Tile {
+        int seq, row, pos, count;
+    };
+    int n_tiles = 0, n_single = 0;
+    attn_counts(n_seqs, q_lens, decode_q_len, attn_tile, &n_tiles, &n_single);
+    std::vector<Tile> tiles;
+    tiles.reserve(static_cast<size_t>(n_tiles));
+    int32_t* work = words;
+    int32_t* single = words + 4 * std::max(n_tiles, 1);
+    work[0] = work[1] = work[2] = work[3] = 0;
+    single[0] = 0;
+    int row0 = 0, k = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        const int n = q_lens[i], first = first_pos[i];
+        if (n <= decode_q_len) {
+            for (int j = 0; j < n; ++j) single[k++] = row0 + j;
+        } else {
+            for (int t0 = 0; t0 < n; t0 += attn_tile) tiles.push_back({i, row0 + t0, first + t0, std::min(attn_tile, n - t0)});
+        }
+        row0 += n;
+    }
+    // a tile's work grows with its last position: the longest first, so that the short ones
+    // fill the gaps at the end
+    std::stable_sort(tiles.begin(), tiles.end(), [](const Tile& a, const Tile& b) { return a.pos + a.count > b.pos + b.count; });
+    for (size_t t = 0; t < tiles.size(); ++t) {
+        work[4 * t] = tiles[t].seq;
+        work[4 * t + 1] = tiles[t].row;
+        work[4 * t + 2] = tiles[t].pos;
+        work[4 * t + 3] = tiles[t].count;
+    }
 }
 
 }  // namespace liyab_host

@@ -1,5 +1,10 @@
 // A step's metadata: one block of int32 words that goes to the device in one copy.
 //
+// The block here holds what every part may need of a step (tokens, positions, requests, block
+// tables, cache slots, wanted rows). What only one kind of part needs (attention's work lists,
+// further down) is that part's own: it is laid out behind this block by the step function, from
+// what the part's planner says, and goes to the device in the same copy.
+//
 // The batch is the reference's list of segments flattened (src/core/transformer.h:890-920):
 // rows are the items' tokens one after the other; a row's position is its request's length
 // before the step plus its index in the item (src/core/transformer.cpp:6689-6693).
@@ -17,25 +22,31 @@ constexpr int kMaxGroups = 16;
 // Sizes of a step and where each array starts in the block (offsets in words).
 struct StepShape {
     int n_tokens, n_seqs, n_logit_rows, n_groups, max_blocks;
-    int mode;        // 0: every request brings at most decode_q_len tokens; 1: some bring more
-    int n_tiles;     // attention tiles of the long portions (mode 1)
-    int n_single;    // rows of the short requests in a mode-1 step
     int max_q_len, max_context;
     int total;       // words in the block
     int off_token_ids, off_positions, off_tok_seq, off_seq_starts, off_context_lens, off_state_slots;
-    int off_logit_rows, off_logit_slots, off_attn_work, off_attn_single;
+    int off_logit_rows, off_logit_slots;
     int off_block_tables[kMaxGroups], off_slots[kMaxGroups];
 };
 
 // From the items' sizes alone (requests by slot, tokens each brings, logits each wants).
 Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int* q_lens, const int* want_counts,
-                  int decode_q_len, int attn_tile, StepShape* out, std::string* err);
+                  StepShape* out, std::string* err);
 
 // Fills the block. `tokens`: the items' token ids one after the other; an id < 0 stands for "the
 // token sampled for slot -1 - id, still on the device". `wants`: places within each item.
 // Pages of every position the step touches must be mapped (reserve comes first).
 Status step_fill(const CacheManager& m, const StepShape& shape, const int* slots, const int* q_lens, const int64_t* tokens,
-                 const int* want_counts, const int* wants, int vocab_size, int decode_q_len, int attn_tile, int32_t* block,
-                 std::string* err);
+                 const int* want_counts, const int* wants, int vocab_size, int32_t* block, std::string* err);
+
+// Attention's own words of a step in which some request brings more than decode_q_len tokens:
+// the long portions cut into tiles of up to attn_tile consecutive queries (4 words a tile: request
+// index, first row, first position, queries; the tile that ends at the latest position first, so
+// that the short ones fill the gaps at the end), and the rows of the short portions, which are
+// attended one by one. attn_counts gives (tiles, single rows); attn_fill writes 4 * max(tiles, 1)
+// words of tiles followed by max(single rows, 1) words of rows. first_pos: each request's length
+// before the step.
+void attn_counts(int n_seqs, const int* q_lens, int decode_q_len, int attn_tile, int* n_tiles, int* n_single);
+void attn_fill(int n_seqs, const int* q_lens, const int* first_pos, int decode_q_len, int attn_tile, int32_t* words);
 
 }  // namespace liyab_host

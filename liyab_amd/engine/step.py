@@ -30,7 +30,7 @@ from .. import host
 from ..cache.pages import CacheManager
 from ..cache.storage import CacheStorage
 from ..errors import InvalidArgument
-from ..parts.base import GroupStep, StepContext, StepHost, Workspace
+from ..parts.base import GroupStep, StepContext, StepFacts, StepHost, Workspace
 
 
 @dataclass
@@ -74,34 +74,15 @@ class _Staging:
         ev.record()
 
 
-ATTN_TILE = 128  # queries of one request that the prefill attention kernel takes together (64 or 128)
-ATTN_TILE_FEW = 64  # the same for steps whose long portions hold few tokens: more, shorter tiles
-ATTN_FEW_TOKENS = 1024  # up to this many tokens in long portions (measured: a step of 256 tokens of one prompt 840 -> 806 us)
-
-
-def attn_tile_for(q_lens) -> int:
-    """The query tile of a step's prefill attention. With few tokens in long portions the tiles
-    are few, and the longest walk over a request's keys is the whole kernel: tiles of 64
-    queries are twice as many, and four waves instead of two share each walk."""
-    long_tokens = int(sum(int(q) for q in q_lens if q > DECODE_Q_LEN))
-    return ATTN_TILE_FEW if long_tokens <= ATTN_FEW_TOKENS else ATTN_TILE
-GRAPH_AFTER_MIXED = 3  # eager runs of a shape with prompt portions before it is captured
-DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
-
-
-def _bucket(n: int, least: int = 256) -> int:
-    b = least
-    while b < n:
-        b *= 2
-    return b
+GRAPH_AFTER_MIXED = 3  # eager runs of a shape that its parts do not expect to recur before it is captured
 
 
 class StepFunction:
-    """`use_graphs`: a step whose shape (tokens, requests, wanted rows, attention mode,
-    context bucket) has been seen before is captured into a HIP graph the second time and
-    replayed from then on; what varies between such steps lives in the metadata block, whose
-    address and layout the shape fixes. Kernels must then depend on the host only through
-    the shape: the ones in this package do."""
+    """`use_graphs`: a step whose shape (tokens, requests, wanted rows, and the key of every
+    part's step planner: attention's mode, context bucket and tiles) has been seen before is
+    captured into a HIP graph the second time and replayed from then on; what varies between
+    such steps lives in the metadata block, whose address and layout the shape fixes. Kernels
+    must then depend on the host only through the shape: the ones in this package do."""
 
     def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0", use_graphs: bool = True,
                  max_graphs: int = 256):
@@ -121,6 +102,9 @@ class StepFunction:
         self._graph_generation = 0
         self.last_tokens = torch.zeros(manager.max_requests, dtype=torch.int32, device=self.device)
         self.last_context: Optional[StepContext] = None
+        self.planners = list(getattr(model, "step_planners", ()))
+        self._key = None  # the prepared step's shape: what its captured graph is kept under
+        self._recurs = True
 
     # -- validation -----------------------------------------------------------
     def _validate(self, items: Sequence[StepItem]) -> None:
@@ -151,8 +135,7 @@ class StepFunction:
             # a workspace buffer moved since the graphs were captured: they hold its old address
             self._graphs.clear()
             self._graph_generation = self.workspace.generation
-        key = (ctx.n_tokens, ctx.n_seqs, ctx.n_logit_rows, ctx.host.attention_mode, ctx.host.context_bucket,
-               ctx.host.n_attn_tiles, ctx.host.attn_tile, ctx.host.n_attn_single)
+        key = self._key
         entry = self._graphs.pop(key, None)
         if entry is not None:
             self._graphs[key] = entry  # back in as the most recently used (a dict keeps insertion order)
@@ -173,7 +156,7 @@ class StepFunction:
         # A decode-only shape comes back step after step: captured at its second sight. A mix of
         # prompt portions and decoded tokens mostly does not, and a capture costs about two eager
         # runs: captured only once it has shown that it recurs.
-        if entry < (1 if ctx.host.attention_mode == "decode" else GRAPH_AFTER_MIXED):
+        if entry < (1 if self._recurs else GRAPH_AFTER_MIXED):
             self._graphs[key] = entry + 1
             return self.model.forward(ctx, self.storage)
         before = self.workspace.generation
@@ -246,15 +229,28 @@ class StepFunction:
         lib = host.lib()
         shape = host.StepShape()
         ip = lambda a: a.ctypes.data_as(host.IP)  # noqa: E731
-        attn_tile = attn_tile_for(q_lens)
-        host.check(lib.liyab_step_shape(mgr.handle, S, ip(slots), ip(q_lens), ip(want_counts), DECODE_Q_LEN, attn_tile,
-                                        ctypes.byref(shape)))
+        host.check(lib.liyab_step_shape(mgr.handle, S, ip(slots), ip(q_lens), ip(want_counts), ctypes.byref(shape)))
+        # the parts' own words stand behind the common block; their keys join the step's shape
+        first_pos = (new_lengths - q_lens).astype(np.intc, copy=False)
         total = shape.total
+        plans = []
+        if self.planners:
+            facts = StepFacts(n_tokens=N, n_seqs=S, q_lens=q_lens, first_pos=first_pos, state_slots=slots,
+                              max_q_len=shape.max_q_len, max_context=shape.max_context, page_size=mgr.page_size)
+            for planner in self.planners:
+                p = planner.plan(facts)
+                plans.append((planner.name, p, total))
+                total += p.n_words
+        self._key = (N, S, R) + tuple((name, p.key, p.n_words) for name, p, _ in plans)
+        self._recurs = all(p.recurs for _, p, _ in plans)
         host_t = self._staging.next(total)
+        base = ctypes.cast(host_t.data_ptr(), ctypes.POINTER(ctypes.c_int32))
         host.check(lib.liyab_step_fill(mgr.handle, ctypes.byref(shape), ip(slots), ip(q_lens),
                                        all_tokens.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), ip(want_counts), ip(wants),
-                                       self.model.vocab_size, DECODE_Q_LEN, attn_tile,
-                                       ctypes.cast(host_t.data_ptr(), ctypes.POINTER(ctypes.c_int32))))
+                                       self.model.vocab_size, base))
+        for _, p, off in plans:
+            if p.n_words:
+                p.fill(ctypes.cast(host_t.data_ptr() + 4 * off, ctypes.POINTER(ctypes.c_int32)))
 
         if self._meta_dev is None or self._meta_dev.numel() < total:
             # sized for the largest step of this engine's lifetime where possible: a new block
@@ -266,7 +262,6 @@ class StepFunction:
         self._staging.copied()
 
         W, G, page = shape.max_blocks, shape.n_groups, mgr.page_size
-        prefill = shape.mode == 1
         starts = np.cumsum(q_lens) - q_lens
         ctx = StepContext(
             n_tokens=N, n_seqs=S,
@@ -279,13 +274,11 @@ class StepFunction:
             logit_rows=dev[shape.off_logit_rows:shape.off_logit_rows + max(R, 1)], n_logit_rows=R,
             groups=[GroupStep(block_tables=dev[shape.off_block_tables[g]:shape.off_block_tables[g] + S * W].view(S, W),
                               slots=dev[shape.off_slots[g]:shape.off_slots[g] + N]) for g in range(G)],
-            host=StepHost(q_lens=q_lens.tolist(), starts=starts.tolist(), first_pos=(new_lengths - q_lens).tolist(),
-                          max_q_len=shape.max_q_len, max_context=shape.max_context,
-                          attention_mode="prefill" if prefill else "decode", context_bucket=_bucket(shape.max_context),
-                          n_attn_tiles=shape.n_tiles, attn_tile=attn_tile, n_attn_single=shape.n_single),
+            host=StepHost(q_lens=q_lens.tolist(), starts=starts.tolist(), first_pos=first_pos.tolist(),
+                          max_q_len=shape.max_q_len, max_context=shape.max_context),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,
             logit_slots=dev[shape.off_logit_slots:shape.off_logit_slots + max(R, 1)], last_tokens=self.last_tokens,
-            attn_work=dev[shape.off_attn_work:shape.off_attn_work + max(4 * shape.n_tiles, 1)] if prefill else None,
-            attn_single_rows=dev[shape.off_attn_single:shape.off_attn_single + max(shape.n_single, 1)] if prefill else None,
+            plans={name: (p.make(dev[off:off + p.n_words] if p.n_words else None) if p.make is not None else None)
+                   for name, p, off in plans},
         )
         return ctx, (slots, new_lengths)

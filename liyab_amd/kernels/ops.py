@@ -787,15 +787,19 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
               block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0,
               splits_ok: bool = False) -> Optional[torch.Tensor]:
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
-    is chosen from the step's shape (`ctx` is the step's StepContext). With `splits_ok`, a
-    step of few tokens may leave `out` unwritten and return the splits of each (token, head)
-    pair instead, float32 [tokens, heads, splits, head size + 4], for `gemm_att_parts`."""
+    is chosen from the step's shape (`ctx` is the step's StepContext; `ctx.plans["attention"]`
+    says how the step's tokens are cut, see parts/attention.py; without it every token goes to
+    the plain kernel). With `splits_ok`, a step of few tokens may leave `out` unwritten and
+    return the splits of each (token, head) pair instead, float32 [tokens, heads, splits, head
+    size + 4], for `gemm_att_parts`."""
     hd = k_cache.shape[3]
     host = ctx.host
-    fast = q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0 and out.stride(0) % 8 == 0
+    plan = ctx.plans.get("attention")
+    fast = (plan is not None and q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0
+            and out.stride(0) % 8 == 0)
 
     def decode(tok_list, n):
-        splits, waves = decode_plan(n, n_head, host.context_bucket)
+        splits, waves = decode_plan(n, n_head, plan.context_bucket)
         partials = None
         if splits > 1:
             partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32)
@@ -804,9 +808,9 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
                          rows_are_requests=tok_list is None and host.max_q_len == 1)
 
-    if fast and host.attention_mode == "decode" and block_tables.shape[1] <= 2048:
+    if fast and plan.mode == "decode" and block_tables.shape[1] <= 2048:
         n = out.shape[0]
-        splits, waves = decode_split_plan(n, n_head, host.context_bucket) if splits_ok else (1, 4)
+        splits, waves = decode_split_plan(n, n_head, plan.context_bucket) if splits_ok else (1, 4)
         if splits > 1 and att_parts_takes(n, splits, hd):
             partials = ctx.workspace.get("attn_partials", (n, n_head, splits, hd + 4), torch.float32)
             attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
@@ -815,17 +819,17 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
             return partials
         decode(None, n)
         return None
-    if fast and prefill_takes(hd) and scale > 0 and ctx.attn_work is not None and block_tables.shape[1] <= 2048:
+    if fast and plan.mode == "prefill" and prefill_takes(hd) and scale > 0 and block_tables.shape[1] <= 2048:
         # long portions in tiles on the matrix cores, the short ones token by token
-        if host.n_attn_tiles:
+        if plan.n_tiles:
             # with fewer workgroups than compute units, two waves share each query group's keys:
             # the longest tile's walk over its keys is then the kernel's critical path, and halves
-            work = host.n_attn_tiles * n_head
-            ksplit = (4 if host.attn_tile == 64 and hd <= 64 and work <= PREFILL_KSPLIT4_WORK else 2) if work <= 256 else 1
-            attention_prefill(out, q, k_cache, v_cache, block_tables, ctx.attn_work, host.n_attn_tiles, n_head=n_head,
-                              scale=scale, window=window, tile=host.attn_tile, ksplit=ksplit)
-        if host.n_attn_single:
-            decode(ctx.attn_single_rows, host.n_attn_single)
+            work = plan.n_tiles * n_head
+            ksplit = (4 if plan.tile == 64 and hd <= 64 and work <= PREFILL_KSPLIT4_WORK else 2) if work <= 256 else 1
+            attention_prefill(out, q, k_cache, v_cache, block_tables, plan.work, plan.n_tiles, n_head=n_head,
+                              scale=scale, window=window, tile=plan.tile, ksplit=ksplit)
+        if plan.n_single:
+            decode(plan.single_rows, plan.n_single)
         return
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)

@@ -43,6 +43,13 @@ class DecoderModel:
         self.final_norm = build_part("norm", plan.final_norm, store, dtype) if plan.final_norm is not None else None
         self.head = build_part("head", plan.head, store, dtype)
         self.order = list(plan.order)
+        # the parts' step planners, one of each name (every attention layer shares attention's)
+        self.step_planners = []
+        for block in self.blocks:
+            for part in (getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn")):
+                planner = getattr(part, "step_planner", None)
+                if planner is not None and all(p.name != planner.name for p in self.step_planners):
+                    self.step_planners.append(planner)
         for e in self.order:
             if not (0 <= e.layer < len(self.blocks)) or not (0 <= e.cache_layer < len(self.blocks)):
                 raise ValueError(f"the run order names layer {e.layer} / cache of {e.cache_layer}; the model has {len(self.blocks)}")

@@ -1,6 +1,6 @@
 """Model parts: mixers, feed-forwards, norms, position encodings, blocks."""
 
-from .base import GroupStep, StepContext, StepHost, Workspace  # noqa: F401
+from .base import GroupStep, PartStepPlan, StepContext, StepFacts, StepHost, Workspace  # noqa: F401
 from .registry import (  # noqa: F401
     build_part,
     find_part,

@@ -2,17 +2,90 @@
 
 from __future__ import annotations
 
+import ctypes
+from dataclasses import dataclass
 from typing import Optional
 
 import torch
 
+from .. import host
 from ..cache.pages import KVSpec
 from ..cache.storage import LayerCache
 from ..errors import Unsupported
 from ..kernels import ops
-from .base import StepContext, settled
+from .base import PartStepPlan, StepContext, StepFacts, settled
 from .linear import linear, linear_deferred, paged_qkv_takes
 from .registry import build_part, register_mixer
+
+
+ATTN_TILE = 128  # queries of one request that the prefill attention kernel takes together (64 or 128)
+ATTN_TILE_FEW = 64  # the same for steps whose long portions hold few tokens: more, shorter tiles
+ATTN_FEW_TOKENS = 1024  # up to this many tokens in long portions (measured: a step of 256 tokens of one prompt 840 -> 806 us)
+DECODE_Q_LEN = 8  # requests that bring at most this many tokens are attended token by token
+
+
+def attn_tile_for(q_lens) -> int:
+    """The query tile of a step's prefill attention. With few tokens in long portions the tiles
+    are few, and the longest walk over a request's keys is the whole kernel: tiles of 64
+    queries are twice as many, and four waves instead of two share each walk."""
+    long_tokens = int(sum(int(q) for q in q_lens if q > DECODE_Q_LEN))
+    return ATTN_TILE_FEW if long_tokens <= ATTN_FEW_TOKENS else ATTN_TILE
+
+
+def _bucket(n: int, least: int = 256) -> int:
+    b = least
+    while b < n:
+        b *= 2
+    return b
+
+
+@dataclass
+class AttentionStep:
+    """How a step's tokens are attended, decided once a step for every attention layer.
+    "decode": every request brings few tokens, each taken on its own. "prefill": the long
+    portions in tiles of up to `tile` queries on the matrix cores (`work`: int32 [n_tiles, 4] on
+    the device = request index, first row, first position, queries), the short ones' rows
+    (`single_rows`: int32 [n_single]) token by token. Grids follow `context_bucket` (the longest
+    context rounded up to a power of two), not the exact length."""
+
+    mode: str
+    context_bucket: int
+    n_tiles: int = 0
+    tile: int = ATTN_TILE
+    n_single: int = 0
+    work: Optional[torch.Tensor] = None
+    single_rows: Optional[torch.Tensor] = None
+
+
+class AttentionStepPlanner:
+    """Attention's words of a step's metadata and its term of the graph key: the reference cuts a
+    pass's attention into per-segment work the same way, on the host, before its kernels run
+    (src/core/transformer.cpp:2169-2174, 2396-2452). The lists are laid out natively
+    (csrc/host/step_meta.cpp: attn_counts, attn_fill)."""
+
+    name = "attention"
+
+    def plan(self, facts: StepFacts) -> PartStepPlan:
+        bucket = _bucket(facts.max_context)
+        if facts.max_q_len <= DECODE_Q_LEN:
+            return PartStepPlan(key=("decode", bucket), make=lambda words: AttentionStep("decode", bucket))
+        lib = host.lib()
+        tile = attn_tile_for(facts.q_lens)
+        counts = (ctypes.c_int * 2)()
+        q_lens, first_pos, S = facts.q_lens, facts.first_pos, facts.n_seqs
+        lib.liyab_attn_counts(S, q_lens.ctypes.data_as(host.IP), DECODE_Q_LEN, tile, counts)
+        n_tiles, n_single = counts[0], counts[1]
+        n_work = 4 * max(n_tiles, 1)
+
+        def fill(address) -> None:
+            lib.liyab_attn_fill(S, q_lens.ctypes.data_as(host.IP), first_pos.ctypes.data_as(host.IP), DECODE_Q_LEN, tile, address)
+
+        def make(words) -> AttentionStep:
+            return AttentionStep("prefill", bucket, n_tiles, tile, n_single, words[:n_work], words[n_work:])
+
+        # a mix of prompt portions mostly does not come back the same
+        return PartStepPlan(key=("prefill", bucket, n_tiles, tile, n_single), n_words=n_work + max(n_single, 1), fill=fill,
+                            make=make, recurs=False)
 
 
 class Attention:
@@ -64,6 +137,7 @@ class Attention:
         return None
 
     defers = True  # forward(..., defer=True) takes the stream split or whole and may hand it back split
+    step_planner = AttentionStepPlanner()  # one plan a step for every attention layer: ctx.plans["attention"]
 
     def forward(self, h: torch.Tensor, ctx: StepContext, cache: LayerCache, state, residual: torch.Tensor,
                 writes_cache: bool = True, defer: bool = False):

@@ -17,6 +17,14 @@ to a class constructed as `cls(spec, store, dtype)`):
   position:  where == "residual": add(ctx, x);  fused_table() -> table | None
   block:     cls(layer_spec, mixer, ffn, norm_mixer, norm_ffn); forward(x, ctx, cache, state, writes_cache)
 
+A part that needs facts of a step laid out for its kernels (work lists, chunk tables), or whose
+launches depend on more of the step than its sizes, has a class attribute `step_planner`: an
+object with a `name` and `plan(facts: StepFacts) -> PartStepPlan`, called once a step for all
+parts that share the name. Its words go to the device with the step's metadata, its key
+becomes a term of the key under which the step's HIP graph is kept, and what its `make`
+returns is handed to the parts as `ctx.plans[name]`. Attention's tiles are planned so
+(`parts/attention.py`).
+
 Optional, and only between parts that declare them: a mixer or feed-forward with `defers`
 may be handed the stream as a `SplitStream` and may return one instead of adding in place;
 a norm with `takes_planes` reads a split stream's planes; a block with `takes_pending` gets
@@ -30,8 +38,9 @@ projection fold the addition into its epilogue.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Any, Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -110,11 +119,41 @@ class StepHost:
     first_pos: List[int]  # position of each request's first token
     max_q_len: int
     max_context: int  # longest context after this step
-    attention_mode: str = "prefill"  # "decode": every request brings few tokens, each taken on its own
-    context_bucket: int = 256  # max_context rounded up to a power of two: grids follow it, not the exact length
-    n_attn_tiles: int = 0  # prefill mode: tiles of up to attn_tile queries of the long portions
-    attn_tile: int = 128
-    n_attn_single: int = 0  # prefill mode: tokens of short portions, attended one by one
+
+
+@dataclass
+class StepFacts:
+    """What a part's step planner sees of a step, on the host, before anything is launched."""
+
+    n_tokens: int
+    n_seqs: int
+    q_lens: np.ndarray  # intc [n_seqs]: tokens each request brings
+    first_pos: np.ndarray  # intc [n_seqs]: each request's length before the step
+    state_slots: np.ndarray  # intc [n_seqs]
+    max_q_len: int
+    max_context: int
+    page_size: int
+
+
+@dataclass
+class PartStepPlan:
+    """What a part's planner decides for one step.
+
+    `key`: everything the part's launches (kernels chosen, grids, scalar arguments) depend on
+    besides the step's sizes (tokens, requests, wanted rows); two steps with equal sizes and
+    equal keys of all planners replay one captured graph, so whatever else varies must reach
+    the kernels through `words`. `n_words` int32 words go to the device behind the step's
+    common metadata in the same copy; `fill(address)` writes them into pinned host memory
+    (a `ctypes` pointer to int32); their count must be a function of the key. `make(words)`
+    (words: the int32 device tensor of n_words, or None) returns what parts find in
+    `ctx.plans[name]`. `recurs`: whether a step of this kind tends to come back the same
+    (decode steps do; a mix of prompt portions mostly does not, and is captured later)."""
+
+    key: Hashable
+    n_words: int = 0
+    fill: Optional[Callable[[Any], None]] = None
+    make: Optional[Callable[[Optional[torch.Tensor]], Any]] = None
+    recurs: bool = True
 
 
 @dataclass
@@ -136,5 +175,4 @@ class StepContext:
     page_size: int
     logit_slots: Optional[torch.Tensor] = None  # int32 [n_rows]: state slot of each wanted row's request
     last_tokens: Optional[torch.Tensor] = None  # int32 [slots]: the token each request drew last (on the device)
-    attn_work: Optional[torch.Tensor] = None  # int32 [n_attn_tiles, 4]: request index, first row, first position, queries
-    attn_single_rows: Optional[torch.Tensor] = None  # int32 [n_attn_single]: rows attended one by one
+    plans: Dict[str, Any] = field(default_factory=dict)  # what each part's step planner made for this step, by its name

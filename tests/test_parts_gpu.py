@@ -774,6 +774,147 @@ def test_toy_position_encoding_inside_attention(dtype):
         assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
 
+# ---------------------------------------------------------------------------
+# a toy mixer that brings its own words of a step's metadata, under graphs and the scheduler
+# ---------------------------------------------------------------------------
+class ScanPlanner:
+    """For each token, how many steps of the recurrence lie between the request's stored state
+    and it (its index in the portion plus one): words of the toy mixer's own, filled on the host
+    and read on the device. Nothing of them enters the key: they vary freely between replays."""
+
+    name = "toy_scan"
+    calls = 0
+
+    def plan(self, facts):
+        from liyab_amd.parts import PartStepPlan
+
+        ScanPlanner.calls += 1
+        since = np.concatenate([np.arange(1, int(n) + 1, dtype=np.int32) for n in facts.q_lens])
+
+        def fill(address):
+            import ctypes
+
+            ctypes.memmove(address, since.ctypes.data, since.nbytes)
+
+        return PartStepPlan(key=(), n_words=int(since.size), fill=fill, make=lambda words: words)
+
+
+class PlannedDecayMixer:
+    """The decay mixer again (s_t = decay * s_{t-1} + h_t, out = s_t . W^T), written so that a
+    captured graph can replay it: nothing is read on the host; which request a token belongs to,
+    where a request's rows end and its state slot come from the step's common metadata, and the
+    distance to the stored state from the words its own planner contributes."""
+
+    step_planner = ScanPlanner()
+
+    def __init__(self, spec, store, dtype):
+        from liyab_amd.config import TensorSource
+
+        self.width, self.decay = spec.width, spec.decay
+        self.weight = store.fetch(TensorSource(spec.prefix + ".w"), (spec.width, spec.width), "matrix")
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        from liyab_amd.cache import StateSpec
+
+        return StateSpec((self.width,), "float32")
+
+    def forward(self, h, ctx, cache, state, residual, writes_cache=True):
+        from liyab_amd.parts import as_tensor
+
+        h = as_tensor(h).float()
+        n = h.shape[0]
+        since = ctx.plans["toy_scan"].long()  # [tokens]
+        seq = ctx.tok_seq.long()
+        rows = torch.arange(n, device=h.device)
+        gap = rows[:, None] - rows[None, :]
+        mask = (seq[:, None] == seq[None, :]) & (gap >= 0)
+        w = torch.pow(self.decay, gap.clamp(min=0).double()) * mask
+        slots = ctx.state_slots.long()[seq]  # each token's request's slot
+        carried = torch.pow(self.decay, since.double())[:, None] * state[slots].double()
+        s = (w @ h.double() + carried).float()
+        ends = ctx.seq_starts.long()[1:] - 1  # each request's last row
+        state.index_copy_(0, ctx.state_slots.long(), s[ends])
+        residual += s @ self.weight.float().t()
+
+
+def planned_model():
+    from liyab_amd.config import LayerSpec, OrderEntry
+    from liyab_amd.parts import register_mixer
+
+    register_mixer("toy_decay_planned", PlannedDecayMixer)
+    d, V, P, eps = 48, 97, 120, 1e-5
+    rng = np.random.default_rng(61)
+
+    class Spec(DecaySpec):
+        kind = "toy_decay_planned"
+
+    layers = [LayerSpec(Spec(d, 0.7, "m0"), ffn_spec("f0", d, 64, "gelu_tanh"), norm_spec("n0a", d, eps), norm_spec("n0b", d, eps)),
+              LayerSpec(attention_spec("a1", d, 3, 3, 16, 0.25), ffn_spec("f1", d, 72, "gelu_erf"), norm_spec("n1a", d, eps), norm_spec("n1b", d, eps)),
+              LayerSpec(Spec(d, 0.9, "m2"), None, norm_spec("n2a", d, eps), None)]
+    tw = {"emb": rand(rng, V, d, scale=0.5), "pos": rand(rng, P, d, scale=0.3), **norm_tensors(rng, "nf", d),
+          "m0.w": rand(rng, d, d, scale=0.05), "m2.w": rand(rng, d, d, scale=0.05), **attention_tensors(rng, "a1", d, 3, 3, 16),
+          **ffn_tensors(rng, "f0", d, 64), **ffn_tensors(rng, "f1", d, 72)}
+    for name in ("n0a", "n0b", "n1a", "n1b", "n2a"):
+        tw.update(norm_tensors(rng, name, d))
+    return make_plan(d, V, P, layers, [OrderEntry(0), OrderEntry(1), OrderEntry(2)], eps), tw, dict(d=d, V=V, P=P, eps=eps)
+
+
+def planned_plain(tw, info, ids):
+    eps, d = info["eps"], info["d"]
+
+    def decay(h, rate, w):
+        s, out = np.zeros(d), np.zeros_like(h)
+        for t in range(len(h)):
+            s = rate * s + h[t]
+            out[t] = s
+        return out @ f64(tw[w]).T
+
+    x = f64(tw["emb"])[ids] + f64(tw["pos"])[:len(ids)]
+    x = x + decay(plain_norm(x, tw, "n0a", eps), 0.7, "m0.w")
+    x = x + plain_ffn(plain_norm(x, tw, "n0b", eps), tw, "f0", "gelu_tanh")
+    a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 3, 3, 16, 0.25)
+    x = x + a
+    x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_erf")
+    x = x + decay(plain_norm(x, tw, "n2a", eps), 0.9, "m2.w")
+    return plain_norm(x, tw, "nf", eps) @ f64(tw["emb"]).T
+
+
+def test_a_part_with_its_own_step_metadata_runs_under_graphs_and_the_scheduler():
+    """A mixer defined here keeps state of its own and has a step planner of its own: its words
+    ride behind the step's common metadata, one plan a step serves both of its layers, and since
+    nothing it does depends on the host it is captured and replayed like the framework's parts.
+    Driven by the scheduler (portions of prompts beside decoding requests, a pool so small that
+    a request is preempted and its state starts again from zero), its greedy tokens are the
+    plain model's."""
+    from liyab_amd import Engine, SamplingParams
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = planned_model()
+    prompts = [tt.random_tokens(70 + i, n, info["V"]) for i, n in enumerate([30, 5, 41, 17])]
+    core = EngineCore.from_plan(plan, tw, dtype="float32", page_size=8, num_pages=14, max_requests=3, use_graphs=True)
+    assert [p.name for p in core.model.step_planners] == ["toy_scan", "attention"]
+    ScanPlanner.calls = 0
+    engine = Engine(core=core, max_num_seqs=3, max_batched_tokens=24, prefill_chunk=16)
+    engine.stop_at_eos = False
+    results = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=30))
+    assert ScanPlanner.calls == core.step_fn.steps  # once a step, not once a layer
+    assert core.step_fn.graph_replays > 0
+    assert any(term[0] == "toy_scan" for key in core.step_fn._graphs for term in key[3:])
+    assert engine.scheduler.stats.preemptions >= 1
+    for prompt, res in zip(prompts, results):
+        ids, want = list(prompt), []
+        for _ in range(30):
+            nxt = int(np.argmax(planned_plain(tw, info, ids)[-1].astype(np.float32)))
+            want.append(nxt)
+            ids.append(nxt)
+        assert res.tokens == want
+    core.manager.check()
+    assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
+
+
 class BareNorm:
     """A LayerNorm that knows nothing of split streams or pending norms (no `takes_planes`, no `lazy`)."""
 

@@ -50,7 +50,7 @@ def test_what_the_folded_norm_takes(ops):
 def test_attention_tile_of_a_step():
     """Steps whose long portions hold few tokens take query tiles of 64, others of 128; short
     portions (taken token by token) do not count."""
-    from liyab_amd.engine import step
+    from liyab_amd.parts import attention as step
 
     assert step.attn_tile_for([1, 1, 1]) == step.ATTN_TILE_FEW
     assert step.attn_tile_for([256, 1, 8]) == step.ATTN_TILE_FEW
@@ -58,3 +58,38 @@ def test_attention_tile_of_a_step():
     assert step.attn_tile_for([1024, 9]) == step.ATTN_TILE
     assert step.attn_tile_for([1024, 1024]) == step.ATTN_TILE
     assert step.attn_tile_for([1024] + [8] * 40) == step.ATTN_TILE_FEW
+
+
+def test_attention_plans_its_own_words_of_a_step():
+    """Attention's planner: a step of single tokens needs no words and is keyed by the context's
+    bucket; a step with long portions gets its tiles (the one that ends latest first) and the
+    short portions' rows, laid out natively, and a key that fixes their counts."""
+    import ctypes
+
+    import numpy as np
+
+    from liyab_amd.parts import StepFacts
+    from liyab_amd.parts.attention import Attention, AttentionStepPlanner
+
+    planner = Attention.step_planner
+    assert isinstance(planner, AttentionStepPlanner) and planner.name == "attention"
+
+    def facts(q_lens, first):
+        q = np.array(q_lens, dtype=np.intc)
+        f = np.array(first, dtype=np.intc)
+        return StepFacts(n_tokens=int(q.sum()), n_seqs=len(q), q_lens=q, first_pos=f, state_slots=np.arange(len(q), dtype=np.intc),
+                         max_q_len=int(q.max()), max_context=int((q + f).max()), page_size=16)
+
+    p = planner.plan(facts([1, 8, 3], [300, 10, 0]))
+    assert p.key == ("decode", 512) and p.n_words == 0 and p.recurs and p.make(None).mode == "decode"
+    p = planner.plan(facts([100, 2, 70, 9], [0, 40, 200, 5]))
+    # tiles of 64: 100 -> 64 + 36, 70 -> 64 + 6, 9 -> 9; the short one's two rows are taken one by one
+    assert p.key == ("prefill", 512, 5, 64, 2) and p.n_words == 4 * 5 + 2 and not p.recurs
+    words = np.full(p.n_words, -7, dtype=np.int32)
+    p.fill(words.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+    tiles = words[:20].reshape(5, 4).tolist()
+    # (request, first row, first position, queries), ordered by the position a tile ends at
+    assert tiles == [[2, 166, 264, 6], [2, 102, 200, 64], [0, 64, 64, 36], [0, 0, 0, 64], [3, 172, 5, 9]]
+    assert words[20:].tolist() == [100, 101]
+    # the same sizes cut another way give the same key when they fall into the same tiles
+    assert planner.plan(facts([90, 2, 80, 9], [10, 40, 190, 5])).key == p.key
