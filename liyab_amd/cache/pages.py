@@ -41,15 +41,26 @@ def _ip(a: np.ndarray):
 
 @dataclass(frozen=True)
 class KVSpec:
-    """What an attention-like mixer needs of the cache."""
+    """What a mixer that keeps rows per position needs of the cache: pages of `rows`, each a
+    named plane `(name, heads, width)` stored as [pages, heads, page_size, width]. Attention keeps
+    keys and values of one shape, which is what `rows` is when it is left empty: ("k", n_kv_head,
+    head_dim) and ("v", n_kv_head, head_dim). A mixer with rows of other widths, or with one
+    compressed row a position instead of a key and a value, names its own planes (the reference
+    pads every layer's rows to its widest instead, src/core/transformer.cpp:2875-2890)."""
 
     n_kv_head: int
     head_dim: int
     window: int = 0  # 0: every position is kept; W > 0: only the last W are read
+    rows: Tuple[Tuple[str, int, int], ...] = ()
 
     @property
-    def key(self) -> Tuple[int, int, int]:
-        return (self.n_kv_head, self.head_dim, self.window)
+    def planes(self) -> Tuple[Tuple[str, int, int], ...]:
+        return self.rows or (("k", self.n_kv_head, self.head_dim), ("v", self.n_kv_head, self.head_dim))
+
+    @property
+    def key(self) -> tuple:
+        """Layers with equal keys share a group: the same pages, one block table a request."""
+        return (self.planes, self.window)
 
 
 @dataclass(frozen=True)

@@ -43,6 +43,8 @@ def build_parser() -> argparse.ArgumentParser:
                     help="precision of the whole path (default bfloat16)")
     ap.add_argument("--json", action="store_true", help="stdout: one JSON line after loading and one for the generation")
     ap.add_argument("--tokenize", action="store_true", help="print the prompt's token ids and exit")
+    ap.add_argument("--phases", action="store_true",
+                    help="time the device per phase of the forward pass (phases_ms in --json, ms per token on stderr); slower: no graphs")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
     ap.add_argument("--num-pages", type=int, default=None, help="pages in the pool (default: enough for every slot)")
@@ -95,8 +97,10 @@ def main(argv=None) -> int:
     try:
         engine = Engine(model_dir, dtype=args.dtype, device=args.device, page_size=args.page_size,
                         num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
-                        max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk, ctx=args.ctx)
+                        max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk, ctx=args.ctx,
+                        phases=args.phases)
         engine.warmup()  # kernels' code loaded here, not inside the first turn's time to first token
+        engine.phases_ms(reset=True)
     except LiyabError as e:
         print(f"liyab-cli: {e}", file=sys.stderr)
         return 1
@@ -118,8 +122,9 @@ def main(argv=None) -> int:
         print(f"liyab-cli: {e}", file=sys.stderr)
         return 1
     s = res.stats
+    phases = {k: round(v, 3) for k, v in engine.phases_ms().items()}
     if args.json:
-        print(json.dumps({"turn": 0, "prompt_tokens": s.prompt_tokens, "cached_prefix_tokens": 0,
+        print(json.dumps({"turn": 0, **({"phases_ms": phases} if args.phases else {}), "prompt_tokens": s.prompt_tokens, "cached_prefix_tokens": 0,
                           "prefill_ms": round(s.prefill_ms, 3), "ttft_ms": round(s.ttft_ms, 3),
                           "generated_tokens": s.generated_tokens, "decode_ms": round(s.decode_ms, 3),
                           "tokens_per_second": round(s.tokens_per_second, 3), "kv_cache_bytes": s.kv_cache_bytes,
@@ -127,6 +132,10 @@ def main(argv=None) -> int:
     print(f"\n=== Generation ===\nprompt: {s.prompt_tokens} tokens (0 reused), {s.prefill_ms:.1f} ms, TTFT {s.ttft_ms:.1f} ms\n"
           f"decode: {s.generated_tokens} tokens, {s.decode_ms:.1f} ms, {s.tokens_per_second:.2f} tok/s\n"
           f"memory: KV {s.kv_cache_bytes / (1024.0 * 1024.0):.1f} MiB", file=sys.stderr)
+    if phases:
+        # as the reference prints them: device ms a generated token, phase by phase (tools/liyab_cli.cpp:198-211)
+        per = max(1, s.generated_tokens)
+        print("phases (ms/token): " + ", ".join(f"{k} {v / per:.3f}" for k, v in phases.items()), file=sys.stderr)
     return 0
 
 

@@ -220,6 +220,28 @@ def build_host(quiet: bool = False) -> str:
     return lib
 
 
+def build_host_selftest(sanitize: bool = True, out_dir: Optional[str] = None) -> str:
+    """Compiles `host/selftest/selftest.cpp` with the host sources into an executable of its own
+    and returns its path. `sanitize`: with the address and undefined-behaviour sanitizers
+    (-fsanitize=address,undefined, no recovery: the first finding ends the run). The executable
+    links nothing of Python or HIP, so the sanitizers' runtime is the only thing loaded with it."""
+    cxx = cxx_path()
+    if cxx is None:
+        raise RuntimeError("no C++ compiler was found (looked at $CXX, g++, c++, clang++, hipcc)")
+    out_dir = out_dir or tempfile.mkdtemp(prefix="liyab_host_selftest_")
+    exe = os.path.join(out_dir, "host_selftest_san" if sanitize else "host_selftest")
+    flags = ["-O1", "-g", "-std=c++17", "-Wall", "-Wextra"]
+    if sanitize:
+        # the sanitizers' runtime linked in, so that it need not come first among preloaded libraries
+        flags += ["-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-fno-omit-frame-pointer",
+                  "-static-libasan", "-static-libubsan"]
+    srcs = [p for p in host_sources() if not p.endswith("c_api.cpp")] + [os.path.join(HOST_DIR, "selftest", "selftest.cpp")]
+    r = subprocess.run([cxx, *flags, "-I", HOST_DIR, "-o", exe, *srcs], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building the host self-test failed:\n{r.stdout}\n{r.stderr}")
+    return exe
+
+
 if __name__ == "__main__":
     print(build_host())
     print(build())

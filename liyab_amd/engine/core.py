@@ -15,6 +15,7 @@ import torch
 
 from ..cache.pages import CacheManager
 from ..cache.storage import CacheStorage
+from .. import log
 from ..errors import InvalidArgument, KernelError
 from ..models.loading import load_model, resolve_dtype
 from .step import StepFunction, StepItem
@@ -57,6 +58,14 @@ class EngineCore:
                                     max_requests=max_requests, max_positions=max_positions)
         self.storage = CacheStorage(self.manager, self.dtype, self.device, self.model.state_specs())
         self.step_fn = StepFunction(self.model, self.manager, self.storage, self.device, use_graphs=use_graphs)
+        # one line at load with the geometry and the cache's cost a token, as the reference logs
+        # (src/core/transformer.cpp:880-884)
+        plan = self.model.plan
+        log.info("%s: %d layers (%d runs), width %d, vocabulary %d, context %d, %s; cache: %d groups, %d pages of %d "
+                 "positions each, %.1f KiB a token, %.1f MiB in all",
+                 plan.architecture, len(plan.layers), len(plan.order), plan.width, plan.vocab_size, max_positions,
+                 str(self.dtype).replace("torch.", ""), len(self.manager.groups), max(1, num_pages), page_size,
+                 self.storage.bytes_per_token() / 1024.0, self.storage.bytes_allocated() / 2.0 ** 20)
 
     @classmethod
     def from_plan(cls, plan, tensors, *, dtype="float32", device="cuda:0", **kw) -> "EngineCore":

@@ -49,12 +49,14 @@ class Engine:
     def __init__(self, model: Optional[str] = None, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_num_seqs: int = 64,
                  max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None,
-                 overlap: bool = True, use_graphs: bool = True, core: Optional[EngineCore] = None):
+                 overlap: bool = True, use_graphs: bool = True, core: Optional[EngineCore] = None,
+                 phases: bool = False):
         """`model`: a folder with config.json and model.safetensors; or `core`: an `EngineCore`
         built elsewhere (`EngineCore.from_plan` for a model made of a plan and tensors), whose
         own dtype, pages and graph setting then hold. `use_graphs`: replay recurring step shapes
         as captured HIP graphs (a part that decides on the host from a step's values, not from
-        its shape, needs this off). `ctx`: the
+        its shape, needs this off). `phases`: time the device per phase of the forward pass (`phases_ms()`;
+        steps are then launched kernel by kernel, so generation is slower). `ctx`: the
         context length (default: the model's). `prefill_chunk`: the longest
         portion of a prompt in one step (the reference's 256,
         src/core/engine.cpp:2863-2864). `num_pages` / `max_tokens` size the
@@ -73,6 +75,10 @@ class Engine:
         self.scheduler = Scheduler(self.core.manager, max_num_seqs=max_num_seqs,
                                    max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
                                    eos_token_id=self.core.model.plan.eos_token_id, on_open=self._reset_slot)
+        if phases:
+            from ..parts.base import PhaseTimer
+
+            self.core.step_fn.phases = PhaseTimer()
         self.sampler = Sampler(self.core.device)
         self._requests: Dict[Hashable, Request] = {}
         self._t_first: Dict[Hashable, float] = {}
@@ -84,6 +90,18 @@ class Engine:
         self._inflight = None  # (batch, wanting requests, pinned host tokens, event) of the step not yet read
         self._host_tokens = [None, None]
         self._turn = 0
+
+    def phases_ms(self, reset: bool = False) -> Dict[str, float]:
+        """Device milliseconds per phase (embed, attention, dense_ffn, lm_head, ...) summed over the
+        steps so far, for an engine made with `phases=True`; the reference's per-phase times
+        (include/liyab/types.h:228-236)."""
+        timer = self.core.step_fn.phases
+        if timer is None:
+            return {}
+        out = timer.totals()
+        if reset:
+            timer.reset()
+        return out
 
     def warmup(self) -> None:
         """Runs a short prompt and a few decoded tokens of a request of its own and drops it: the

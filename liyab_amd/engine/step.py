@@ -30,7 +30,7 @@ from .. import host
 from ..cache.pages import CacheManager
 from ..cache.storage import CacheStorage
 from ..errors import InvalidArgument
-from ..parts.base import GroupStep, StepContext, StepFacts, StepHost, Workspace
+from ..parts.base import GroupStep, PhaseTimer, StepContext, StepFacts, StepHost, Workspace
 
 
 @dataclass
@@ -102,6 +102,7 @@ class StepFunction:
         self._graph_generation = 0
         self.last_tokens = torch.zeros(manager.max_requests, dtype=torch.int32, device=self.device)
         self.last_context: Optional[StepContext] = None
+        self.phases: Optional[PhaseTimer] = None  # set: every step is launched kernel by kernel and timed per phase
         self.planners = list(getattr(model, "step_planners", ()))
         self._key = None  # the prepared step's shape: what its captured graph is kept under
         self._recurs = True
@@ -129,7 +130,8 @@ class StepFunction:
 
     # -- eager or replayed ----------------------------------------------------
     def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
-        if not self.use_graphs:
+        if not self.use_graphs or self.phases is not None:
+            ctx.phases = self.phases
             return self.model.forward(ctx, self.storage)
         if self.workspace.generation != self._graph_generation:
             # a workspace buffer moved since the graphs were captured: they hold its old address

@@ -80,8 +80,13 @@ def load() -> ctypes.CDLL:
         except Exception as e:  # noqa: BLE001
             raise KernelError(f"the HIP kernel library is not built and building it failed: {e}") from e
     elif _build.is_stale(path):
-        print(f"[liyab_amd] warning: {path} was built from other sources than those in csrc/; "
-              f"run `python -m liyab_amd.csrc.build`", file=sys.stderr, flush=True)
+        # built from other sources than those in csrc/: never serve them silently
+        print(f"[liyab_amd] {path} was built from other sources than those in csrc/: building it again",
+              file=sys.stderr, flush=True)
+        try:
+            path = _build.build()
+        except Exception as e:  # noqa: BLE001
+            raise KernelError(f"the HIP kernel library is stale and building it again failed: {e}") from e
     try:
         lib = ctypes.CDLL(path)
     except OSError as e:

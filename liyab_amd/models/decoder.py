@@ -82,6 +82,9 @@ class DecoderModel:
             return self._forward(ctx, storage)
 
     def _forward(self, ctx: StepContext, storage) -> Optional[torch.Tensor]:
+        phases = ctx.phases
+        if phases is not None:
+            phases.mark("embed")
         x = ctx.workspace.get("residual", (ctx.n_tokens, self.width), torch.float32)
         fused = self.residual_position.fused_table() if self.residual_position is not None else None
         self.embedding.forward(ctx, x, position_table=fused)
@@ -98,6 +101,15 @@ class DecoderModel:
                     pending.settle()
                     pending = None
                 block.forward(*args, writes_cache=e.writes_cache)
+        if phases is not None:
+            phases.mark("lm_head")
+            try:
+                return self._head(ctx, x, pending)
+            finally:
+                phases.finish()
+        return self._head(ctx, x, pending)
+
+    def _head(self, ctx: StepContext, x, pending) -> Optional[torch.Tensor]:
         if ctx.n_logit_rows == 0:
             return None  # nobody reads the stream again
         if self.final_norm is not None:

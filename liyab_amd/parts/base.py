@@ -102,6 +102,43 @@ class Workspace:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
 
 
+class PhaseTimer:
+    """Device time per phase of the model's forward pass (embed, each mixer kind, each
+    feed-forward kind, lm_head), summed over steps: the reference's PhaseTimer adds wall time per
+    phase the same way (src/core/transformer.cpp:463-481, phases in src/core/transformer.h:341-353)
+    and its command line prints them per token (tools/liyab_cli.cpp:198-211). `mark(name)` says
+    that the phase `name` starts now on the current stream; the time up to the next mark (or
+    `finish`) is that phase's. Events are read only in `totals()`, which waits for the device.
+    Steps are launched kernel by kernel while a timer is set: a replayed graph has no marks."""
+
+    def __init__(self):
+        self._marks = []  # (phase name or None for the end of a step, event)
+        self._totals: Dict[str, float] = {}
+        self.steps = 0
+
+    def mark(self, name: Optional[str]) -> None:
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self._marks.append((name, ev))
+
+    def finish(self) -> None:
+        self.mark(None)
+        self.steps += 1
+
+    def totals(self) -> Dict[str, float]:
+        """Milliseconds per phase since the timer was made (or `reset`)."""
+        if self._marks:
+            self._marks[-1][1].synchronize()
+            for (name, ev), (_, nxt) in zip(self._marks, self._marks[1:]):
+                if name is not None:
+                    self._totals[name] = self._totals.get(name, 0.0) + ev.elapsed_time(nxt)
+            self._marks = []
+        return dict(self._totals)
+
+    def reset(self) -> None:
+        self._marks, self._totals, self.steps = [], {}, 0
+
+
 @dataclass
 class GroupStep:
     """A cache group's view of the step."""
@@ -176,3 +213,4 @@ class StepContext:
     logit_slots: Optional[torch.Tensor] = None  # int32 [n_rows]: state slot of each wanted row's request
     last_tokens: Optional[torch.Tensor] = None  # int32 [slots]: the token each request drew last (on the device)
     plans: Dict[str, Any] = field(default_factory=dict)  # what each part's step planner made for this step, by its name
+    phases: Optional[PhaseTimer] = None  # set: the model and its blocks mark where each phase starts

@@ -15,6 +15,9 @@ class PreNormBlock:
 
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
+        # phases are named after the parts' kinds (the reference's: attention, dense_ffn, ...)
+        self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
+        self.ffn_phase = getattr(getattr(spec, "ffn", None), "kind", "ffn")
 
     takes_pending = True  # forward(..., pending=) takes the stream split and may return it split
 
@@ -23,6 +26,8 @@ class PreNormBlock:
         previous layer left it split (x is then stale). Returns the stream as a SplitStream if
         this layer leaves it split, else None (x holds it)."""
         stream = pending if pending is not None else x
+        if ctx.phases is not None:
+            ctx.phases.mark(self.mixer_phase)
         h, stream = self._normed(self.norm_mixer, stream, ctx)
         if getattr(self.mixer, "defers", False):
             stream = self.mixer.forward(h, ctx, cache, state, stream, writes_cache=writes_cache, defer=True) or x
@@ -30,6 +35,8 @@ class PreNormBlock:
             self.mixer.forward(h, ctx, cache, state, settled(stream), writes_cache=writes_cache)
             stream = x
         if self.ffn is not None:
+            if ctx.phases is not None:
+                ctx.phases.mark(self.ffn_phase)
             h, stream = self._normed(self.norm_ffn, stream, ctx)
             if getattr(self.ffn, "defers", False):
                 stream = self.ffn.forward(h, ctx, stream, defer=True) or x

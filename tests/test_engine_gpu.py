@@ -56,8 +56,8 @@ def make_core(model_dir, dtype, max_tokens, page_size=16, poison=True):
     core = EngineCore(model_dir, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8)
     if poison:  # free pages hold NaN: a kernel that reads past a request's length shows it
         for c in core.storage.layers.values():
-            c.k.fill_(float("nan"))
-            c.v.fill_(float("nan"))
+            for t in c.rows.values():
+                t.fill_(float("nan"))
         torch.cuda.synchronize()
     return core
 
@@ -286,6 +286,14 @@ def test_command_line_json(model_dirs, plain_models):
     eos = config.get("eos_token_id")
     assert turn["tokens"] == expect[:len(turn["tokens"])] and (len(turn["tokens"]) == 12 or turn["tokens"][-1] == eos)
     assert "decode:" in p.stderr and "prompt: 9 tokens" in p.stderr
+    assert "phases_ms" not in turn
+    # per-phase device times behind a flag; the tokens are the same
+    p2 = subprocess.run(cmd + ["--phases"], capture_output=True, text=True, timeout=600)
+    assert p2.returncode == 0, p2.stderr[-3000:]
+    turn2 = [json.loads(l) for l in p2.stdout.splitlines() if l.startswith("{")][1]
+    assert turn2["tokens"] == turn["tokens"]
+    assert set(turn2["phases_ms"]) == {"embed", "attention", "dense_ffn", "lm_head"}
+    assert all(v > 0 for v in turn2["phases_ms"].values()) and "phases (ms/token)" in p2.stderr
 
 
 # ---------------------------------------------------------------------------

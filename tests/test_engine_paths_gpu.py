@@ -45,8 +45,8 @@ def test_preempted_requests_are_recomputed_to_the_same_tokens(dtype, overlap, mo
                        prefill_chunk=32, overlap=overlap)
         tight.stop_at_eos = False
         for c in tight.core.storage.layers.values():  # free pages hold NaN
-            c.k.fill_(float("nan"))
-            c.v.fill_(float("nan"))
+            for t in c.rows.values():
+                t.fill_(float("nan"))
         together = tight.generate(prompts, sp)
         stats = tight.scheduler.stats
         assert stats.preemptions >= 1, "the pool held every request: nothing was preempted"
@@ -199,8 +199,8 @@ def test_fallback_geometries_whole_and_mixed(name, tmp_path):
                              ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48, 2)))):
             core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=8)
             for c in core.storage.layers.values():
-                c.k.fill_(float("nan"))
-                c.v.fill_(float("nan"))
+                for t in c.rows.values():
+                    t.fill_(float("nan"))
             got = tt.run_schedule(core, steps)
             tt.check_against_plain(got, reqs, refs, TOL[dtype], f"{name} {label} {dtype}", family=f"fallback:{name}")
             core.manager.check()

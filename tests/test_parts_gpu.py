@@ -915,6 +915,106 @@ def test_a_part_with_its_own_step_metadata_runs_under_graphs_and_the_scheduler()
     assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
 
+# ---------------------------------------------------------------------------
+# a toy mixer that keeps one narrow row a position instead of a key and a value
+# ---------------------------------------------------------------------------
+class NarrowSpec:
+    kind = "toy_narrow"
+
+    def __init__(self, width, rank, prefix):
+        self.width, self.rank, self.prefix = width, rank, prefix
+
+
+class NarrowMixer:
+    """c_t = h_t . Wc^T (a row of `rank` values, the only thing cached: one plane "c" of one head);
+    out_t = (mean of c_j over j <= t) . Wo^T. A test's toy in torch: it writes its rows to its own
+    plane of the pages at the step's cache slots and reads a request's rows back through its
+    block table, so what it keeps is paged, shared and given back like keys and values."""
+
+    def __init__(self, spec, store, dtype):
+        from liyab_amd.config import TensorSource
+
+        self.rank = spec.rank
+        self.down = store.fetch(TensorSource(spec.prefix + ".down"), (spec.rank, spec.width), "matrix")
+        self.up = store.fetch(TensorSource(spec.prefix + ".up"), (spec.width, spec.rank), "matrix")
+
+    def cache_spec(self):
+        from liyab_amd.cache import KVSpec
+
+        return KVSpec(1, self.rank, rows=(("c", 1, self.rank),))
+
+    def state_spec(self):
+        return None
+
+    def forward(self, h, ctx, cache, state, residual, writes_cache=True):
+        from liyab_amd.parts import as_tensor
+
+        h = as_tensor(h)
+        plane = cache.rows["c"]  # [pages, 1, page_size, rank]
+        assert set(cache.rows) == {"c"} and plane.shape[1:] == (1, ctx.page_size, self.rank)
+        group = ctx.groups[cache.group]
+        c = (h.float() @ self.down.float().t()).to(plane.dtype)
+        flat = plane.view(-1, self.rank)  # one head: slot = page * page_size + offset indexes rows directly
+        if writes_cache:
+            flat.index_copy_(0, group.slots.long(), c)
+        out = torch.empty(h.shape[0], self.rank, device=h.device)
+        tables = group.block_tables.tolist()
+        for i, (a, n, first) in enumerate(zip(ctx.host.starts, ctx.host.q_lens, ctx.host.first_pos)):
+            length = first + n
+            pages = torch.tensor(tables[i][:-(-length // ctx.page_size)], device=h.device)
+            kept = plane[pages, 0].reshape(-1, self.rank)[:length].float()
+            means = kept.cumsum(0) / torch.arange(1, length + 1, device=h.device)[:, None]
+            out[a:a + n] = means[first:]
+        residual += out @ self.up.float().t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_rows_of_its_own_in_the_pages(dtype):
+    """The pages of a group hold whatever planes of rows its mixers name: here one row of 24
+    values a position beside an attention layer's keys and values of 5 heads of 16 (two groups,
+    each with its pages and block tables). Whole, in portions and mixed with few pages."""
+    from liyab_amd.config import LayerSpec, OrderEntry
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.parts import register_mixer
+
+    register_mixer("toy_narrow", NarrowMixer)
+    d, V, P, eps, r = 80, 150, 140, 1e-5, 24
+    rng = np.random.default_rng(73)
+    layers = [LayerSpec(NarrowSpec(d, r, "m0"), ffn_spec("f0", d, 96, "gelu_tanh"), norm_spec("n0a", d, eps), norm_spec("n0b", d, eps)),
+              LayerSpec(attention_spec("a1", d, 5, 5, 16, 0.25), None, norm_spec("n1a", d, eps), None)]
+    tw = {"emb": rand(rng, V, d, scale=0.5), "pos": rand(rng, P, d, scale=0.3), **norm_tensors(rng, "nf", d),
+          "m0.down": rand(rng, r, d, scale=0.2), "m0.up": rand(rng, d, r, scale=0.2), **attention_tensors(rng, "a1", d, 5, 5, 16),
+          **ffn_tensors(rng, "f0", d, 96), **norm_tensors(rng, "n0a", d), **norm_tensors(rng, "n0b", d), **norm_tensors(rng, "n1a", d)}
+    if dtype == "bfloat16":
+        tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tw.items()}
+    plan = make_plan(d, V, P, layers, [OrderEntry(0), OrderEntry(1)], eps)
+
+    def plain_model(ids):
+        x = f64(tw["emb"])[ids] + f64(tw["pos"])[:len(ids)]
+        c = plain_norm(x, tw, "n0a", eps) @ f64(tw["m0.down"]).T
+        means = np.cumsum(c, axis=0) / np.arange(1, len(ids) + 1)[:, None]
+        x = x + means @ f64(tw["m0.up"]).T
+        x = x + plain_ffn(plain_norm(x, tw, "n0b", eps), tw, "f0", "gelu_tanh")
+        a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 5, 5, 16, 0.25)
+        return plain_norm(x + a, tw, "nf", eps) @ f64(tw["emb"]).T
+
+    reqs = {f"n{i}": tt.random_tokens(20 + i, n, V) for i, n in enumerate([50, 140, 4, 77])}
+    ref = {rid: plain_model(toks) for rid, toks in reqs.items()}
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=6))):
+        core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4,
+                                    use_graphs=False)  # the toy reads block tables on the host
+        assert sorted(g.spec.planes for g in core.manager.groups) == [(("c", 1, r),), (("k", 5, 16), ("v", 5, 16))]
+        assert core.storage.bytes_per_token() == (r + 2 * 5 * 16) * (4 if dtype == "float32" else 2)
+        for c in core.storage.layers.values():
+            for t in c.rows.values():
+                t.fill_(float("nan"))
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, TOL_TOY[dtype], f"narrow toy {name} {dtype}", family="toy:narrow")
+        core.manager.check()
+        assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
+
+
 class BareNorm:
     """A LayerNorm that knows nothing of split streams or pending norms (no `takes_planes`, no `lazy`)."""
 

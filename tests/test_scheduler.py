@@ -341,3 +341,20 @@ def test_native_scheduler_decides_as_the_plain_one(seed, lagged):
     native, plain = drive(True), drive(False)
     assert native[0] == plain[0]
     assert native[1] == plain[1]
+
+
+def test_host_library_under_the_sanitizers(tmp_path):
+    """The host C++ (page pools, cache manager, scheduler, a step's metadata) compiled with the
+    address and undefined-behaviour sanitizers into a driver of its own that needs no Python,
+    and run over random stories of requests: any access out of bounds, use after release or
+    overflow ends it with a report."""
+    import os
+    import subprocess
+
+    from liyab_amd.csrc import build
+
+    exe = build.build_host_selftest(sanitize=True, out_dir=str(tmp_path))
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    p = subprocess.run([exe, "120", "120"], capture_output=True, text=True, timeout=300, env=env)
+    assert p.returncode == 0, (p.stdout[-2000:], p.stderr[-6000:])
+    assert "selftest ok" in p.stdout
