@@ -3,6 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|xl] [--layers L]
     python bench.py --sequences 1,2,4,8 [-n 128]     # together against in turns, and whether replies are the same
     python bench.py --prefill-tokens 512,2048,8192   # prefill tokens a second per length
+    python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
+    python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -61,12 +63,12 @@ def prefill_flops(cfg, prompt_lens, logit_rows):
     return flops + 2.0 * logit_rows * d * V
 
 
-def make_engine(model_dir, dtype, batch, ctx):
+def make_engine(model_dir, dtype, batch, ctx, page_size=64, prefill_chunk=1024, batch_invariant=False):
     from liyab_amd import Engine
 
-    pages = batch * (-(-ctx // 64)) + 4
-    return Engine(model_dir, dtype=dtype, page_size=64, num_pages=pages, max_num_seqs=max(batch, 2),
-                  max_batched_tokens=max(2048, batch), prefill_chunk=1024, ctx=ctx)
+    pages = batch * (-(-ctx // page_size)) + 4
+    return Engine(model_dir, dtype=dtype, page_size=page_size, num_pages=pages, max_num_seqs=max(batch, 2),
+                  max_batched_tokens=max(2048, batch), prefill_chunk=prefill_chunk, ctx=ctx, batch_invariant=batch_invariant)
 
 
 def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
@@ -99,6 +101,78 @@ def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
     for r in list(engine.scheduler.running):
         engine.abort(r.rid)
     return batch * steps / dt, dt * 1e3 / steps, bytes_per_step
+
+
+def workload_run(engine, cfg, prompts, params_of, label):
+    """A whole workload through the engine's loop: requests arrive together, prompts go in portions
+    beside decoding requests. Returns generated tokens a second, all tokens (prompt and generated)
+    a second, and the share of the HBM roofline: the bytes every step has to read (each weight
+    once, and the cache of the positions its requests hold) over the whole time."""
+    import torch
+
+    elt = 2 if engine.core.dtype == torch.bfloat16 else 4
+    w_bytes, kv_pos = weight_bytes(cfg, elt), kv_bytes_per_position(cfg, elt)
+    engine.stop_at_eos = False
+    rids = [engine.add_request(p, params_of(i), rid=f"{label}-{i}") for i, p in enumerate(prompts)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = bytes_read = 0
+    while engine.has_unfinished():
+        before = engine.core.step_fn.steps
+        engine.step()
+        if engine.core.step_fn.steps > before:
+            h = engine.core.step_fn.last_context.host
+            bytes_read += w_bytes + kv_pos * sum(f + q for f, q in zip(h.first_pos, h.q_lens))
+            steps += 1
+    engine.flush()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    results = [engine.result(r) for r in rids]
+    for r in rids:
+        engine.release(r)
+    generated = sum(len(r.tokens) for r in results)
+    prompt_tokens = sum(len(p) for p in prompts)
+    return {"generated_tok_s": round(generated / dt, 1), "all_tok_s": round((generated + prompt_tokens) / dt, 1),
+            "seconds": round(dt, 4), "steps": steps, "ms_per_step": round(dt * 1e3 / max(steps, 1), 4),
+            "generated": generated, "prompt_tokens": prompt_tokens,
+            "preemptions": sum(r.stats.preemptions for r in results),
+            "roofline_frac": round(bytes_read / dt / 1e9 / HBM_PEAK_GBS, 4)}, [r.tokens for r in results]
+
+
+def link_floor(device="cuda:0", links=100):
+    """What a dependent kernel costs at least inside a replayed graph, measured with the library's
+    own kernels: a chain of kernels that each write one word (the distance from one kernel's end
+    to the next one's start), and a chain of norms over 8 rows of 768 in which each reads what the
+    one before wrote (a boundary, a first read of fresh data, a few hundred cycles of work, a write)."""
+    import torch
+
+    from liyab_amd.kernels import ops
+
+    dev = torch.device(device)
+    one = torch.zeros(64, dtype=torch.int32, device=dev)
+    a = torch.randn(8, 768, device=dev)
+    b = torch.empty_like(a)
+    w, bias = torch.ones(768, device=dev), torch.zeros(768, device=dev)
+    out = {}
+    for name, body in (("a kernel that writes one word", lambda i: ops.fill_(one[:1], i)),
+                       ("a norm of 8 rows of 768 that reads the one before", lambda i: ops.layernorm(b if i % 2 == 0 else a, a if i % 2 == 0 else b, w, bias, 1e-5))):
+        for i in range(3):
+            body(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(links):
+                body(i)
+        best = float("inf")
+        for _ in range(6):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            e1.synchronize()
+            best = min(best, e0.elapsed_time(e1))
+        out[name] = round(best * 1e3 / links, 3)
+    return {"metric": "microseconds a dependent kernel of a replayed graph", "links": links, "us_per_link": out}
 
 
 def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
@@ -179,6 +253,12 @@ def main():
     ap.add_argument("--sequences", default="", help="e.g. 1,2,4: that many sequences together against one after the other "
                     "(the reference's liyab-seq-bench): tokens a second both ways and whether every reply equals its reply alone")
     ap.add_argument("-n", type=int, default=128, help="tokens generated per sequence with --sequences")
+    ap.add_argument("--workload", default="", choices=["", "medium16", "xl64"],
+                    help="medium16: GPT-2 medium's sizes, 16 requests with prompts of 64 to 1,023 tokens, portions of 256, 128 greedy "
+                         "tokens each; xl64: GPT-2 XL's sizes, 64 requests with prompts of 256 tokens decoding to 1,024, greedy and at temperature 1")
+    ap.add_argument("--page-size", type=int, default=64, help="positions a cache page (default 64; the engine's own default is 16)")
+    ap.add_argument("--batch-invariant", action="store_true", help="kernels chosen from sizes and positions only (reproducible bfloat16 replies)")
+    ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -187,6 +267,11 @@ def main():
 
     from liyab_amd.weights import write_random_model
 
+    if args.link_floor:
+        print(json.dumps(link_floor()))
+        return 0
+    if args.workload:
+        args.size = "medium" if args.workload == "medium16" else "xl"
     cfg = dict(SMALL, **SIZES[args.size])
     full_layers = cfg["n_layer"]
     if args.layers:
@@ -199,7 +284,42 @@ def main():
         slots = max(args.batch, 64 if not args.no_points else args.batch)
         if args.prefill_tokens:
             slots = max(slots, max(-(-int(x) // ctx) for x in args.prefill_tokens.split(",")))
-        engine = make_engine(d, args.dtype, slots, ctx)
+        if args.workload:
+            import numpy as np
+
+            from liyab_amd import SamplingParams
+
+            layers_note = {"n_layer": cfg["n_layer"], "n_layer_full": full_layers}
+            if args.workload == "medium16":
+                # BASELINE's workload for GPT-2 medium's sizes: 16 requests, prompt lengths uniform in [64, 1024) and ids
+                # from seed 21, continuously batched with portions of 256, 128 greedy tokens each (capped at the positions)
+                rng = np.random.default_rng(21)
+                lens = rng.integers(64, 1024, 16).tolist()
+                prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in lens]
+                engine = make_engine(d, args.dtype, 16, ctx, page_size=args.page_size, prefill_chunk=256, batch_invariant=args.batch_invariant)
+                engine.warmup()
+                runs = {}
+                for rep in range(2):  # the second run finds its recurring shapes captured
+                    runs["greedy"], _ = workload_run(engine, cfg, prompts, lambda i: SamplingParams(temperature=0.0, max_tokens=128), f"m{rep}")
+                print(json.dumps({"metric": "GPT-2 medium sizes: 16 requests, prompts of 64 to 1,023 tokens in portions of 256, 128 greedy tokens each",
+                                  "dtype": short, "data": "synthetic", "page_size": args.page_size, **layers_note,
+                                  "prompt_lens": lens, "runs": runs}))
+            else:
+                # BASELINE's workload for GPT-2 XL's sizes: 64 requests, prompts of 256 ids from seed 31, decoding to 1,024
+                # positions, greedy and at temperature 1
+                rng = np.random.default_rng(31)
+                prompts = [rng.integers(0, cfg["vocab_size"], 256).tolist() for _ in range(64)]
+                engine = make_engine(d, args.dtype, 64, ctx, page_size=args.page_size, prefill_chunk=256, batch_invariant=args.batch_invariant)
+                engine.warmup()
+                runs = {}
+                n_new = ctx - 256 + 1
+                for name, make in (("greedy", lambda i: SamplingParams(temperature=0.0, max_tokens=n_new)),
+                                   ("temperature 1.0", lambda i: SamplingParams(temperature=1.0, top_k=0, top_p=1.0, seed=1000 + i, max_tokens=n_new))):
+                    runs[name], _ = workload_run(engine, cfg, prompts, make, name[:1])
+                print(json.dumps({"metric": "GPT-2 XL sizes: 64 requests, prompts of 256 tokens decoding to 1,024 positions",
+                                  "dtype": short, "data": "synthetic", "page_size": args.page_size, **layers_note, "runs": runs}))
+            return 0
+        engine = make_engine(d, args.dtype, slots, ctx, page_size=args.page_size, batch_invariant=args.batch_invariant)
         if args.prefill_tokens:
             runs = []
             for total in [int(x) for x in args.prefill_tokens.split(",")]:
@@ -227,7 +347,8 @@ def main():
             "config": {"model": f"gpt2-{args.size}-sizes-random-weights", "n_layer": cfg["n_layer"], "n_layer_full": full_layers,
                        "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": cfg["n_embd"] // cfg["n_head"],
                        "n_inner": cfg["n_inner"], "vocab_size": cfg["vocab_size"], "n_positions": cfg["n_positions"],
-                       "global_batch": args.batch, "seq_len": ctx, "prompt_len": args.prompt, "page_size": 64,
+                       "global_batch": args.batch, "seq_len": ctx, "prompt_len": args.prompt, "page_size": args.page_size,
+                       "batch_invariant": bool(args.batch_invariant),
                        "weights_seed": WEIGHT_SEEDS[args.size], "ids_seed": 11, "parallelism": "single-gpu"},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -238,11 +359,24 @@ def main():
             flops = prefill_flops(cfg, lens, len(lens))
             out["prefill"] = {"value": round(ptps, 1), "tokens": sum(lens), "ms": round(pms, 4),
                               "frac": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)}
+            # every point over at least 64 steps after at least 3 of its own shape, whatever --steps says: fewer do
+            # not outlast the first sight of a shape (an eager run, then a capture)
             points = {}
+            k, w = min(max(steps, 64), 256, ctx - args.prompt - 8), max(args.warmup, 3)
             for b in (1, 64):
-                k = min(steps, 256)
-                t, _, _ = decode_run(engine, cfg, b, args.prompt, k, args.warmup)
+                t, pms_b, pbytes = decode_run(engine, cfg, b, args.prompt, k, w)
                 points[f"decode_b{b}"] = round(t, 1)
+                points[f"decode_b{b}_ms_per_step"] = round(pms_b, 4)
+                points[f"decode_b{b}_mbytes_per_step"] = round(pbytes / 1e6, 1)
+                points[f"decode_b{b}_roofline_frac"] = round(pbytes / (pms_b * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            points["steps_per_point"] = k
+            if args.page_size != 16:
+                # the headline batch again with pages of 16 positions, the engine's own default
+                small_pages = make_engine(d, args.dtype, args.batch, ctx, page_size=16, batch_invariant=args.batch_invariant)
+                t, pms_b, _ = decode_run(small_pages, cfg, args.batch, args.prompt, k, w)
+                points[f"decode_b{args.batch}_page16"] = round(t, 1)
+                points[f"decode_b{args.batch}_page16_ms_per_step"] = round(pms_b, 4)
+                del small_pages
             out["points"] = points
     print(json.dumps(out))
     return 0

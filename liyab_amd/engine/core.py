@@ -24,11 +24,14 @@ from .step import StepFunction, StepItem
 class EngineCore:
     def __init__(self, model_dir: Optional[str] = None, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_requests: int = 64,
-                 context_length: Optional[int] = None, use_graphs: bool = True, model=None, config=None):
+                 context_length: Optional[int] = None, use_graphs: bool = True, model=None, config=None,
+                 batch_invariant: bool = False):
         """`model_dir`: a folder with config.json and model.safetensors (or pass a built
         `model`, see `from_plan`). `num_pages`: pages per cache group; or `max_tokens`: the
         most tokens live requests hold together (rounded up to whole pages per request by the
-        caller's accounting). With neither, every request slot can reach the full context."""
+        caller's accounting). With neither, every request slot can reach the full context.
+        `batch_invariant`: a request's bfloat16 logits have the same bits alone and in any batch
+        (kernels chosen from sizes and positions only: slower; float32 is so either way)."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: this engine runs on gfx950 only and has no CPU path")
         from ..kernels import ops
@@ -57,7 +60,8 @@ class EngineCore:
         self.manager = CacheManager(self.model.cache_groups(), page_size=page_size, num_pages=max(1, num_pages),
                                     max_requests=max_requests, max_positions=max_positions)
         self.storage = CacheStorage(self.manager, self.dtype, self.device, self.model.state_specs())
-        self.step_fn = StepFunction(self.model, self.manager, self.storage, self.device, use_graphs=use_graphs)
+        self.step_fn = StepFunction(self.model, self.manager, self.storage, self.device, use_graphs=use_graphs,
+                                    batch_invariant=batch_invariant)
         # one line at load with the geometry and the cache's cost a token, as the reference logs
         # (src/core/transformer.cpp:880-884)
         plan = self.model.plan

@@ -50,12 +50,14 @@ class Engine:
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_num_seqs: int = 64,
                  max_batched_tokens: int = 2048, prefill_chunk: int = 256, ctx: Optional[int] = None,
                  overlap: bool = True, use_graphs: bool = True, core: Optional[EngineCore] = None,
-                 phases: bool = False):
+                 phases: bool = False, batch_invariant: bool = False):
         """`model`: a folder with config.json and model.safetensors; or `core`: an `EngineCore`
         built elsewhere (`EngineCore.from_plan` for a model made of a plan and tensors), whose
         own dtype, pages and graph setting then hold. `use_graphs`: replay recurring step shapes
         as captured HIP graphs (a part that decides on the host from a step's values, not from
-        its shape, needs this off). `phases`: time the device per phase of the forward pass (`phases_ms()`;
+        its shape, needs this off). `batch_invariant`: every reply, greedy or seeded, is the same alone and in any batch in
+        bfloat16 too, as the reference promises (include/liyab/engine.h:987-990): kernels are chosen
+        from the model's sizes and a token's position only, which costs speed. `phases`: time the device per phase of the forward pass (`phases_ms()`;
         steps are then launched kernel by kernel, so generation is slower). `ctx`: the
         context length (default: the model's). `prefill_chunk`: the longest
         portion of a prompt in one step (the reference's 256,
@@ -71,7 +73,7 @@ class Engine:
         else:
             self.core = EngineCore(model, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
                                    max_tokens=max_tokens, max_requests=max_num_seqs, context_length=ctx,
-                                   use_graphs=use_graphs)
+                                   use_graphs=use_graphs, batch_invariant=batch_invariant)
         self.scheduler = Scheduler(self.core.manager, max_num_seqs=max_num_seqs,
                                    max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
                                    eos_token_id=self.core.model.plan.eos_token_id, on_open=self._reset_slot)

@@ -85,7 +85,7 @@ class StepFunction:
     must then depend on the host only through the shape: the ones in this package do."""
 
     def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0", use_graphs: bool = True,
-                 max_graphs: int = 256):
+                 max_graphs: int = 256, batch_invariant: bool = False):
         self.model = model
         self.manager = manager
         self.storage = storage
@@ -97,6 +97,7 @@ class StepFunction:
         self.tokens = 0
         self.use_graphs = use_graphs
         self.max_graphs = max_graphs
+        self.batch_invariant = batch_invariant  # kernels chosen from sizes and positions only (ops.batch_invariant)
         self._graphs = {}  # shape -> (graph, logits) once captured, or the count of eager runs
         self.graph_replays = 0
         self._graph_generation = 0
@@ -130,6 +131,12 @@ class StepFunction:
 
     # -- eager or replayed ----------------------------------------------------
     def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        from ..kernels import ops
+
+        with ops.batch_invariant(self.batch_invariant):
+            return self._run(ctx)
+
+    def _run(self, ctx: StepContext) -> Optional[torch.Tensor]:
         if not self.use_graphs or self.phases is not None:
             ctx.phases = self.phases
             return self.model.forward(ctx, self.storage)

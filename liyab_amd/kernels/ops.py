@@ -53,6 +53,37 @@ class on_current_stream:
         return False
 
 
+_invariant = False
+
+
+class batch_invariant:
+    """Within this context the kernels that serve a row are chosen from the model's sizes and the
+    row's own position only, never from what else the step holds: products by the tiled
+    matrix-core kernels whose sums run over k in one order whatever the tile (no streaming kernel,
+    no cut over K, no norm folded into a product), attention token by token with one split on
+    four waves. A row's bfloat16 results then have the same bits alone and in any batch, as the
+    reference promises of its passes (include/liyab/engine.h:987-990, src/core/transformer.h:746-751);
+    the step-shaped choices outside this context are faster and differ from these by rounding."""
+
+    def __init__(self, on: bool = True):
+        self.on = on
+
+    def __enter__(self):
+        global _invariant
+        self._before = _invariant
+        _invariant = self.on
+        return self
+
+    def __exit__(self, *exc):
+        global _invariant
+        _invariant = self._before
+        return False
+
+
+def is_batch_invariant() -> bool:
+    return _invariant
+
+
 def _dev(t: torch.Tensor, what: str) -> None:
     if not t.is_cuda:
         raise KernelError(f"{what} must be on the GPU")
@@ -505,7 +536,7 @@ def k_parts(M: int, N: int, K: int) -> int:
     then streams through those few; cut over K it covers the chip. Measured at 8 rows, whole
     and in parts (us): 3,072 -> 768 7.2 and 4.5 (four parts), 768 -> 768 4.6 and 3.4 (four),
     6,400 -> 1,600 13.4 and 8.5 (two), 1,600 -> 1,600 5.4 and 4.6 (two)."""
-    if M > 32 or K % 8 != 0:
+    if M > 32 or K % 8 != 0 or _invariant:
         return 1
     groups, units = (N + 15) // 16 * ((M + 15) // 16), (K + 63) // 64  # workgroups uncut; units of 64 k
     parts = 1
@@ -529,7 +560,7 @@ def tiled_k_parts(M: int, N: int, K: int) -> int:
     1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: inner
     dimensions from 3,072 gain, in 4 parts (ms a step at 64 rows, whole and cut: GPT-2 small's
     sizes 0.806 and 0.797, medium's 1.767 and 1.715; XL's 5.19 and 4.90)."""
-    if K % 64 != 0 or M <= 32:
+    if K % 64 != 0 or M <= 32 or _invariant:
         return 1
     if M <= 64:
         return 4 if K >= 3072 and N <= 2048 else 1
@@ -590,7 +621,7 @@ def skinny_ln_pays(M: int, N: int, K: int) -> bool:
     with more workgroups (16 or 32 output features each) than compute units they run in two
     rounds, which costs more than the norm's kernel (GPT-2 XL's 1,600 -> 4,800 at 8 rows in
     strips of 16: 15.2 us folded against 9 + 4.5)."""
-    return skinny_ln_takes(M, K) and (N + (31 if M <= 16 else 15)) // (32 if M <= 16 else 16) <= compute_units()
+    return not _invariant and skinny_ln_takes(M, K) and (N + (31 if M <= 16 else 15)) // (32 if M <= 16 else 16) <= compute_units()
 
 
 def gemm_mfma_dl(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out=None, residual=None,
@@ -618,6 +649,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
     """The product kernel for these operands: matrix cores for bfloat16 shapes they take,
     the plain tiled kernel for float32 and everything else. `kv` = (k_cache, v_cache, slots,
     q_dim) with the paged QKV epilogue."""
+    if _invariant and mfma_takes(a, w):
+        # one family of kernels whatever the number of rows: their sum over k has one order for
+        # every tile shape (units of 64 k in turn, 16 k an instruction), so a row's bits do not
+        # depend on the rows beside it
+        if a.shape[1] % 64 == 0:
+            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv,
+                         tile=8 if a.shape[0] * w.shape[0] >= 2048 * 2048 else (6 if a.shape[1] >= 2048 else 2))
+        else:
+            gemm_mfma(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=2)
+        return
     if mfma_takes(a, w):
         M, N = a.shape[0], w.shape[0]
         if 12 < M <= 128 and N >= 16384 and a.shape[1] % 64 == 0:
@@ -808,6 +849,13 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
                          rows_are_requests=tok_list is None and host.max_q_len == 1)
 
+    if fast and _invariant and block_tables.shape[1] <= 2048:
+        # every token on its own, its keys in one split on four waves: which lane adds which key
+        # follows from the token's position alone
+        n = out.shape[0]
+        attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
+                         window=window, n_splits=1, waves=4, rows_are_requests=host.max_q_len == 1)
+        return None
     if fast and plan.mode == "decode" and block_tables.shape[1] <= 2048:
         n = out.shape[0]
         splits, waves = decode_split_plan(n, n_head, plan.context_bucket) if splits_ok else (1, 4)

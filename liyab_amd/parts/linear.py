@@ -67,6 +67,8 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
     next product cut this way writes its own under another name."""
     from .base import SplitStream
 
+    if ops.is_batch_invariant():
+        return None  # no cut over K: its parts would follow the step's size
     a = a.tensor() if isinstance(a, Normed) else a
     in_splits = a.dim() == 4  # attention's output as its splits [tokens, heads, splits, head size + 4]
     M, K = (a.shape[0], a.shape[1] * (a.shape[3] - 4)) if in_splits else a.shape

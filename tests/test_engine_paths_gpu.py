@@ -252,3 +252,68 @@ def test_head_sizes_the_kernels_cannot_take_are_refused_at_load(tmp_path):
     write_safetensors(str(folder / "model.safetensors"), {k: torch.zeros(s) for k, s in shapes.items()}, {})
     with pytest.raises(Unsupported, match="272"):
         EngineCore(str(folder), dtype="float32", page_size=16, max_tokens=64)
+
+
+# ---------------------------------------------------------------------------
+# bfloat16 replies that do not depend on the batch
+# ---------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def small_widths_model(tmp_path_factory):
+    """GPT-2 small's widths and vocabulary, three layers."""
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 3, "n_embd": 768, "n_head": 12, "n_inner": 3072, "vocab_size": 50257,
+           "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    d = str(tmp_path_factory.mktemp("small_widths"))
+    write_random_model(d, cfg, 10, dtype="bfloat16")
+    return d, cfg
+
+
+def test_batch_invariant_logits_have_the_same_bits_alone_and_together(small_widths_model):
+    """With batch_invariant the bfloat16 logits of a position are the same bits however the
+    tokens are cut into steps and whatever else a step holds: whole prompts, the last tokens
+    one by one, portions of changing size, and mixed batches of up to four requests."""
+    from liyab_amd.engine import EngineCore
+
+    d, cfg = small_widths_model
+    V = cfg["vocab_size"]
+    reqs = {f"i{i}": tt.random_tokens(500 + i, n, V) for i, n in enumerate([150, 33, 9, 70, 260])}
+    runs = {}
+    for label, steps in (("whole", tt.schedule_whole(reqs)), ("tail", tt.schedule_bulk_tail(reqs, tail=12)),
+                         ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48, 2, 31, 7))),
+                         ("mixed", tt.schedule_mixed(reqs, seed=4, decode_tail=10))):
+        core = EngineCore(d, dtype="bfloat16", page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=8,
+                          batch_invariant=True)
+        runs[label] = tt.run_schedule(core, steps)
+        assert core.step_fn.graph_replays > 0 or label == "whole"
+        del core
+    for label in ("tail", "portions", "mixed"):
+        for rid, toks in reqs.items():
+            for p in range(len(toks)):
+                assert np.array_equal(runs[label][rid][p], runs["whole"][rid][p]), \
+                    f"{label}: request {rid} position {p} differs from its logits alone and whole"
+    # the step-shaped kernels of the default mode agree with these within the tolerance, not bit for bit
+    steps = tt.schedule_mixed(reqs, seed=4, decode_tail=10)
+    core = EngineCore(d, dtype="bfloat16", page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=8)
+    fast = tt.run_schedule(core, steps)
+    worst = max(tt.rel_err(fast[rid][p], runs["whole"][rid][p]) for rid, toks in reqs.items() for p in range(len(toks)))
+    assert 0 < worst <= TOL["bfloat16"]
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_batch_invariant_replies_are_the_same_alone_and_among_eight(small_widths_model, overlap):
+    """Greedy and seeded replies in bfloat16 at GPT-2 small's widths: the same tokens for a
+    request alone and among eight, with random weights, whose logits lie close together."""
+    from liyab_amd import Engine, SamplingParams
+
+    d, cfg = small_widths_model
+    prompts = [tt.random_tokens(600 + i, n, cfg["vocab_size"]) for i, n in enumerate([40, 7, 120, 64, 1, 90, 33, 15])]
+    engine = Engine(d, dtype="bfloat16", page_size=16, max_num_seqs=8, max_batched_tokens=256, prefill_chunk=64,
+                    batch_invariant=True, overlap=overlap)
+    engine.stop_at_eos = False
+    for sp in (SamplingParams(temperature=0.0, max_tokens=32),
+               SamplingParams(temperature=0.8, top_k=40, top_p=0.95, seed=21, max_tokens=32)):
+        together = engine.generate(prompts, sp)
+        alone = [engine.generate(p, sp) for p in prompts]
+        for i, (a, b) in enumerate(zip(together, alone)):
+            assert a.tokens == b.tokens, f"prompt {i}: the reply among eight differs from the reply alone"
