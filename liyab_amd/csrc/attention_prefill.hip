@@ -23,6 +23,14 @@
 // Maximum, exponentials, sums and outputs are 32-bit. A query's result depends
 // on its position and the block grid (multiples of 32 from the window's start),
 // not on the batch or the pages. Head sizes: multiples of 16 up to 128.
+//
+// A block's work is one chain: fragments from LDS, four products into one accumulator, the
+// maximum across two lanes, sixteen exponentials, fragments of the values, four products; alone
+// it takes about 2,000 cycles for 600 of arithmetic (measured: a tile that walks 1,024 keys took
+// 24 us on an otherwise idle chip, 0.018 us a key). With NS = 2 a wave walks two blocks a step
+// as two streams with a running maximum, sum and output each: nothing in one stream waits for the
+// other, so their chains overlap, and the streams are merged once at the end (in registers, then
+// the KS partial results as before).
 #include "common.h"
 
 namespace liyab {
@@ -39,10 +47,10 @@ union QFrag {
 
 constexpr int AP_KEYS = 32;     // keys per block
 constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
-constexpr int AP_DEPTH = 6;     // blocks of keys and values in flight in registers
+constexpr int kDepth = 6;       // blocks of keys and values in flight in registers
 constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LDS
 
-template <int DB, int QG, int KS>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS blocks of keys a step
+template <int DB, int QG, int KS, int NS = 1>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS x NS blocks of keys a step, NS a wave
 __global__ void __launch_bounds__(64 * QG * KS)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -51,7 +59,8 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
     constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
-    constexpr int STEP_KEYS = AP_KEYS * KS;  // keys staged a step
+    constexpr int AP_DEPTH = kDepth / NS;  // the same bytes in flight whatever a step holds
+    constexpr int STEP_KEYS = AP_KEYS * KS * NS;  // keys staged a step
     constexpr int STAGE = STEP_KEYS * LDK;
     // values are kept transposed, [dimension][key of the step], rows padded by 4 keys: the 8-byte
     // reads of 32 lanes (32 dimensions, one group of 4 keys) then fall in 64 different banks
@@ -92,12 +101,19 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
             if (s < n_slabs) qf[s].u = *reinterpret_cast<const u32x4*>(qrow + 16 * s + 8 * g2);
         }
     }
-    floatx16 o[DB];
+    // per stream: outputs, the reference the exponentials are taken against, and this lane's part
+    // of the sum (its own keys: the two lanes of a query add theirs up at the end)
+    floatx16 o_s[NS][DB];
+    float m_s[NS], l_s[NS];
 #pragma unroll
-    for (int d = 0; d < DB; ++d)
+    for (int z = 0; z < NS; ++z) {
+        m_s[z] = -INFINITY;
+        l_s[z] = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_s[z][d][r] = 0.0f;
+    }
 
     const int k_hi = pos0 + nq - 1;  // last key any query of the tile sees
     const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
@@ -159,78 +175,107 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
         if (kb_step > k_hi) break;
         const bool more = kb_step + STEP_KEYS <= k_hi;
         fetch(kb_step + AP_DEPTH * STEP_KEYS, rk[ring], rv[ring]);  // this set's keys are in LDS already
-        const int kb = kb_step + ks * AP_KEYS;  // this wave's block of the step
-        const bf16_t* Ks = Kb + cur * STAGE + ks * AP_KEYS * LDK;
-        const bf16_t* Vs = Vb + cur * VSTAGE + ks * AP_KEYS;
-        if (wave_has && kb <= wave_last) {
-            // S^T[key][query] = sum_d K[key][d] Q[query][d]
-            floatx16 st;
+        const int kb0w = kb_step + ks * NS * AP_KEYS;  // this wave's first block of the step; its NS blocks are consecutive
+        const bf16_t* Ks = Kb + cur * STAGE + ks * NS * AP_KEYS * LDK;
+        const bf16_t* Vs = Vb + cur * VSTAGE + ks * NS * AP_KEYS;
+        if (wave_has && kb0w <= wave_last) {
+            // S^T[key][query] = sum_d K[key][d] Q[query][d], a block a stream. Every slab of the
+            // padded head dimension, without a branch (queries and staged keys are zero past the head
+            // dimension); the reads of LDS go out together, ahead of the products, and the streams'
+            // products alternate. A stream whose block lies past the wave's last query sees every
+            // key masked and changes nothing.
+            floatx16 st[NS];
+            QFrag kf[NS][2 * DB];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) st[r] = 0.0f;
-            // every slab of the padded head dimension, without a branch (queries and staged keys
-            // are zero past the head dimension): the reads of LDS go out together, ahead of the products
-            QFrag kf[2 * DB];
+            for (int z = 0; z < NS; ++z) {
 #pragma unroll
-            for (int s = 0; s < 2 * DB; ++s) kf[s].u = *reinterpret_cast<const u32x4*>(Ks + ql * LDK + 16 * s + 8 * g2);
+                for (int r = 0; r < 16; ++r) st[z][r] = 0.0f;
 #pragma unroll
-            for (int s = 0; s < 2 * DB; ++s) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s].v, qf[s].v, st, 0, 0, 0);
+                for (int sl = 0; sl < 2 * DB; ++sl)
+                    kf[z][sl].u = *reinterpret_cast<const u32x4*>(Ks + (z * AP_KEYS + ql) * LDK + 16 * sl + 8 * g2);
+            }
+#pragma unroll
+            for (int sl = 0; sl < 2 * DB; ++sl)
+#pragma unroll
+                for (int z = 0; z < NS; ++z) st[z] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[z][sl].v, qf[sl].v, st[z], 0, 0, 0);
             // this lane: query ql, keys kb + 8 (r / 4) + 4 g2 + r % 4. A block every query of the
             // wave sees whole needs no mask. The maximum is taken over the raw scores (the scale is
             // positive); exponentials are 2^(score * scale2 - reference), one fused multiply-add and
             // one v_exp_f32 a score.
-            const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * qg && (window <= 0 || kb > wave_last - window);
-            float bm = -INFINITY;
-            if (whole) {
+            float bm[NS];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) bm = fmaxf(bm, st[r]);
-            } else {
+            for (int z = 0; z < NS; ++z) {
+                const int kb = kb0w + z * AP_KEYS;
+                const bool whole = kb + AP_KEYS - 1 <= pos0 + 32 * qg && (window <= 0 || kb > wave_last - window);
+                bm[z] = -INFINITY;
+                if (whole) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
-                    const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
-                    st[r] = ok ? st[r] : -INFINITY;
-                    bm = fmaxf(bm, st[r]);
+                    for (int r = 0; r < 16; ++r) bm[z] = fmaxf(bm[z], st[z][r]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
+                        const bool ok = kp <= qpos && (window <= 0 || kp > qpos - window);
+                        st[z][r] = ok ? st[z][r] : -INFINITY;
+                        bm[z] = fmaxf(bm[z], st[z][r]);
+                    }
                 }
             }
-            bm = fmaxf(bm, __shfl_xor(bm, 32, 64)) * scale2;
-            // the reference m_run is raised only when the block's maximum passes it by more than
+            float other[NS];
+#pragma unroll
+            for (int z = 0; z < NS; ++z) other[z] = __shfl_xor(bm[z], 32, 64);  // the query's other lane: both exchanges in flight together
+            // the reference m_s is raised only when the block's maximum passes it by more than
             // kLag: until then exponentials may reach 2^kLag, which 32-bit sums and bfloat16
             // products hold as well as values below 1
             constexpr float kLag = 8.0f;
-            float corr = 1.0f;
-            if (bm > m_run + kLag) {  // also the first block with a visible key (m_run = -inf)
-                corr = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - bm);
-                m_run = bm;
-            }
-            const float ref = m_run == -INFINITY ? 0.0f : m_run;  // nothing visible yet: every score is -inf, 2^-inf = 0
-            float bs = 0.0f;
-            QFrag pf[2];
+            float corr[NS];
+            QFrag pf[NS][2];
+            bool any = false;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float p = __builtin_amdgcn_exp2f(fmaf(st[r], scale2, -ref));  // 0 for masked keys
-                bs += p;
-                pf[r / 8].h[r % 8] = float_to_bf16(p);
+            for (int z = 0; z < NS; ++z) {
+                const float b = fmaxf(bm[z], other[z]) * scale2;
+                corr[z] = 1.0f;
+                if (b > m_s[z] + kLag) {  // also the first block with a visible key (m_s = -inf)
+                    corr[z] = m_s[z] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_s[z] - b);
+                    m_s[z] = b;
+                }
+                const float ref = m_s[z] == -INFINITY ? 0.0f : m_s[z];  // nothing visible yet: every score is -inf, 2^-inf = 0
+                float bs = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float pr = __builtin_amdgcn_exp2f(fmaf(st[z][r], scale2, -ref));  // 0 for masked keys
+                    bs += pr;
+                    pf[z][r / 8].h[r % 8] = float_to_bf16(pr);
+                }
+                l_s[z] = l_s[z] * corr[z] + bs;  // the reference, and so corr, is the same in both lanes of a query
+                any = any || corr[z] != 1.0f;
             }
-            bs += __shfl_xor(bs, 32, 64);
-            l_run = l_run * corr + bs;
-            const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.0f) != 0;
+            const bool rescale = __builtin_amdgcn_ballot_w64(any) != 0;
             // O^T[d][query] += sum_key V[key][d] P[key][query]; instruction s2 contracts the keys
             // of accumulator registers 8 s2 .. 8 s2 + 7: rows 16 s2 + 4 g2 + {0..3} and + 8
 #pragma unroll
             for (int d = 0; d < DB; ++d) {
                 if (rescale) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o[d][r] *= corr;
-                }
+                    for (int z = 0; z < NS; ++z)
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                    // this lane: dimension 32 d + ql, keys 16 s2 + 4 g2 + {0..3} and the same + 8
-                    union { uint2 u[2]; bf16x8 v; } vf;
-                    const bf16_t* vrow = Vs + (32 * d + ql) * LDV + 16 * s2 + 4 * g2;
-                    vf.u[0] = *reinterpret_cast<const uint2*>(vrow);
-                    vf.u[1] = *reinterpret_cast<const uint2*>(vrow + 8);
-                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[s2].v, o[d], 0, 0, 0);
+                        for (int r = 0; r < 16; ++r) o_s[z][d][r] *= corr[z];
                 }
+                union { uint2 u[2]; bf16x8 v; } vf[NS][2];
+#pragma unroll
+                for (int z = 0; z < NS; ++z)
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        // this lane: dimension 32 d + ql, keys 16 s2 + 4 g2 + {0..3} and the same + 8 of the stream's block
+                        const bf16_t* vrow = Vs + (32 * d + ql) * LDV + z * AP_KEYS + 16 * s2 + 4 * g2;
+                        vf[z][s2].u[0] = *reinterpret_cast<const uint2*>(vrow);
+                        vf[z][s2].u[1] = *reinterpret_cast<const uint2*>(vrow + 8);
+                    }
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                    for (int z = 0; z < NS; ++z)
+                        o_s[z][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[z][s2].v, pf[z][s2].v, o_s[z][d], 0, 0, 0);
             }
         }
         if (more) stash(cur ^ 1, kb_step + STEP_KEYS, rk[(ring + 1) % AP_DEPTH], rv[(ring + 1) % AP_DEPTH]);  // the next step's keys, fetched long ago
@@ -238,6 +283,23 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
         cur ^= 1;
       }
     }
+    // the streams of a wave into the first, in their order; then the two lanes of a query add up
+    // their parts of the sum
+    floatx16 (&o)[DB] = o_s[0];
+    float m_run = m_s[0], l_run = l_s[0];
+#pragma unroll
+    for (int z = 1; z < NS; ++z) {
+        const float M = fmaxf(m_run, m_s[z]);
+        const float wa = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
+        const float wb = m_s[z] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_s[z] - M);
+        l_run = wa * l_run + wb * l_s[z];
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[d][r] = wa * o[d][r] + wb * o_s[z][d][r];
+        m_run = M;
+    }
+    l_run += __shfl_xor(l_run, 32, 64);
     if constexpr (KS > 1) {
         // the query group's partial results, merged into wave (qg, 0) in the order of ks (the
         // walk's last barrier has passed: nobody reads keys or values any more)
@@ -329,9 +391,8 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     auto* pk = static_cast<const bf16_t*>(kc);
     auto* pv = static_cast<const bf16_t*>(vc);
 #define LIYAB_RUN(D, Q, S)                                                                                          \
-    attention_prefill_kernel<D, Q, S><<<grid, 64 * Q * S, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
-                                                                       max_blocks, work, scale, window, n_head, n_kv_head, \
-                                                                       hd, page_size, page_shift)
+    attention_prefill_kernel<D, Q, S, (D <= 2 && Q == 4 && S <= 2) ? 2 : 1><<<grid, 64 * Q * S, 0, stream>>>(                          \
+        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift)
 #define LIYAB_RUN4(D) LIYAB_RUN(D, 2, 4)
 #define LIYAB_SKIP4(D) (void)0  // four stages of 128 keys do not fit LDS at these head sizes (refused above)
 #define LIYAB_GO(D, FOUR)                           \
