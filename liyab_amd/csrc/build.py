@@ -220,6 +220,39 @@ def build_host(quiet: bool = False) -> str:
     return lib
 
 
+# -- the C library over the engine --------------------------------------------------------
+CAPI_DIR = os.path.join(CSRC, "capi")
+CAPI_LIB_NAME = "libliyab_engine.so"
+
+
+def build_engine_capi(quiet: bool = False) -> str:
+    """Builds `capi/liyab_engine_c.cpp` (the engine for C programs: it runs `liyab_amd` in a Python
+    interpreter inside the caller's process) into `_lib/libliyab_engine.so`, linked against this
+    interpreter's library. Returns its path."""
+    import sysconfig
+
+    cxx = cxx_path()
+    if cxx is None:
+        raise RuntimeError("no C++ compiler was found (looked at $CXX, g++, c++, clang++, hipcc)")
+    out_dir = next((d for d in host_lib_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError("no writable folder for the engine's C library: tried " + ", ".join(host_lib_dirs()))
+    include = sysconfig.get_config_var("INCLUDEPY")
+    version = sysconfig.get_config_var("LDVERSION") or sysconfig.get_config_var("VERSION")
+    libdirs = [d for d in (sysconfig.get_config_var("LIBDIR"), sysconfig.get_config_var("LIBPL")) if d]
+    lib = os.path.join(out_dir, CAPI_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-I", include, "-I", CAPI_DIR, "-o", tmp,
+           os.path.join(CAPI_DIR, "liyab_engine_c.cpp"), *[f"-L{d}" for d in libdirs], f"-lpython{version}", "-ldl",
+           *[f"-Wl,-rpath,{d}" for d in libdirs]]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building {CAPI_LIB_NAME} failed:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, lib)
+    _say(f"built {lib}", quiet)
+    return lib
+
+
 def build_host_selftest(sanitize: bool = True, out_dir: Optional[str] = None) -> str:
     """Compiles `host/selftest/selftest.cpp` with the host sources into an executable of its own
     and returns its path. `sanitize`: with the address and undefined-behaviour sanitizers
