@@ -459,7 +459,10 @@ int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, co
 using namespace liyab;
 
 // tile: 2 = 64x64 tiles, three stages deep, on four waves; 6 = the same with four stages; 8 = 128x128, two
-// stages, on eight waves; 16 = 64x32 on four groups of two waves that walk K side by side, three stages of
+// stages, on eight waves; 17 = 32x32 on four waves that walk K side by side (a workgroup then brings in a
+// third less of the operands, and twice as many workgroups pull: 64 rows with cold weights, 768 -> 2,304 in
+// 5.05 us against 5.53, 1,024 -> 3,072 in 5.97 against 6.85; for as long as every tile has a compute unit
+// of its own: 1,600 -> 4,800 in 13.9 against 9.7); 16 = 64x32 on four groups of two waves that walk K side by side, three stages of
 // four units (for one tile of rows: 8.2 us for 64 x 4,800 x 1,600 where two waves walking K alone, four
 // stages deep, took 10.3; deeper rings for those took longer, 11.1 with eight stages: the walk waits on
 // its own chain of load, barrier, fragments and products, not on the loads in flight); 0 = chosen from
@@ -485,6 +488,7 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 16: return launch_dl<64, 32, 3, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
+        case 17: return launch_dl<32, 32, 3, 1, 1, 4>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }
@@ -492,7 +496,7 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
 // The same product cut over K: parts[p * part_stride + m * N + n] = sum over the p-th of `kparts` parts
 // of K (whole tiles of 64) of a[m, k] w[n, k]. With `base` (n_base planes [M, N], base_stride floats
 // apart, not overlapping `parts`) the first plane also takes bias[n] and base[0] + base[1] + ...;
-// without it `bias` must be null. tile: 6 = 64x64 tiles, 16 = 64x32 (for one tile of rows).
+// without it `bias` must be null. tile: 6 = 64x64 tiles, 16 = 64x32 (for one tile of rows), 17 = 32x32.
 extern "C" int liyab_gemm_mfma_dl_parts(const void* a, int64_t lda, const void* w, int M, int N, int K, int kparts, int tile,
                                         float* parts, int64_t part_stride, const float* bias, const float* base, int n_base,
                                         int64_t base_stride, hipStream_t stream) {
@@ -526,5 +530,6 @@ extern "C" int liyab_gemm_mfma_dl_parts(const void* a, int64_t lda, const void* 
     auto* pw = static_cast<const bf16_t*>(w);
     if (tile == 6) return launch_dl_parts<64, 64, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
     if (tile == 16) return launch_dl_parts<64, 32, 3, 2, 1, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
-    return fail(1, "gemm_mfma_dl_parts: unknown tile %d (6 or 16)", tile);
+    if (tile == 17) return launch_dl_parts<32, 32, 3, 1, 1, 4>(pa, lda, pw, M, N, K, kparts, epi, pp, stream);
+    return fail(1, "gemm_mfma_dl_parts: unknown tile %d (6, 16 or 17)", tile);
 }

@@ -472,7 +472,7 @@ def gemm_mfma_dl_parts(a: torch.Tensor, w: torch.Tensor, planes: torch.Tensor, *
                        base: Optional[torch.Tensor] = None, tile: int = 6) -> None:
     """The tiled matrix-core product cut over K (K a multiple of 64), as `gemm_skinny_parts` for
     any number of rows: planes float32 [parts, M, N]; with `base` the first plane also takes
-    `bias` and the rows of `base`. tile: 6 = 64 x 64 tiles, 16 = 64 x 32."""
+    `bias` and the rows of `base`. tile: 6 = 64 x 64 tiles, 16 = 64 x 32, 17 = 32 x 32."""
     lda = _rows(a, "a")
     M, K = a.shape
     _dev(w, "w")
@@ -676,7 +676,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             # tiles of rows as long as every tile has a compute unit of its own (the stages fill
             # a unit's LDS; 128 rows: 6.1 against 7.7 us for 768 -> 2,304 in 64 x 64 tiles; with
             # more tiles than units, 400 rows: 10.7 against 8.0)
-            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=16)
+            # tiles of 32 x 32 while each has a compute unit of its own: a workgroup brings in a third
+            # less of the operands and twice as many pull (64 rows, cold weights: 5.05 against 5.53 us
+            # for 768 -> 2,304, 5.97 against 6.85 for 1,024 -> 3,072; 13.9 against 9.7 for 1,600 -> 4,800)
+            small = (M + 31) // 32 * ((N + 31) // 32) <= compute_units()
+            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=17 if small else 16)
         elif M <= 16 or (M <= 64 and N <= 8192):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
             # kernel's shared loads beat every workgroup re-reading the tokens)

@@ -97,7 +97,8 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
         # 64 x 32 tiles while every tile of every part has a compute unit of its own (128 rows,
         # 3,072 -> 768 in four parts: 6.5 against 7.5 us in 64 x 64 tiles), 64 x 64 tiles beyond
         few = (M + 63) // 64 * ((w.shape[0] + 31) // 32) * parts <= ops.compute_units()
-        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=16 if M <= 64 or few else 6)
+        fewer = (M + 31) // 32 * ((w.shape[0] + 31) // 32) * parts <= ops.compute_units()  # 32 x 32 tiles each on a compute unit of its own
+        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=17 if fewer else (16 if M <= 64 or few else 6))
     else:
         ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
     return SplitStream(planes, stream.home if split else stream)

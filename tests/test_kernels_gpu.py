@@ -144,7 +144,7 @@ def test_gemm_skinny_parts(ops, M, N, K, parts):
         ops.gemm_skinny_parts(a, w, planes, base=planes[:1])
 
 
-@pytest.mark.parametrize("tile", [6, 16])
+@pytest.mark.parametrize("tile", [6, 16, 17])
 @pytest.mark.parametrize("M,N,K,parts", [(64, 768, 3072, 4), (2048, 768, 3072, 2), (200, 100, 448, 3), (33, 1600, 6400, 4), (1, 40, 64, 1),
                                          (130, 777, 1088, 5)])
 def test_gemm_tiled_parts(ops, tile, M, N, K, parts):
@@ -213,7 +213,7 @@ def test_gemm_float32(ops, M, N, K, epilogue):
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
-                                    "dl2", "dl6", "dl8", "dl16"])
+                                    "dl2", "dl6", "dl8", "dl16", "dl17"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
                                                  (500, 300, 128), (129, 193, 192), (20, 4800, 1600)])
