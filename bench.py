@@ -175,6 +175,27 @@ def link_floor(device="cuda:0", links=100):
     return {"metric": "microseconds a dependent kernel of a replayed graph", "links": links, "us_per_link": out}
 
 
+def copy_bandwidth(device="cuda:0", mbytes=1024, repeat=5):
+    """GB/s of a device-to-device copy of `mbytes` (bytes read plus bytes written over the best
+    time): what this machine's memory gives a plain stream, beside the published peak that the
+    roofline shares are taken against (the reference measures its read ceiling the same way,
+    tools/liyab_bench.cpp:1-9)."""
+    import torch
+
+    n = mbytes * (1 << 20) // 4
+    a = torch.empty(n, dtype=torch.float32, device=device).normal_()
+    b = torch.empty_like(a)
+    best = float("inf")
+    for _ in range(repeat + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        b.copy_(a)
+        e1.record()
+        e1.synchronize()
+        best = min(best, e0.elapsed_time(e1))
+    return 2.0 * n * 4 / (best * 1e-3) / 1e9
+
+
 def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
     """Best of `repeat`: (tokens/s, ms) of one step that holds the whole prompts."""
     import numpy as np
@@ -353,6 +374,8 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4)},
         }
+        if not args.no_points:
+            out["roofline"]["measured_copy"] = round(copy_bandwidth(), 1)  # a 1 GiB device-to-device copy on this machine, GB/s
         if not args.no_points:
             lens = [1024, 1024]
             ptps, pms = prefill_run(engine, cfg, lens)
