@@ -7,6 +7,8 @@
 // starts is 32-bit on both paths.
 #include "common.h"
 
+#include <algorithm>
+
 namespace liyab {
 
 // An id below zero is a reference: -1 - id indexes `last_tokens`, where the sampler left the
@@ -60,9 +62,47 @@ __global__ void kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc, const T*
     }
 }
 
+// out[r] = x[rows[r]] (or x[r]) in the output's precision: the rows whose logits are wanted, for a
+// head that no norm stands before (a norm gathers them itself).
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows, int d) {
+    const int r = blockIdx.x;
+    const float* src = x + static_cast<int64_t>(rows != nullptr ? rows[r] : r) * d;
+    T* dst = out + static_cast<int64_t>(r) * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = from_float<T>(src[i]);
+}
+
+// p[i] *= scale (logits times a model's logit scale, the reference's finish_logits,
+// src/core/transformer.cpp:2613-2620)
+__global__ void scale_kernel(float* __restrict__ p, float scale, int64_t n) {
+    int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (; i < n; i += step) p[i] *= scale;
+}
+
 }  // namespace liyab
 
 using namespace liyab;
+
+extern "C" int liyab_gather_rows(void* out, int out_dtype, const float* x, const int* rows, int n, int d, hipStream_t stream) {
+    LIYAB_REQUIRE(out && x, "gather_rows: null pointer");
+    LIYAB_REQUIRE(d > 0 && n >= 0, "gather_rows: bad sizes n=%d d=%d", n, d);
+    LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "gather_rows: unknown dtype %d", out_dtype);
+    if (n == 0) return 0;
+    const int threads = d >= 256 ? 256 : 64;
+    if (out_dtype == kF32) gather_rows_kernel<float><<<n, threads, 0, stream>>>(static_cast<float*>(out), x, rows, d);
+    else gather_rows_kernel<bf16_t><<<n, threads, 0, stream>>>(static_cast<bf16_t*>(out), x, rows, d);
+    return check_launch("gather_rows");
+}
+
+extern "C" int liyab_scale(float* p, float scale, int64_t n, hipStream_t stream) {
+    LIYAB_REQUIRE(p != nullptr || n == 0, "scale: null pointer");
+    LIYAB_REQUIRE(n >= 0, "scale: negative count");
+    if (n == 0) return 0;
+    const int blocks = static_cast<int>(std::min<int64_t>((n + 255) / 256, 4096));
+    scale_kernel<<<blocks, 256, 0, stream>>>(p, scale, n);
+    return check_launch("scale");
+}
 
 extern "C" int liyab_embed(float* x, const void* tok, const void* pos, int dtype, const int* ids, const int* positions,
                            int n, int d, float scale, const int* last_tokens, hipStream_t stream) {

@@ -38,6 +38,8 @@ _SIGNATURES = {
     "liyab_add_into": [P, P, c_int, c_int64, P],
     "liyab_embed": [P, P, P, c_int, P, P, c_int, c_int, c_float, P, P],
     "liyab_add_rows": [P, P, c_int, P, c_int, c_int, P],
+    "liyab_gather_rows": [P, c_int, P, P, c_int, c_int, P],
+    "liyab_scale": [P, c_float, c_int64, P],
     "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
     "liyab_layernorm": [P, c_int, P, P, P, P, c_int, c_int, c_float, P],
     "liyab_layernorm_parts": [P, c_int, P, c_int, c_int64, c_int, P, P, P, c_int, c_int, c_float, P],

@@ -189,6 +189,29 @@ def add_rows_(x: torch.Tensor, table: torch.Tensor, rows: torch.Tensor) -> None:
     _lib.call("liyab_add_rows", x.data_ptr(), table.data_ptr(), dtype_code(table.dtype), rows.data_ptr(), n, d, _stream())
 
 
+def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = x[rows[r]] (x[r] without rows) in out's dtype; x float32 [*, d], out [n, d]."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = out.shape
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"gather_rows: x must be contiguous float32 [*, {d}] and out contiguous, got {tuple(x.shape)} {x.dtype}")
+    if rows is not None:
+        _i32(rows, "rows", n)
+    elif x.shape[0] < n:
+        raise KernelError("gather_rows: fewer input rows than output rows")
+    _lib.call("liyab_gather_rows", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(rows), n, d, _stream())
+
+
+def scale_(t: torch.Tensor, scale: float) -> torch.Tensor:
+    """t *= scale; t contiguous float32."""
+    _dev(t, "scale target")
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        raise KernelError("scale: the target must be contiguous float32")
+    _lib.call("liyab_scale", t.data_ptr(), float(scale), t.numel(), _stream())
+    return t
+
+
 def _planes(x: torch.Tensor, what: str):
     """Rows given as they are, float32 [rows, d], or as a sum of planes, float32 [parts, rows, d]
     (row r is x[0][r] + x[1][r] + ..., added in that order). Returns (pointer, parts, floats

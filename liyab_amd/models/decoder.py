@@ -121,5 +121,8 @@ class DecoderModel:
                 rows = pending.planes if takes is not None and takes(pending.planes) else pending.settle()
             h = norm.lazy(rows, ctx, **kw) if hasattr(norm, "lazy") else norm.forward(rows, ctx, **kw)
         else:
-            raise NotImplementedError("a model without a final norm is not implemented")
+            # no norm before the head: the wanted rows of the stream as they are, in the compute dtype
+            rows = pending.settle() if pending is not None else x
+            h = ctx.workspace.get("head_in", (ctx.n_logit_rows, self.width), self.dtype)
+            ops.gather_rows(h, rows, ctx.logit_rows)
         return self.head.forward(h, ctx)

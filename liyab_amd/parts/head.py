@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import ops
 from .base import StepContext
 from .linear import linear
 from .registry import register_head
@@ -19,8 +20,6 @@ class LMHead:
     def __init__(self, spec, store, dtype: torch.dtype):
         self.width, self.vocab_size = spec.width, spec.vocab_size
         self.logit_scale = float(spec.logit_scale)
-        if self.logit_scale != 1.0:
-            raise NotImplementedError("a logit scale other than 1 is not implemented")
         t = spec.tensors
         self.weight = store.fetch(t["weight"], (self.vocab_size, self.width), "table")
         self.bias = store.fetch(t["bias"], (self.vocab_size,), "vector") if "bias" in t else None
@@ -28,6 +27,8 @@ class LMHead:
     def forward(self, h, ctx: StepContext) -> torch.Tensor:
         logits = ctx.workspace.get("logits", (h.shape[0], self.vocab_size), torch.float32)
         linear(h, self.weight, self.bias, out=logits)
+        if self.logit_scale != 1.0:
+            ops.scale_(logits, self.logit_scale)  # after the bias, as the reference's finish_logits does (:2613-2620)
         return logits
 
 

@@ -735,3 +735,28 @@ def test_drawn_shapes_of_the_folded_and_the_cut_products(ops, seed):
             planes = torch.full((parts, M, N), float("nan"), device=DEV)
             ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=rng.choice([6, 16]))
             close(planes.double().sum(0), want, 1e-5, f"tiled product in parts M={M} K={K} N={N} parts={parts}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,d,indexed", [(1, 16, True), (7, 100, True), (33, 1600, False), (5, 257, True)])
+def test_gather_rows(dtype, n, d, indexed):
+    """out[r] = x[rows[r]] in the output's dtype; without rows the first n rows."""
+    from liyab_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(n * 1000 + d)
+    x = torch.randn(n + 9, d, generator=g).to(DEV)
+    rows = torch.randint(0, n + 9, (n,), generator=g, dtype=torch.int32).to(DEV) if indexed else None
+    out = torch.full((n, d), 7.0, dtype=dtype, device=DEV)
+    ops.gather_rows(out, x, rows)
+    want = (x[rows.long()] if indexed else x[:n]).to(dtype)
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("n", [1, 255, 50257 * 3, 4096 * 256 + 5])
+def test_scale_in_place(n):
+    from liyab_amd.kernels import ops
+
+    x = torch.randn(n, generator=torch.Generator().manual_seed(n)).to(DEV)
+    want = x * 0.37
+    ops.scale_(x, 0.37)
+    assert torch.equal(x, want)

@@ -774,6 +774,49 @@ def test_toy_position_encoding_inside_attention(dtype):
         assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_head_without_a_norm_before_it_with_a_bias_and_a_logit_scale(dtype):
+    """The plan's last two options, as data: no norm before the head (the wanted rows of the stream
+    go to the product as they are) and logits times a scale, after the bias
+    (src/core/transformer.cpp:2613-2620). The plain formula here is the turned toy's without its
+    last norm; that bias and scale are in it shows in the difference from the unscaled one."""
+    import dataclasses
+
+    from liyab_amd.config import HeadSpec
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = turned_model(dtype)
+    scale = 0.37
+    tw = {k: v for k, v in tw.items() if not k.startswith("nf.")}  # the loader refuses tensors that nobody reads
+    tw["head_bias"] = rand(np.random.default_rng(77), info["V"], scale=0.5)
+    plan = dataclasses.replace(plan, final_norm=None, head=HeadSpec("lm_head", info["d"], info["V"], scale,
+                                                                    {"weight": T("emb"), "bias": T("head_bias")}))
+
+    def plain_logits(ids):
+        eps = info["eps"]
+        rot = lambda hd, base: (lambda x, heads: plain_turn(x, heads, hd, base, 0))
+        x = f64(tw["emb"])[ids]
+        a, _ = plain_attention(plain_norm(x, tw, "n0a", eps), tw, "a0", 4, 2, 32, 0.2, rotate=rot(32, 100.0))
+        x = x + a
+        x = x + plain_ffn(plain_norm(x, tw, "n0b", eps), tw, "f0", "gelu_tanh")
+        a, _ = plain_attention(plain_norm(x, tw, "n1a", eps), tw, "a1", 3, 3, 16, 0.3, window=20, rotate=rot(16, 10000.0))
+        x = x + a
+        x = x + plain_ffn(plain_norm(x, tw, "n1b", eps), tw, "f1", "gelu_erf")
+        if dtype == "bfloat16":  # the product reads the stream in the compute dtype
+            x = torch.from_numpy(x).to(torch.bfloat16).double().numpy()
+        return (x @ f64(tw["emb"]).T + f64(tw["head_bias"])) * scale
+
+    reqs = {f"h{i}": tt.random_tokens(60 + i, n, info["V"]) for i, n in enumerate([45, 130, 3, 71])}
+    ref = {rid: plain_logits(toks) for rid, toks in reqs.items()}
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3, 40))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=9))):
+        core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        assert core.model.final_norm is None and core.model.head.logit_scale == scale
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, TOL_TOY[dtype], f"bare head {name} {dtype}", family="toy:bare_head")
+        core.manager.check()
+
+
 # ---------------------------------------------------------------------------
 # a toy mixer that brings its own words of a step's metadata, under graphs and the scheduler
 # ---------------------------------------------------------------------------
