@@ -252,6 +252,12 @@ sample_kernel(int* __restrict__ out, const float* __restrict__ logits, int64_t l
 constexpr int kMassBits = 44;
 constexpr int kWaveCandidates = 64;
 constexpr int kPool = 1024;  // keys that may be among the k largest, for one wave to choose from
+// Top-p over many candidates: masses are first added up in bins by the logit's distance below
+// the largest, kBins of them over the 44 powers of two that a mass can lie under the largest
+// (a bin is a monotone function of the key, so the bins are intervals of the descending order).
+constexpr int kBins = 2048;
+constexpr int kBinPad = 32;  // one word of padding every 32 bins: a lane's 32 bins in a row, the lanes' on different banks
+__device__ __forceinline__ int bin_slot(int b) { return b + b / kBinPad; }
 
 __device__ __forceinline__ unsigned long long fixed_mass(uint32_t key, float lmax, float scale2) {
     // exp((l - l_max) / T) through the hardware's 2^x (scale2 = log2(e) / T), in [0, 1]; times
@@ -351,6 +357,12 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     __shared__ int pool_id[kPool];
     __shared__ int n_pool;
     __shared__ uint32_t pool_floor;
+    // top-p over many candidates: the bins' masses, and what one wave finds for all
+    __shared__ unsigned long long bin_mass[PLAIN ? 1 : kBins + kBins / kBinPad];
+    __shared__ unsigned long long bins_above;
+    __shared__ double bins_target;
+    __shared__ int bin_star, bins_ok, found_ties;
+    __shared__ uint32_t found_tau;
 
     const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const float* row = logits + static_cast<int64_t>(r) * ld;
@@ -417,7 +429,12 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     auto kept_bits = [&](uint32_t t, int ties, uint32_t (&bits)[(EPT + 31) / 32]) {
         int n_ties = 0;
 #pragma unroll
-        for (int j = 0; j < EPT; ++j) n_ties += keys[j] == t && keys[j] != 0u;
+        for (int j = 0; j < EPT; ++j) {
+            // (compared afresh: the same comparisons come again in the ranks below, and kept from here to
+            // there they are a lane mask an id, more scalar registers than there are)
+            const uint32_t key = again(keys[j]);
+            n_ties += key == t && key != 0u;
+        }
         const int all_ties = block_count<WAVES>(n_ties, redi);
 #pragma unroll
         for (int w = 0; w < (EPT + 31) / 32; ++w) bits[w] = 0u;
@@ -457,7 +474,8 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
 
     uint32_t bits[(EPT + 31) / 32];
     // is id j of this thread kept? (PLAIN: every element of the row is)
-    auto is_kept = [&](int j) { return PLAIN ? keys[j] != 0u : ((bits[j / 32] >> (j % 32)) & 1u) != 0u; };
+    // (the word of bits is read afresh each time, for the same reason: no lane mask an id is kept between the passes)
+    auto is_kept = [&](int j) { return PLAIN ? keys[j] != 0u : ((again(bits[j / 32]) >> (j % 32)) & 1u) != 0u; };
     if constexpr (!PLAIN) {
     // ---- one wave among at most 64 candidates in cand_key / cand_id: nucleus cut and draw ----
     auto wave_finish = [&]() {
@@ -634,7 +652,145 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     // ---- top-p over many candidates: the key where the descending cumulative mass reaches top_p ----
     uint32_t tau = tau_k;
     int ties = ties_k;
+    bool cut_found = false;
     if (use_p) {
+        // ---- by bins: one pass adds the masses up in bins, one wave finds the bin in which the
+        // descending cumulative mass reaches top_p, the keys of that bin alone are gathered, and the
+        // same wave finds the key among them. The sums are integers, so the bins' total and every
+        // prefix are the sums the bisection below would find, and so are the key and the ties kept.
+        // A bin with more keys than the pool holds (thousands of nearly equal logits), or nothing
+        // to cut, leaves it to the bisection.
+        const unsigned long long tie_mass = use_k ? static_cast<unsigned long long>(ties_k) * fixed_mass(tau_k, lmax, inv_t) : 0ull;
+        auto bin_of = [&](uint32_t key) {
+            const float below = (lmax - key_value(key)) * inv_t;  // powers of two under the largest mass, >= 0
+            return static_cast<int>(fminf(below * (static_cast<float>(kBins) / kMassBits), static_cast<float>(kBins - 1)));
+        };
+        for (int i = tid; i < kBins + kBins / kBinPad; i += THREADS) bin_mass[i] = 0ull;
+        if (tid == 0) bins_ok = 0;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            const uint32_t key = again(keys[j]);
+            if (key != 0u && key > tau_k) {
+                const unsigned long long m = fixed_mass(key, lmax, inv_t);
+                if (m != 0ull) atomicAdd(&bin_mass[bin_slot(bin_of(key))], m);
+            }
+        }
+        if (tid == 0 && tie_mass != 0ull) atomicAdd(&bin_mass[bin_slot(bin_of(tau_k))], tie_mass);
+        __syncthreads();
+        if (wave == 0) {
+            constexpr int PER_LANE = kBins / kWave;
+            unsigned long long mine_sum = 0;
+#pragma unroll
+            for (int i = 0; i < PER_LANE; ++i) mine_sum += bin_mass[bin_slot(lane * PER_LANE + i)];
+            unsigned long long incl = mine_sum;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                const unsigned long long o = shfl_up_u64(incl, d);
+                if (lane >= d) incl += o;
+            }
+            const unsigned long long total = lane_value64(incl, kWave - 1);
+            const double target = static_cast<double>(tp) * static_cast<double>(total);
+            const unsigned long long reached = __ballot(static_cast<double>(incl) >= target);
+            if (total > 0ull && target > 0.0 && reached != 0ull && lane == __ffsll(static_cast<long long>(reached)) - 1) {
+                unsigned long long cum = incl - mine_sum;
+                for (int i = 0; i < PER_LANE; ++i) {
+                    const unsigned long long next = cum + bin_mass[bin_slot(lane * PER_LANE + i)];
+                    if (static_cast<double>(next) >= target) {
+                        bin_star = lane * PER_LANE + i;
+                        bins_above = cum;
+                        bins_target = target;
+                        bins_ok = 1;
+                        break;
+                    }
+                    cum = next;
+                }
+            }
+        }
+        __syncthreads();
+        if (bins_ok != 0) {
+            const int star = bin_star;
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const uint32_t key = again(keys[j]);
+                if (key != 0u && key > tau_k && bin_of(key) == star) {
+                    const int at = atomicAdd(&n_pool, 1);  // the order of arrival does not matter: only keys count here
+                    if (at < kPool) pool_key[at] = key;
+                }
+            }
+            __syncthreads();
+            const int n = n_pool;
+            if (n <= kPool) {
+                if (wave == 0) {
+                    constexpr int PER = kPool / kWave;
+                    const bool k_here = tie_mass != 0ull && bin_of(tau_k) == star;  // the top-k ties lie in this bin
+                    const unsigned long long k_mass = k_here ? tie_mass : 0ull;
+                    uint32_t pk[PER];  // (their masses are taken again wherever they are needed: registers are short here)
+                    auto pm = [&](int i) { return pk[i] != 0u ? fixed_mass(again(pk[i]), lmax, inv_t) : 0ull; };
+                    uint32_t lo = k_here ? tau_k : 0xffffffffu, hi = k_here ? tau_k : 0u;
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        const int e = lane + kWave * i;
+                        pk[i] = e < n ? pool_key[e] : 0u;
+                        if (e < n) { lo = min(lo, pk[i]); hi = max(hi, pk[i]); }
+                    }
+#pragma unroll
+                    for (int off = kWave / 2; off > 0; off >>= 1) {
+                        lo = min(lo, static_cast<uint32_t>(__shfl_xor(static_cast<int>(lo), off, kWave)));
+                        hi = max(hi, static_cast<uint32_t>(__shfl_xor(static_cast<int>(hi), off, kWave)));
+                    }
+                    const unsigned long long above_bin = bins_above;
+                    const double target = bins_target;
+                    // the largest key whose mass from it upwards reaches the target: it lies in this bin,
+                    // so only the bits in which the bin's keys differ are open
+                    const int open_bits = lo == hi ? 0 : 32 - __clz(lo ^ hi);
+                    uint32_t tau_p = open_bits >= 32 ? 0u : (hi >> open_bits) << open_bits;
+                    for (int bit = open_bits - 1; bit >= 0; --bit) {
+                        const uint32_t cand = tau_p | (1u << bit);
+                        unsigned long long m = 0;
+#pragma unroll
+                        for (int i = 0; i < PER; ++i)
+                            if (i * kWave < n) m += pk[i] >= cand ? pm(i) : 0ull;  // (the same for the whole wave: a bin mostly holds far fewer keys than the pool)
+                        m = wave_sum_u64(m) + (k_here && tau_k >= cand ? k_mass : 0ull) + above_bin;
+                        if (static_cast<double>(m) >= target) tau_p = cand;
+                    }
+                    unsigned long long above = 0;
+                    int avail = 0;
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        if (i * kWave < n) {
+                            above += pk[i] > tau_p ? pm(i) : 0ull;
+                            avail += __popcll(__ballot(pk[i] == tau_p && pk[i] != 0u));
+                        }
+                    }
+                    above = wave_sum_u64(above) + above_bin;
+                    if (k_here && tau_p == tau_k) avail = ties_k;
+                    // the prefix grows one tie at a time until its share reaches top_p
+                    const unsigned long long p_tie = fixed_mass(tau_p, lmax, inv_t);
+                    int need = 1;
+                    if (p_tie > 0ull) {
+                        unsigned long long cum = above;
+                        need = 0;
+                        while (need < avail) {
+                            cum += p_tie;
+                            ++need;
+                            if (static_cast<double>(cum) >= target) break;
+                        }
+                        if (need < 1) need = 1;
+                    }
+                    if (lane == 0) {
+                        found_tau = tau_p;
+                        found_ties = need < avail ? need : avail;
+                    }
+                }
+                __syncthreads();
+                tau = found_tau;
+                ties = found_ties;
+                cut_found = true;
+            }
+        }
+    }
+    if (use_p && !cut_found) {
         const unsigned long long tie_mass_k = use_k ? static_cast<unsigned long long>(ties_k) * fixed_mass(tau_k, lmax, inv_t) : 0ull;
         // mass of {key >= cand} within the top-k set (ties at tau_k counted ties_k times)
         auto mass_ge = [&](uint32_t cand) -> unsigned long long {

@@ -571,7 +571,7 @@ def test_argmax_ties_go_to_the_lowest_id(ops, rows, V):
     assert out.tolist() == rnd(rows, V, seed=4).argmax(dim=1).tolist()
 
 
-@pytest.mark.parametrize("V", [1000, 50257, 70001])
+@pytest.mark.parametrize("V", [1000, 50257, 60000, 70001])
 def test_sampler_against_the_plain_sampler(ops, V):
     """Temperature, top-k and top-p per row against the plain implementation's rules, at
     vocabularies that take each of the sampling kernels (the row in registers with a one-wave
@@ -602,6 +602,55 @@ def test_sampler_against_the_plain_sampler(ops, V):
             if got[r] != want:
                 cdf = np.cumsum(probs)
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, params[r], got[r], want)
+
+
+@pytest.mark.parametrize("V", [3000, 50257, 65533])
+def test_top_p_over_many_candidates_keeps_exactly_the_nucleus(ops, V):
+    """Top-p alone (and with a top-k too wide for one wave) at rows made so that a wrong cut shows
+    in the draws: a few heavy ids over a light floor, the cut falling between them, inside a run
+    of ties (the lowest ids of the run are kept), on the top-k boundary's ties, in a flat row where
+    every key shares a bin, and in a peaked row whose masses span every bin. 48 draws a row are
+    compared with the plain sampler's; a draw may differ only where the uniform number lies
+    within rounding of a boundary between two ids."""
+    import plain_gpt2 as plain
+
+    g = torch.Generator().manual_seed(V)
+    cases = []  # (logits row, temperature, top_k, top_p)
+    floor = torch.randn(V, generator=g) * 0.5 - 12.0
+    heavy = floor.clone()
+    heavy[[5, 900, 1777, 2500, 40, 41]] = torch.tensor([3.0, 2.9, 2.5, 2.45, 1.0, 0.9])
+    for p in (0.2, 0.4, 0.63, 0.8, 0.97, 0.99999):
+        cases.append((heavy, 1.0, 0, p))
+    ties = floor.clone()
+    ties[[10, 20, 30]] = 6.0
+    ties[100:2100:250] = 5.0  # eight ties: the cut falls among them
+    for p in (0.3, 0.5, 0.7, 0.85, 0.95):
+        cases.append((ties, 1.0, 0, p))
+    cases.append((ties, 0.5, 0, 0.9))
+    wide = torch.randn(V, generator=g) * 2.0
+    wide[200:330] = 4.0  # 130 ties on the boundary of top-k 100: 100 - (keys above) of them are in the set
+    for k, p in ((100, 0.5), (100, 0.9), (100, 0.999), (400, 0.3), (V - 1, 0.6)):
+        cases.append((wide, 1.0, k, p))
+    cases.append((torch.full((V,), 0.25), 1.0, 0, 0.5))  # every key in one bin: more than the pool holds
+    cases.append((torch.randn(V, generator=g) * 0.01, 1.0, 0, 0.9))  # nearly flat: a few bins hold the row
+    peaked = torch.linspace(0.0, -40.0, V)[torch.randperm(V, generator=g)]
+    for T, p in ((1.0, 0.9), (0.3, 0.5), (3.0, 0.95)):
+        cases.append((peaked, T, 0, p))
+    draws = 48
+    for row, T, k, p in cases:
+        logits = row.to(DEV).repeat(draws, 1)
+        u = [plain.uniform(1000 + k, i) for i in range(draws)]
+        u[0], u[1] = 0.0, 1.0 - 2.0 ** -40  # the first and the last id that are kept
+        out = torch.empty(draws, dtype=torch.int32, device=DEV)
+        ops.sample(out, logits, torch.full((draws,), T, dtype=torch.float32, device=DEV),
+                   torch.full((draws,), k, dtype=torch.int32, device=DEV),
+                   torch.full((draws,), p, dtype=torch.float32, device=DEV), torch.tensor(u, dtype=torch.float64, device=DEV))
+        probs = plain.probabilities(row.numpy(), T, k, p)
+        cdf = np.cumsum(probs)
+        for i, got in enumerate(out.tolist()):
+            want = plain.sample(probs, u[i])
+            if got != want:
+                assert probs[got] > 0 and np.abs(cdf - u[i]).min() < 1e-5, (V, T, k, p, i, got, want)
 
 
 @pytest.mark.parametrize("V", [1000, 50257, 70001])
