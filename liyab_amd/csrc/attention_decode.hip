@@ -1,6 +1,6 @@
 // Attention for tokens taken one at a time (decoding, short prompt portions)
-// over paged bfloat16 keys and values, with the keys of a token cut into
-// splits so that few tokens still fill the chip.
+// over paged keys and values (bfloat16, or 32-bit for the 32-bit path), with
+// the keys of a token cut into splits so that few tokens still fill the chip.
 //
 // Grid (token, query head, split). A workgroup of 4 or 16 waves walks its split's
 // keys; LPK lanes share a key (each holds 8 consecutive dimensions, 16
@@ -9,6 +9,8 @@
 // weighted values (the reference's per-span partial softmax,
 // src/core/transformer.cpp:2327-2358); groups, then waves, then splits are
 // merged in a fixed order by rescaling to the common maximum (:2367-2385).
+// With one split on four waves which lane adds which key follows from the
+// token's position alone: the form the 32-bit path always takes.
 // The reference cuts a token's keys by its position only (:2136-2139,
 // 2225-2227) to keep bits equal; here the number of splits follows the batch
 // (more splits when few tokens are in flight), which moves results by
@@ -30,26 +32,44 @@ __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
     }
 }
 
+// 8 consecutive elements of a row as they are loaded (bfloat16 stays packed until it is used), and as floats
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+struct Raw8F { f32x4 a, b; };
+__device__ __forceinline__ u32x4 fetch8(const bf16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ Raw8F fetch8(const float* p) {
+    return Raw8F{*reinterpret_cast<const f32x4*>(p), *reinterpret_cast<const f32x4*>(p + 4)};
+}
+__device__ __forceinline__ void unpack8(const Raw8F& v, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f[i] = v.a[i]; f[4 + i] = v.b[i]; }
+}
+template <typename T> struct Raw8 { typedef u32x4 type; };
+template <> struct Raw8<float> { typedef Raw8F type; };
+// exponentials of scores: the fast one beside bfloat16 data, the library's beside 32-bit data
+template <typename T> __device__ __forceinline__ float exp_for(float x) { return __expf(x); }
+template <> __device__ __forceinline__ float exp_for<float>(float x) { return expf(x); }
+
 struct Partial {
     float m, l;
     float acc[8];
 };
 
 // this <- merge(this, other): both rescaled to the larger maximum; this comes first.
+template <typename T>
 __device__ __forceinline__ void merge_partial(Partial& a, float mo, float lo, const float* acco) {
     const float M = fmaxf(a.m, mo);
-    const float wa = a.m == -INFINITY ? 0.0f : __expf(a.m - M);
-    const float wb = mo == -INFINITY ? 0.0f : __expf(mo - M);
+    const float wa = a.m == -INFINITY ? 0.0f : exp_for<T>(a.m - M);
+    const float wb = mo == -INFINITY ? 0.0f : exp_for<T>(mo - M);
     a.l = wa * a.l + wb * lo;
 #pragma unroll
     for (int e = 0; e < 8; ++e) a.acc[e] = wa * a.acc[e] + wb * acco[e];
     a.m = M;
 }
 
-template <int LPK, int AD_WAVES, int AD_U>
+template <typename T, int LPK, int AD_WAVES, int AD_U>
 __global__ void __launch_bounds__(64 * AD_WAVES)
-attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
-                        const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
+                        const T* __restrict__ kc, const T* __restrict__ vc,
                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
                         int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
@@ -73,10 +93,10 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
     // lanes past the head dimension read column 0 and multiply it by a zero query
     const int col = active ? c * 8 : 0;
     float qf[8];
-    {
-        u32x4 qv = *reinterpret_cast<const u32x4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * hd + col);
-        if (!active) qv = u32x4{0, 0, 0, 0};
-        unpack8(qv, qf);
+    unpack8(fetch8(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * hd + col), qf);
+    if (!active) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[e] = 0.0f;
     }
     __syncthreads();
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
@@ -92,7 +112,7 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
     const int64_t head_off = static_cast<int64_t>(hkv) * page_size * hd + col;
     const int64_t page_stride = static_cast<int64_t>(n_kv_head) * page_size * hd;
     for (int j0 = k_begin + wave * KPP; j0 < k_end; j0 += AD_WAVES * KPP * AD_U) {
-        u32x4 kv[AD_U], vv[AD_U];
+        typename Raw8<T>::type kv[AD_U], vv[AD_U];
         bool valid[AD_U];
 #pragma unroll
         for (int u = 0; u < AD_U; ++u) {
@@ -103,8 +123,8 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
             const int lp = page_shift >= 0 ? jc >> page_shift : jc / page_size;
             const int off = page_shift >= 0 ? jc & (page_size - 1) : jc % page_size;
             const int64_t at = static_cast<int64_t>(sbt[lp]) * page_stride + head_off + static_cast<int64_t>(off) * hd;
-            kv[u] = *reinterpret_cast<const u32x4*>(kc + at);
-            vv[u] = *reinterpret_cast<const u32x4*>(vc + at);
+            kv[u] = fetch8(kc + at);
+            vv[u] = fetch8(vc + at);
         }
         float s[AD_U];
         float m_new = st.m;
@@ -120,14 +140,14 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
             m_new = fmaxf(m_new, s[u]);
         }
         if (m_new == -INFINITY) continue;  // this lane group had no key in this trip (and none before)
-        const float corr = st.m == -INFINITY ? 0.0f : __expf(st.m - m_new);
+        const float corr = st.m == -INFINITY ? 0.0f : exp_for<T>(st.m - m_new);
         st.l *= corr;
 #pragma unroll
         for (int e = 0; e < 8; ++e) st.acc[e] *= corr;
 #pragma unroll
         for (int u = 0; u < AD_U; ++u) {
             if (!valid[u]) continue;
-            const float p = __expf(s[u] - m_new);
+            const float p = exp_for<T>(s[u] - m_new);
             st.l += p;
             float vf[8];
             unpack8(vv[u], vf);
@@ -143,7 +163,7 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
         float ao[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) ao[e] = __shfl_xor(st.acc[e], off, 64);
-        merge_partial(st, mo, lo, ao);
+        merge_partial<T>(st, mo, lo, ao);
     }
     if (kg == 0) {
         lds[wave][c][0] = st.m;
@@ -154,12 +174,12 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
     __syncthreads();
     if (wave == 0 && kg == 0 && active) {
 #pragma unroll
-        for (int w = 1; w < AD_WAVES; ++w) merge_partial(st, lds[w][c][0], lds[w][c][1], &lds[w][c][2]);
+        for (int w = 1; w < AD_WAVES; ++w) merge_partial<T>(st, lds[w][c][0], lds[w][c][1], &lds[w][c][2]);
         if (n_splits == 1) {
-            bf16_t* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
+            T* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
             const float inv = 1.0f / st.l;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = float_to_bf16(st.acc[e] * inv);
+            for (int e = 0; e < 8; ++e) o[e] = from_float<T>(st.acc[e] * inv);
         } else {
             // partials [token slot][head][split][hd + 4]: values, then maximum and sum (and two
             // unused, which keep every split's values 16-byte aligned)
@@ -175,7 +195,8 @@ attention_decode_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16
 }
 
 // Splits of a (token, head) merged in split order.
-__global__ void attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
+template <typename T>
+__global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
                                        const float* __restrict__ partials, int n_head, int hd, int n_splits) {
     const int slot = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
     if (e >= hd) return;
@@ -187,63 +208,39 @@ __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_str
     for (int z = 0; z < n_splits; ++z) {
         const float m = p[z * (hd + 4) + hd];
         if (m == -INFINITY) continue;
-        const float w = __expf(m - M);
+        const float w = exp_for<T>(m - M);
         sum += w * p[z * (hd + 4) + hd + 1];
         o += w * p[z * (hd + 4) + e];
     }
-    out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = float_to_bf16(o / sum);
+    out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = from_float<T>(o / sum);
 }
 
-}  // namespace liyab
-
-using namespace liyab;
-
-// Tokens tok_list[0..n) (or 0..n-1 when tok_list is null), each on its own. `partials` must hold
-// n * n_head * n_splits * (hd + 4) floats when n_splits > 1. With `leave_splits` (n_splits > 1)
-// the splits are not merged and `out` is not written: partials[token slot][head][split] holds
-// hd weighted values, then the split's maximum and sum (an empty split: -inf and 0), for a
-// reader that merges them as it loads them (the output projection cut over its inner dimension).
-extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
-                                      const void* vc, const int* block_tables, int max_blocks, const int* tok_list,
-                                      const int* tok_seq, const int* tok_pos, int n, float scale, int window,
-                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
-                                      int rows_are_requests, float* partials, int leave_splits, hipStream_t stream) {
-    LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
-    LIYAB_REQUIRE(!leave_splits || n_splits > 1, "attention_decode: splits are left only when there are several");
-    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
-    LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
-    LIYAB_REQUIRE(hd >= 8 && hd <= 256 && hd % 8 == 0, "attention_decode: head size %d is not a multiple of 8 in 8..256", hd);
-    LIYAB_REQUIRE(q_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(q) & 15) == 0 && (reinterpret_cast<uintptr_t>(kc) & 15) == 0 &&
-                      (reinterpret_cast<uintptr_t>(vc) & 15) == 0,
-                  "attention_decode: queries and caches must be 16-byte aligned with a query stride that is a multiple of 8");
-    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
-                  "attention_decode: row strides are shorter than heads x head size");
-    LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
-    LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
-    LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
-    LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
-    LIYAB_REQUIRE(waves == 4 || waves == 8 || waves == 16, "attention_decode: %d waves per workgroup is not 4, 8 or 16", waves);
-    if (n == 0) return 0;
+template <typename T>
+int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc,
+                            const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq,
+                            const int* tok_pos, int n, float scale, int window, int n_head, int n_kv_head, int hd,
+                            int page_size, int n_splits, int waves, int rows_are_requests, float* partials,
+                            int leave_splits, hipStream_t stream) {
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
         if ((1 << b) == page_size) page_shift = b;
     dim3 grid(n, n_head, n_splits);
-    auto* o = static_cast<bf16_t*>(out);
-    auto* pq = static_cast<const bf16_t*>(q);
-    auto* pk = static_cast<const bf16_t*>(kc);
-    auto* pv = static_cast<const bf16_t*>(vc);
+    auto* o = static_cast<T*>(out);
+    auto* pq = static_cast<const T*>(q);
+    auto* pk = static_cast<const T*>(kc);
+    auto* pv = static_cast<const T*>(vc);
 #define LIYAB_GO(L)                                                                                                  \
     do {                                                                                                             \
         if (waves == 4)                                                                                              \
-            attention_decode_kernel<L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
                                                                     window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
         else if (waves == 8)                                                                                         \
-            attention_decode_kernel<L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
                                                                     window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
         else                                                                                                         \
-            attention_decode_kernel<L, 16, 8><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
                                                                       window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
     } while (0)
@@ -256,21 +253,67 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
 #undef LIYAB_GO
     if (int rc = check_launch("attention_decode")) return rc;
     if (n_splits > 1 && !leave_splits) {
-        attention_merge_kernel<<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits);
+        attention_merge_kernel<T><<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits);
         return check_launch("attention_merge");
     }
     return 0;
 }
+}  // namespace liyab
+
+using namespace liyab;
+
+// Tokens tok_list[0..n) (or 0..n-1 when tok_list is null), each on its own. `partials` must hold
+// n * n_head * n_splits * (hd + 4) floats when n_splits > 1. With `leave_splits` (n_splits > 1)
+// the splits are not merged and `out` is not written: partials[token slot][head][split] holds
+// hd weighted values, then the split's maximum and sum (an empty split: -inf and 0), for a
+// reader that merges them as it loads them (the output projection cut over its inner dimension).
+// dtype: the element type of out, q and the caches (bfloat16 or 32-bit floats).
+extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                      const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
+                                      const int* tok_seq, const int* tok_pos, int n, float scale, int window,
+                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
+                                      int rows_are_requests, float* partials, int leave_splits, hipStream_t stream) {
+    LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
+    LIYAB_REQUIRE(dtype == kBF16 || dtype == kF32, "attention_decode: unknown dtype %d", dtype);
+    LIYAB_REQUIRE(!leave_splits || n_splits > 1, "attention_decode: splits are left only when there are several");
+    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_decode: bad sizes");
+    LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_decode: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
+    LIYAB_REQUIRE(hd >= 8 && hd <= 256 && hd % 8 == 0, "attention_decode: head size %d is not a multiple of 8 in 8..256", hd);
+    const int per16 = dtype == kBF16 ? 8 : 4;  // elements in 16 bytes
+    LIYAB_REQUIRE(q_stride % per16 == 0 && (reinterpret_cast<uintptr_t>(q) & 15) == 0 && (reinterpret_cast<uintptr_t>(kc) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(vc) & 15) == 0,
+                  "attention_decode: queries and caches must be 16-byte aligned with a query stride that is a multiple of 16 bytes");
+    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd && q_stride >= static_cast<int64_t>(n_head) * hd,
+                  "attention_decode: row strides are shorter than heads x head size");
+    LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
+    LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
+    LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
+    LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
+    LIYAB_REQUIRE(waves == 4 || waves == 8 || waves == 16, "attention_decode: %d waves per workgroup is not 4, 8 or 16", waves);
+    if (n == 0) return 0;
+    if (dtype == kF32)
+        return launch_attention_decode<float>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
+                                              tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, waves,
+                                              rows_are_requests, partials, leave_splits, stream);
+    return launch_attention_decode<bf16_t>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
+                                           tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, waves,
+                                           rows_are_requests, partials, leave_splits, stream);
+}
 
 // out[m, h * hd + e] = the splits of (m, h) merged in split order: for splits that
 // liyab_attention_decode left unmerged and no reader takes as they are.
-extern "C" int liyab_attention_merge(void* out, int64_t out_stride, const float* partials, int n, int n_head, int hd,
-                                     int n_splits, hipStream_t stream) {
+extern "C" int liyab_attention_merge(void* out, int out_dtype, int64_t out_stride, const float* partials, int n, int n_head,
+                                     int hd, int n_splits, hipStream_t stream) {
     LIYAB_REQUIRE(out && partials, "attention_merge: null pointer");
     LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_head <= 65535 && hd > 0 && hd <= 1024 && n_splits >= 1, "attention_merge: bad sizes");
     LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd, "attention_merge: the row stride is shorter than heads x head size");
+    LIYAB_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "attention_merge: unknown dtype %d", out_dtype);
     if (n == 0) return 0;
-    attention_merge_kernel<<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, nullptr, partials,
-                                                                                 n_head, hd, n_splits);
+    const dim3 grid(n, n_head);
+    const int threads = ((hd + 63) / 64) * 64;
+    if (out_dtype == kF32)
+        attention_merge_kernel<float><<<grid, threads, 0, stream>>>(static_cast<float*>(out), out_stride, nullptr, partials, n_head, hd, n_splits);
+    else
+        attention_merge_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, nullptr, partials, n_head, hd, n_splits);
     return check_launch("attention_merge");
 }

@@ -725,7 +725,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
                      rows_are_requests: bool = False, leave_splits: bool = False) -> None:
-    """Each token on its own over its request's bfloat16 cache, its keys cut into `n_splits`.
+    """Each token on its own over its request's cache (bfloat16, or float32 throughout), its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
     request t (every request brings one token), which saves the kernel a lookup. With
     `leave_splits` (several splits) `out` is not written: `partials`, viewed as [tokens, heads,
@@ -739,8 +739,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
     n = rows if n_tokens is None else n_tokens
     if q.shape[0] != rows or q.shape[1] < n_head * hd or out.shape[1] != n_head * hd:
         raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {n_head} heads of {hd}")
-    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16):
-        raise KernelError("attention_decode: q, out and the caches must be bfloat16")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype) or q.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("attention_decode: q, out and the caches must all be bfloat16 or all float32")
     _dev(block_tables, "block_tables")
     if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
         raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
@@ -757,22 +757,22 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
         if partials is None or partials.dtype != torch.float32 or partials.numel() < need or not partials.is_contiguous():
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
-              block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
+              dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
               n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, 1 if rows_are_requests else 0,
               _ptr(partials), 1 if leave_splits else 0, _stream())
 
 
 def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
-    """out [tokens, heads * head size] bfloat16 = the splits that `attention_decode(...,
+    """out [tokens, heads * head size] (bfloat16 or float32) = the splits that `attention_decode(...,
     leave_splits=True)` left in partials [tokens, heads, splits, head size + 4], merged in split order."""
     _dev(partials, "partials")
     os_ = _rows(out, "out")
     if partials.dtype != torch.float32 or partials.dim() != 4 or not partials.is_contiguous():
         raise KernelError("attention_merge: partials must be contiguous float32 [tokens, heads, splits, head size + 4]")
     n, H, S, hd4 = partials.shape
-    if out.dtype != torch.bfloat16 or tuple(out.shape) != (n, H * (hd4 - 4)):
-        raise KernelError(f"attention_merge: out must be bfloat16 [{n}, {H * (hd4 - 4)}]")
-    _lib.call("liyab_attention_merge", out.data_ptr(), os_, partials.data_ptr(), n, H, hd4 - 4, S, _stream())
+    if out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (n, H * (hd4 - 4)):
+        raise KernelError(f"attention_merge: out must be bfloat16 or float32 [{n}, {H * (hd4 - 4)}]")
+    _lib.call("liyab_attention_merge", out.data_ptr(), dtype_code(out.dtype), os_, partials.data_ptr(), n, H, hd4 - 4, S, _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -876,6 +876,13 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
                          rows_are_requests=tok_list is None and host.max_q_len == 1)
 
+    if (plan is not None and q.dtype == torch.float32 and hd % 8 == 0 and q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0
+            and block_tables.shape[1] <= 2048):
+        # the 32-bit path: every token on its own, one split on four waves, as in the invariant mode below:
+        # the order of a token's sums follows from its position alone, so its bits do not depend on the batch
+        attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
+                         window=window, n_splits=1, waves=4, rows_are_requests=host.max_q_len == 1)
+        return None
     if fast and _invariant and block_tables.shape[1] <= 2048:
         # every token on its own, its keys in one split on four waves: which lane adds which key
         # follows from the token's position alone

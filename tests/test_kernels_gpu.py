@@ -190,8 +190,14 @@ def gemm_reference(a, w, bias, epilogue, residual=None):
 GEMM_SHAPES = [(1, 64, 64), (7, 200, 96), (33, 777, 144), (130, 50, 320), (64, 1000, 96), (257, 130, 72)]
 
 
+# beside those: each width of the row-wise kernel (4, 8 and 16 features a workgroup), chunks of K
+# with a tail, more chunks than waves, a K that is no multiple of 4 (the one-thread-an-element form)
+F32_SHAPES = GEMM_SHAPES + [(16, 1500, 100), (9, 2600, 260), (5, 3000, 72), (12, 40, 6), (40, 2561, 132), (3, 1024, 1028),
+                            (16, 33, 3076), (20, 70, 50)]
+
+
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
-@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("M,N,K", F32_SHAPES)
 def test_gemm_float32(ops, M, N, K, epilogue):
     a, w, bias = rnd(M, K), rnd(N, K, seed=1, scale=0.2), rnd(N, seed=2)
     if epilogue == "residual":
@@ -203,13 +209,16 @@ def test_gemm_float32(ops, M, N, K, epilogue):
         out = torch.empty(M, N, device=DEV)
         ops.gemm(a, w, bias, out=out, epilogue=ops.ACTIVATION_EPILOGUE[epilogue])
         close(out, gemm_reference(a, w, bias, epilogue), 2e-6, f"gemm f32 {epilogue}")
-    # a row's result does not depend on the rows around it
+    # a row's result does not depend on the rows around it, nor on which kernel their number chooses
     if M > 1:
         one = torch.empty(1, N, device=DEV)
         ops.gemm(a[M // 2:M // 2 + 1], w, bias, out=one)
         full = torch.empty(M, N, device=DEV)
         ops.gemm(a, w, bias, out=full)
         assert torch.equal(one[0], full[M // 2])
+        many = torch.empty(40 + M, N, device=DEV)  # among 40 rows more: the tiled kernel
+        ops.gemm(torch.cat([rnd(40, K, seed=9), a]), w, bias, out=many)
+        assert torch.equal(many[40:], full)
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
@@ -422,14 +431,15 @@ def test_attention_generic(ops, case_id, dtype, window):
 
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("splits,waves", [(1, 4), (1, 16), (2, 4), (5, 16), (32, 4), (1, 8), (3, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
-def test_attention_decode(ops, case_id, splits, waves, window):
+def test_attention_decode(ops, case_id, dtype, splits, waves, window):
     ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
-    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, torch.bfloat16, seed=case_id)
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, dtype, seed=case_id)
     scale = 0.7 / math.sqrt(hd)
     out = run_attention(ops, case, H, hd, scale, window, "decode", splits, waves=waves)
     assert torch.isfinite(out.float()).all()
-    close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, f"decode splits={splits}")
+    close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3 if dtype == torch.bfloat16 else 2e-6, f"decode splits={splits}")
     # a subset of the rows through tok_list: the others stay untouched
     if case["n"] > 2:
         rows = list(range(case["n"]))[::2]
