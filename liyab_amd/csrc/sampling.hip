@@ -25,8 +25,10 @@ namespace liyab {
 constexpr int S_THREADS = 1024;
 constexpr int S_WAVES = S_THREADS / kWave;
 
+// Unsigned keys in the order of the floats. -0 becomes +0 first (x + 0 does that and nothing
+// else), so that the two zeros are one value with one key, ties like any others.
 __device__ __forceinline__ uint32_t ordered_key(float f) {
-    const uint32_t u = __float_as_uint(f);
+    const uint32_t u = __float_as_uint(f + 0.0f);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 __device__ __forceinline__ float key_value(uint32_t k) {

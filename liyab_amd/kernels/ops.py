@@ -715,7 +715,6 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
         return
     if epilogue == EPI_QKV_PAGED:
         # the plain kernel writes the whole projection; a second kernel moves keys and values
-        k_cache, v_cache, slots, q_dim = kv
         raise KernelError("gemm: the paged QKV epilogue is for the matrix-core kernels; use gemm + kv_write")
     gemm_simple(a, w, bias, out=out, residual=residual, epilogue=epilogue)
 

@@ -642,6 +642,10 @@ def test_top_p_over_many_candidates_keeps_exactly_the_nucleus(ops, V):
     for k, p in ((100, 0.5), (100, 0.9), (100, 0.999), (400, 0.3), (V - 1, 0.6)):
         cases.append((wide, 1.0, k, p))
     cases.append((torch.full((V,), 0.25), 1.0, 0, 0.5))  # every key in one bin: more than the pool holds
+    zeros = (torch.randn(V, generator=g) * 1.5).round()  # thousands of ties a value, and both zeros, which are one value
+    assert (zeros == 0).sum() > 100 and torch.signbit(zeros[zeros == 0]).any() and not torch.signbit(zeros[zeros == 0]).all()
+    for T, k, p in ((1.0, 0, 0.6), (1.7, 0, 0.95), (1.0, 200, 0.9), (0.0, 0, 1.0), (1.0, 30, 1.0)):
+        cases.append((zeros.clamp(max=0.0) if T == 0.0 else zeros, T, k, p))
     cases.append((torch.randn(V, generator=g) * 0.01, 1.0, 0, 0.9))  # nearly flat: a few bins hold the row
     peaked = torch.linspace(0.0, -40.0, V)[torch.randperm(V, generator=g)]
     for T, p in ((1.0, 0.9), (0.3, 0.5), (3.0, 0.95)):
