@@ -21,6 +21,8 @@
 #include "common.h"
 #include "epilogue.h"
 
+#include <type_traits>
+
 namespace liyab {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -60,7 +62,7 @@ struct PartsParams {
 // 8 different pieces: the piece index is XORed with (row / 2) % 8.
 __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1>
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1, int SETS = 1>
 __global__ void __launch_bounds__(64 * WM * WN * WK)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
                     EpiParams epi, int vec_ok, int page_shift, PartsParams parts) {
@@ -68,7 +70,10 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     // A stage holds WK consecutive units of 64 k, one a group: the groups walk K side by side (a
     // tile of few rows has few products a unit, and its walk is a chain of waits: load, barrier,
     // fragments, products; WK of them run at once), and their sums are added at the end in the
-    // groups' order.
+    // groups' order. SETS (with WK = 1): the one group keeps SETS sums, unit u of 64 k going to sum
+    // u % SETS, added at the end in the sums' order: what WK = SETS groups would have left, bit
+    // for bit, so that a row has one result in tiles of every shape (the batch-invariant mode).
+    static_assert(SETS == 1 || (WK == 1 && SETS == 4), "sums by unit are for one group of waves, four of them");
     constexpr int GROUP = WM * WN, WAVES = GROUP * WK, TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int UNIT = (BM + BN) * DBK;       // elements of one unit of 64 k: the tile of a, then the tile of w
     constexpr int STAGE = WK * UNIT;            // elements per stage
@@ -115,13 +120,15 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         }
     };
 
-    floatx16 acc[TM][TN];
+    floatx16 sums[SETS][TM][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int s = 0; s < SETS; ++s)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sums[s][i][j][r] = 0.0f;
 
     if constexpr (EPI == kEpiParts) {
         // this workgroup's part of K: units [kt0, kt0 + units)
@@ -136,7 +143,8 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 #pragma unroll
     for (int p = 0; p < AHEAD; ++p)
         if (p < nk) issue(p, p);
-    for (int kt = 0; kt < nk; ++kt) {
+    auto step = [&](int kt, auto set) {
+        floatx16 (&acc)[TM][TN] = sums[decltype(set)::value];
         // tile kt must have landed: the loads of the tiles after it may still be in flight (a
         // wave's loads complete in order, A_LOADS + W_LOADS a tile)
         const int later = min(nk - 1 - kt, AHEAD - 1);
@@ -156,7 +164,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         if (kt + AHEAD < nk) issue(kt + AHEAD, (kt + AHEAD) % DSTAGES);  // into the stage tile kt - 1 used
         const bf16_t* sa = lds + (kt % DSTAGES) * STAGE + wk * UNIT;
         const bf16_t* sw = sa + BM * DBK;
-        if (WK > 1 && kt * WK + wk >= units) continue;  // this group's unit is past the end of K (the last stage only)
+        if (WK > 1 && kt * WK + wk >= units) return;  // this group's unit is past the end of K (the last stage only)
         // fragments of slab ks + 1 are read from LDS while slab ks multiplies
         bf16x8 fa[2][TM], fw[2][TN];
         auto read_frags = [&](int ks, int buf) {
@@ -182,7 +190,26 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0);
         }
+    };
+    if constexpr (SETS == 1) {
+        for (int kt = 0; kt < nk; ++kt) step(kt, std::integral_constant<int, 0>{});
+    } else {
+        for (int kt = 0; kt < nk; kt += 4) {
+            step(kt, std::integral_constant<int, 0>{});
+            if (kt + 1 < nk) step(kt + 1, std::integral_constant<int, 1>{});
+            if (kt + 2 < nk) step(kt + 2, std::integral_constant<int, 2>{});
+            if (kt + 3 < nk) step(kt + 3, std::integral_constant<int, 3>{});
+        }
+#pragma unroll
+        for (int q = 1; q < SETS; ++q)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sums[0][i][j][r] += sums[q][i][j][r];
     }
+    floatx16 (&acc)[TM][TN] = sums[0];
     if constexpr (WK > 1) {
         // the groups' sums, added in the groups' order by the first group, which alone stores:
         // the others go through the epilogue as a tile below the last row
@@ -385,11 +412,11 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     }
 }
 
-template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1>
+template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1, int SETS = 1>
 int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     const int grid = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
     const size_t smem = static_cast<size_t>(DSTAGES) * WK * (BM + BN) * DBK * sizeof(bf16_t);
-    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN, WK>;
+    auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN, WK, SETS>;
     static bool ready = false;  // once per instantiation, outside any stream capture's first use
     if (!ready) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
@@ -436,21 +463,21 @@ int launch_dl_parts(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N,
     return check_launch("gemm_mfma_dl_parts");
 }
 
-template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2, int WK = 1>
+template <int BM, int BN, int DSTAGES, int WM = 2, int WN = 2, int WK = 1, int SETS = 1>
 int launch_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     auto* pa = static_cast<const bf16_t*>(a);
     auto* pw = static_cast<const bf16_t*>(w);
-    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.mode == kEpiResidual) return launch_dl_as<BM, BN, DSTAGES, float, kEpiResidual, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
     if (epi.out_dtype == kF32) {
-        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
-        return launch_dl_as<BM, BN, DSTAGES, float, -1, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        if (epi.mode == kEpiNone) return launch_dl_as<BM, BN, DSTAGES, float, kEpiNone, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
+        return launch_dl_as<BM, BN, DSTAGES, float, -1, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
     }
     switch (epi.mode) {
-        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
-        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
-        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1, WM, WN, WK>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiNone: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiNone, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluTanh: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluTanh, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiGeluErf: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiGeluErf, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
+        case kEpiQkvPaged: return launch_dl_as<BM, BN, DSTAGES, bf16_t, kEpiQkvPaged, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
+        default: return launch_dl_as<BM, BN, DSTAGES, bf16_t, -1, WM, WN, WK, SETS>(pa, lda, pw, M, N, K, epi, stream);
     }
 }
 
@@ -489,6 +516,10 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 16: return launch_dl<64, 32, 3, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
         case 17: return launch_dl<32, 32, 3, 1, 1, 4>(a, lda, w, M, N, K, epi, stream);
+        // 102, 106, 108: the tiles of 2, 6 and 8 with four sums by unit of K, whose results are those of 16 and 17 bit for bit
+        case 102: return launch_dl<64, 64, 3, 2, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
+        case 106: return launch_dl<64, 64, 4, 2, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
+        case 108: return launch_dl<128, 128, 2, 4, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
         default: return fail(1, "gemm_mfma_dl: unknown tile %d", tile);
     }
 }

@@ -674,11 +674,17 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
     q_dim) with the paged QKV epilogue."""
     if _invariant and mfma_takes(a, w):
         # one family of kernels whatever the number of rows: their sum over k has one order for
-        # every tile shape (units of 64 k in turn, 16 k an instruction), so a row's bits do not
-        # depend on the rows beside it
-        if a.shape[1] % 64 == 0:
-            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv,
-                         tile=8 if a.shape[0] * w.shape[0] >= 2048 * 2048 else (6 if a.shape[1] >= 2048 else 2))
+        # every tile shape, so a row's bits do not depend on the rows beside it. K a multiple of 64:
+        # four sums, unit u of 64 k going to sum u % 4 (16 k an instruction), added in their order;
+        # up to 64 rows four groups of waves walk K side by side, a sum each, in small tiles that
+        # cover the chip; more rows take the large tiles, whose one group keeps the four sums.
+        M, N, K = a.shape[0], w.shape[0], a.shape[1]
+        if K % 64 == 0:
+            if M <= 64:
+                tile = 17 if (M + 31) // 32 * ((N + 31) // 32) <= compute_units() else 16
+            else:
+                tile = 108 if M * N >= 2048 * 2048 else (106 if K >= 2048 else 102)
+            gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=tile)
         else:
             gemm_mfma(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=2)
         return

@@ -697,6 +697,30 @@ def test_sampler_without_cuts(ops, V):
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, T, got[r], want)
 
 
+@pytest.mark.parametrize("K", [64, 768, 832, 3072])
+def test_tiles_of_every_shape_give_a_row_the_same_bits(ops, K):
+    """The tiled products of the batch-invariant mode: the small tiles whose four groups of waves
+    walk K side by side (16, 17) and the large ones whose one group keeps four sums by unit of K
+    (102, 106, 108) leave the same bits in a row, whatever rows are beside it; K of one unit, of
+    whole rounds of four units and of 13 units."""
+    M, N = 200, 320
+    a, w, bias = rnd(M, K, dtype=torch.bfloat16, seed=K), rnd(N, K, dtype=torch.bfloat16, seed=K + 1, scale=0.2), rnd(N, seed=2)
+    want = gemm_reference(a.float(), w.float(), bias, "none")
+    full = {}
+    for tile in (102, 106, 108, 16, 17):
+        out = torch.empty(M, N, device=DEV)
+        ops.gemm_mfma_dl(a, w, bias, out=out, tile=tile)
+        close(out, want, 2e-5, f"tile {tile}")
+        full[tile] = out
+    for tile in (106, 108, 16, 17):
+        assert torch.equal(full[tile], full[102]), f"tile {tile} against 102"
+    for rows in (slice(0, 8), slice(37, 38), slice(100, 164)):
+        for tile in (16, 17):
+            out = torch.empty(rows.stop - rows.start, N, device=DEV)
+            ops.gemm_mfma_dl(a[rows], w, bias, out=out, tile=tile)
+            assert torch.equal(out, full[108][rows]), f"rows {rows} in tiles {tile}"
+
+
 @pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "dl16", "auto"])
 @pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
