@@ -89,26 +89,26 @@ gemm_simple_kernel(OutT* __restrict__ out, int64_t ldo, const T* __restrict__ a,
 }
 
 // The same product for steps of few rows (decoding), in the same order of sums, so a row's
-// result has the same bits whichever of the two kernels computed it. A workgroup of four
-// waves takes NB output features and 16 rows (blockIdx.y: which 16); the chunks of K go round the waves. A wave
+// result has the same bits whichever of the two kernels computed it. A workgroup of four or
+// eight waves takes NB output features and 16 rows (blockIdx.y: which 16); the chunks of K go round the waves. A wave
 // brings its chunk of the NB rows of `w` and of the rows of `a` through registers into LDS of
 // its own (256 bytes a row and load, the next chunk in flight meanwhile); lane (feature, row
-// group) then runs the chunk's chain for its rows; after each round of four chunks one thread
-// an output element adds the four sums in chunk order. Few features a workgroup where N is
+// group) then runs the chunk's chain for its rows; after each round of chunks one thread
+// an output element adds the round's sums in chunk order. Few features a workgroup where N is
 // small: the weights then stream through enough compute units.
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 constexpr int kRowwiseRows = 16;     // rows a workgroup
 constexpr int kRowwiseMaxRows = 64;  // steps of at most this many rows take the row-wise kernel
 
-template <int NB, int EPI, bool EXACT>
-__global__ void __launch_bounds__(256)
+template <int NB, int WAVES, int EPI, bool EXACT>
+__global__ void __launch_bounds__(64 * WAVES)
 gemm_rowwise_f32_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ a, int64_t lda,
                         const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ residual,
                         int64_t ldr, int M_all, int N, int K) {
     const int row0 = blockIdx.y * kRowwiseRows, M = min(kRowwiseRows, M_all - row0);
     a += static_cast<int64_t>(row0) * lda;
-    constexpr int WAVES = 4, LD = kChunk + 4;  // (rows 16 bytes apart in the banks: a lane's 16-byte reads do not collide)
+    constexpr int LD = kChunk + 4;  // (rows 16 bytes apart in the banks: a lane's 16-byte reads do not collide)
     constexpr int MG = 64 / NB;                // row groups of lanes
     constexpr int RPL = kRowwiseRows / MG;     // rows a lane
     constexpr int W_LOADS = NB / 4, A_LOADS = kRowwiseRows / 4;  // a load covers 4 rows: 16 lanes a row, 16 bytes a lane
@@ -230,9 +230,11 @@ int launch_rowwise_f32_epi(float* out, int64_t ldo, const float* a, int64_t lda,
     }
     // about two hundred workgroups or more: 4 features each up to 1,024 of them, 8 up to 2,560, 16 beyond
     const int row_blocks = (M + kRowwiseRows - 1) / kRowwiseRows;
-    if (N <= 1024) gemm_rowwise_f32_kernel<4, EPI, true><<<dim3((N + 3) / 4, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
-    else if (N <= 2560) gemm_rowwise_f32_kernel<8, EPI, true><<<dim3((N + 7) / 8, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
-    else gemm_rowwise_f32_kernel<16, EPI, true><<<dim3((N + 15) / 16, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
+    // (few features and a long K: eight waves share the chunks, twice as many loads in flight)
+    if (N <= 1024 && K >= 2048) gemm_rowwise_f32_kernel<4, 8, EPI, true><<<dim3((N + 3) / 4, row_blocks), 512, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
+    else if (N <= 1024) gemm_rowwise_f32_kernel<4, 4, EPI, true><<<dim3((N + 3) / 4, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
+    else if (N <= 2560) gemm_rowwise_f32_kernel<8, 4, EPI, true><<<dim3((N + 7) / 8, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
+    else gemm_rowwise_f32_kernel<16, 4, EPI, true><<<dim3((N + 15) / 16, row_blocks), 256, 0, stream>>>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K);
     return check_launch("gemm_rowwise");
 }
 

@@ -681,7 +681,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
         M, N, K = a.shape[0], w.shape[0], a.shape[1]
         if K % 64 == 0:
             if M <= 64:
-                tile = 17 if (M + 31) // 32 * ((N + 31) // 32) <= compute_units() else 16
+                tile = 17 if M <= 32 or 2 * ((N + 31) // 32) <= compute_units() else 16
             else:
                 tile = 108 if M * N >= 2048 * 2048 else (106 if K >= 2048 else 102)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=tile)
