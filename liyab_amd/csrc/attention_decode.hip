@@ -9,8 +9,10 @@
 // weighted values (the reference's per-span partial softmax,
 // src/core/transformer.cpp:2327-2358); groups, then waves, then splits are
 // merged in a fixed order by rescaling to the common maximum (:2367-2385).
-// With one split on four waves which lane adds which key follows from the
-// token's position alone: the form the 32-bit path always takes.
+// With `chunk` keys a split (instead of the token's keys divided by the number of
+// splits) and four waves, which lane adds which key and which sums are merged
+// follow from the token's position alone, as the reference cuts (:2136-2139):
+// the form of the 32-bit path and of the batch-invariant mode.
 // The reference cuts a token's keys by its position only (:2136-2139,
 // 2225-2227) to keep bits equal; here the number of splits follows the batch
 // (more splits when few tokens are in flight), which moves results by
@@ -22,6 +24,7 @@ namespace liyab {
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int AD_MAX_BLOCKS = 2048;  // page ids of a request kept in LDS
+constexpr int AD_LOOP_CHUNKS = 16;   // splits by position that one workgroup walks in turn, at most
 
 
 __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
@@ -73,9 +76,9 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
                         int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
-                        int n_splits, float* __restrict__ partials) {
+                        int n_splits, int chunk, float* __restrict__ partials) {
     constexpr int KPP = 64 / LPK;  // keys per wave and pass
-    __shared__ float lds[AD_WAVES][LPK][10];
+    __shared__ float lds2[2][AD_WAVES][LPK][10];  // the waves' sums, for the first wave to merge; two of them in turn, so that one barrier a split is enough
     const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
     const int h = blockIdx.y, z = blockIdx.z;
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -101,8 +104,19 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
     __syncthreads();
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
     const int n_keys = pos - first + 1;
-    const int k_begin = first + static_cast<int>(static_cast<int64_t>(n_keys) * z / n_splits);
-    const int k_end = first + static_cast<int>(static_cast<int64_t>(n_keys) * (z + 1) / n_splits);
+    // Splits by position launched as one (chunk > 0, n_splits == 1): the workgroup walks the token's
+    // splits one after the other, keeps each one's sums apart and merges them at the end as the merge
+    // kernel would, operation for operation: the bits of the split launch without its traffic, for
+    // steps of many tokens.
+    const bool walks_all = chunk > 0 && n_splits == 1;
+    const int z_count = walks_all ? min(AD_LOOP_CHUNKS, max(1, (n_keys + chunk - 1) / chunk)) : 1;  // (the launcher has checked that they fit)
+    __shared__ float stash[AD_LOOP_CHUNKS][LPK][10];
+    for (int zi = 0; zi < z_count; ++zi) {
+    float (&lds)[AD_WAVES][LPK][10] = lds2[zi & 1];
+    const int zz = walks_all ? zi : z;
+    // split zz: its share of the keys, or keys [zz * chunk, (zz + 1) * chunk) of them (none, for a short context)
+    const int k_begin = first + (chunk > 0 ? zz * chunk : static_cast<int>(static_cast<int64_t>(n_keys) * zz / n_splits));
+    const int k_end = chunk > 0 ? min(pos + 1, k_begin + chunk) : first + static_cast<int>(static_cast<int64_t>(n_keys) * (zz + 1) / n_splits);
     Partial st;
     st.m = -INFINITY;
     st.l = 0.0f;
@@ -175,11 +189,23 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
     if (wave == 0 && kg == 0 && active) {
 #pragma unroll
         for (int w = 1; w < AD_WAVES; ++w) merge_partial<T>(st, lds[w][c][0], lds[w][c][1], &lds[w][c][2]);
-        if (n_splits == 1) {
-            T* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
-            const float inv = 1.0f / st.l;
+        if (z_count > 1) {
+            stash[zi][c][0] = st.m;
+            stash[zi][c][1] = st.l;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = from_float<T>(st.acc[e] * inv);
+            for (int e = 0; e < 8; ++e) stash[zi][c][2 + e] = st.acc[e];
+        } else if (n_splits == 1) {
+            T* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
+            if (chunk > 0) {
+                // as the merge of several splits divides: a token has the same bits alone in one split
+                // and beside longer contexts, its later splits empty
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = from_float<T>(st.acc[e] / st.l);
+            } else {
+                const float inv = 1.0f / st.l;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = from_float<T>(st.acc[e] * inv);
+            }
         } else {
             // partials [token slot][head][split][hd + 4]: values, then maximum and sum (and two
             // unused, which keep every split's values 16-byte aligned)
@@ -192,9 +218,29 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
             }
         }
     }
+    }
+    if (z_count > 1 && wave == 0 && kg == 0 && active) {
+        // (each lane reads what it wrote itself)
+        float M = -INFINITY;
+        for (int zi = 0; zi < z_count; ++zi) M = fmaxf(M, stash[zi][c][0]);
+        float sum = 0.0f, o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = 0.0f;
+        for (int zi = 0; zi < z_count; ++zi) {
+            const float m = stash[zi][c][0];
+            if (m == -INFINITY) continue;
+            const float w = exp_for<T>(m - M);
+            sum = fmaf(w, stash[zi][c][1], sum);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = fmaf(w, stash[zi][c][2 + e], o[e]);
+        }
+        T* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[e] = from_float<T>(o[e] / sum);
+    }
 }
 
-// Splits of a (token, head) merged in split order.
+// Splits of a (token, head) merged in split order (the same operations as the end of the kernel above).
 template <typename T>
 __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
                                        const float* __restrict__ partials, int n_head, int hd, int n_splits) {
@@ -209,8 +255,8 @@ __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, 
         const float m = p[z * (hd + 4) + hd];
         if (m == -INFINITY) continue;
         const float w = exp_for<T>(m - M);
-        sum += w * p[z * (hd + 4) + hd + 1];
-        o += w * p[z * (hd + 4) + e];
+        sum = fmaf(w, p[z * (hd + 4) + hd + 1], sum);
+        o = fmaf(w, p[z * (hd + 4) + e], o);
     }
     out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = from_float<T>(o / sum);
 }
@@ -219,7 +265,7 @@ template <typename T>
 int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc,
                             const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq,
                             const int* tok_pos, int n, float scale, int window, int n_head, int n_kv_head, int hd,
-                            int page_size, int n_splits, int waves, int rows_are_requests, float* partials,
+                            int page_size, int n_splits, int chunk, int waves, int rows_are_requests, float* partials,
                             int leave_splits, hipStream_t stream) {
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
@@ -234,15 +280,15 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
         if (waves == 4)                                                                                              \
             attention_decode_kernel<T, L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
         else if (waves == 8)                                                                                         \
             attention_decode_kernel<T, L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
         else                                                                                                         \
             attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
-                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, partials); \
+                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
     } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);
@@ -267,11 +313,13 @@ using namespace liyab;
 // the splits are not merged and `out` is not written: partials[token slot][head][split] holds
 // hd weighted values, then the split's maximum and sum (an empty split: -inf and 0), for a
 // reader that merges them as it loads them (the output projection cut over its inner dimension).
-// dtype: the element type of out, q and the caches (bfloat16 or 32-bit floats).
+// dtype: the element type of out, q and the caches (bfloat16 or 32-bit floats). chunk: 0 = each
+// split an equal share of the token's keys; > 0 = split z takes keys [z * chunk, (z + 1) * chunk)
+// of the token's (n_splits * chunk must cover the longest context: keys beyond are not read).
 extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                       const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
                                       const int* tok_seq, const int* tok_pos, int n, float scale, int window,
-                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int waves,
+                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
                                       int rows_are_requests, float* partials, int leave_splits, hipStream_t stream) {
     LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
     LIYAB_REQUIRE(dtype == kBF16 || dtype == kF32, "attention_decode: unknown dtype %d", dtype);
@@ -287,16 +335,21 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
                   "attention_decode: row strides are shorter than heads x head size");
     LIYAB_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || partials != nullptr), "attention_decode: bad split count %d", n_splits);
     LIYAB_REQUIRE(window >= 0 && n_head <= 65535, "attention_decode: bad window or head count");
+    LIYAB_REQUIRE(chunk >= 0, "attention_decode: a negative number of keys a split");
+    LIYAB_REQUIRE(chunk == 0 || n_splits > 1 || static_cast<int64_t>(chunk) * AD_LOOP_CHUNKS >= static_cast<int64_t>(max_blocks) * page_size ||
+                      (window > 0 && static_cast<int64_t>(chunk) * AD_LOOP_CHUNKS >= window),
+                  "attention_decode: one workgroup walks at most %d splits of %d keys; contexts of %lld need a launch in splits", AD_LOOP_CHUNKS,
+                  chunk, static_cast<long long>(max_blocks) * page_size);
     LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
     LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
     LIYAB_REQUIRE(waves == 4 || waves == 8 || waves == 16, "attention_decode: %d waves per workgroup is not 4, 8 or 16", waves);
     if (n == 0) return 0;
     if (dtype == kF32)
         return launch_attention_decode<float>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
-                                              tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, waves,
+                                              tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
                                               rows_are_requests, partials, leave_splits, stream);
     return launch_attention_decode<bf16_t>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
-                                           tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, waves,
+                                           tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
                                            rows_are_requests, partials, leave_splits, stream);
 }
 

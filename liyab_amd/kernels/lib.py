@@ -53,7 +53,7 @@ _SIGNATURES = {
     "liyab_attention_generic": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, P],
     "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_int, c_int, P, c_int, P],
+                               c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, P],
     "liyab_attention_merge": [P, c_int, c_int64, P, c_int, c_int, c_int, c_int, P],
     "liyab_gemm_att_parts": [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_skinny_ln": [P, c_int, c_int64, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],

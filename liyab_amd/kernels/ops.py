@@ -729,13 +729,15 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
-                     rows_are_requests: bool = False, leave_splits: bool = False) -> None:
+                     rows_are_requests: bool = False, leave_splits: bool = False, chunk: int = 0) -> None:
     """Each token on its own over its request's cache (bfloat16, or float32 throughout), its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
     request t (every request brings one token), which saves the kernel a lookup. With
     `leave_splits` (several splits) `out` is not written: `partials`, viewed as [tokens, heads,
     splits, head size + 4], keeps each split's weighted values, maximum and sum for a reader
-    that merges them (`gemm_att_parts`)."""
+    that merges them (`gemm_att_parts`). `chunk` > 0: split z takes keys [z * chunk, (z + 1) * chunk) of a
+    token's keys instead of an equal share (`n_splits * chunk` must cover the longest context): a token's
+    sums then follow from its position alone."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
     _, hkv, page, hd = k_cache.shape
@@ -763,7 +765,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
-              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, waves, 1 if rows_are_requests else 0,
+              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, int(chunk), waves, 1 if rows_are_requests else 0,
               _ptr(partials), 1 if leave_splits else 0, _stream())
 
 
@@ -851,6 +853,10 @@ SPLIT4_PAIRS, SPLIT2_PAIRS = 192, 192
 ATTENTION_MAX_HEAD_DIM = 256  # what the attention kernels take (attention_generic.hip, attention_decode.hip)
 
 
+INVARIANT_CHUNK = 256  # keys a split where splits go by position alone
+INVARIANT_SPLIT_WORK = 1024  # (token, head, split) workgroups up to which such splits are launched side by side
+
+
 def attention_takes(head_dim: int) -> bool:
     """Whether some attention kernel of the library takes this head size, in either precision."""
     return 0 < head_dim <= ATTENTION_MAX_HEAD_DIM
@@ -881,19 +887,22 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
                          rows_are_requests=tok_list is None and host.max_q_len == 1)
 
-    if (plan is not None and q.dtype == torch.float32 and hd % 8 == 0 and q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0
-            and block_tables.shape[1] <= 2048):
-        # the 32-bit path: every token on its own, one split on four waves, as in the invariant mode below:
-        # the order of a token's sums follows from its position alone, so its bits do not depend on the batch
-        attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
-                         window=window, n_splits=1, waves=4, rows_are_requests=host.max_q_len == 1)
-        return None
-    if fast and _invariant and block_tables.shape[1] <= 2048:
-        # every token on its own, its keys in one split on four waves: which lane adds which key
-        # follows from the token's position alone
+    if (plan is not None and block_tables.shape[1] <= 2048
+            and (fast and _invariant or q.dtype == torch.float32 and hd % 8 == 0 and q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0)):
+        # the 32-bit path and the batch-invariant mode: every token on its own on four waves, its keys
+        # in splits of INVARIANT_CHUNK from its first key on, merged in their order: the order of a
+        # token's sums follows from its position alone, so its bits do not depend on the batch
         n = out.shape[0]
+        splits = max(1, -(-min(plan.context_bucket, window if window > 0 else plan.context_bucket) // INVARIANT_CHUNK))
+        # many tokens: a workgroup walks its token's splits in turn (the same bits: the kernel merges them
+        # as the merge kernel does), which saves the splits' traffic and leaves the chip as full
+        reach = block_tables.shape[1] * k_cache.shape[2] if window <= 0 else min(window, block_tables.shape[1] * k_cache.shape[2])
+        if n * n_head * splits > INVARIANT_SPLIT_WORK and reach <= INVARIANT_CHUNK * 16:
+            splits = 1
+        partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32) if splits > 1 else None
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
-                         window=window, n_splits=1, waves=4, rows_are_requests=host.max_q_len == 1)
+                         window=window, n_splits=splits, partials=partials, waves=4, chunk=INVARIANT_CHUNK,
+                         rows_are_requests=host.max_q_len == 1)
         return None
     if fast and plan.mode == "decode" and block_tables.shape[1] <= 2048:
         n = out.shape[0]

@@ -447,6 +447,52 @@ def test_attention_decode(ops, case_id, dtype, splits, waves, window):
         assert torch.equal(part[rows], out[rows]) and (part[1::2] == 0).all()
 
 
+@pytest.mark.parametrize("window", [0, 37, 300])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("case_id", range(len(ATT_CASES)))
+def test_attention_splits_by_position(ops, case_id, dtype, window):
+    """Splits of a fixed number of keys from a token's first key on: right against the plain
+    formula, and the same bits whether the step has just the splits the longest context needs or
+    more (a longer context beside it), the later ones empty; a context within one split has the
+    bits of the unsplit call."""
+    ctx_lens, q_lens, H, Hkv, hd, page = ATT_CASES[case_id]
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, dtype, seed=case_id)
+    scale = 0.7 / math.sqrt(hd)
+    dev = lambda x: x.to(DEV)  # noqa: E731
+    q, kc, vc, bt = dev(case["q"]), dev(case["kc"]), dev(case["vc"]), dev(case["bt"])
+    tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor(case["tok_pos"], dtype=torch.int32, device=DEV)
+    chunk = 64
+    longest = max(ctx_lens) if window == 0 else min(max(ctx_lens), window)
+    need = -(-longest // chunk)
+    outs = []
+    for splits in (need, need + 1, 2 * need + 3):
+        out = torch.zeros(case["n"], H * hd, dtype=dtype, device=DEV)
+        partials = torch.full((case["n"] * H * splits * (hd + 4),), float("nan"), device=DEV) if splits > 1 else None
+        ops.attention_decode(out, q[:, :H * hd], kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
+                             n_splits=splits, partials=partials, waves=4, chunk=chunk)
+        assert torch.isfinite(out.float()).all()
+        outs.append(out)
+    close(outs[0], attention_reference(case, H, Hkv, hd, scale, window), 8e-3 if dtype == torch.bfloat16 else 2e-6, "splits by position")
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    # launched as one split, a workgroup walking its token's splits in turn: the same bits again
+    if need <= 16:
+        out = torch.zeros(case["n"], H * hd, dtype=dtype, device=DEV)
+        ops.attention_decode(out, q[:, :H * hd], kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
+                             n_splits=1, waves=4, chunk=chunk)
+        assert torch.equal(out, outs[0]), "one workgroup walking the splits"
+    # each request alone, with the splits its own context needs
+    for s_, n_ctx in enumerate(ctx_lens):
+        rows = [t for t, r in enumerate(case["tok_seq"]) if r == s_]
+        own = -(-(n_ctx if window == 0 else min(n_ctx, window)) // chunk)
+        out = torch.zeros(case["n"], H * hd, dtype=dtype, device=DEV)
+        partials = torch.empty(len(rows) * H * own * (hd + 4), device=DEV) if own > 1 else None
+        ops.attention_decode(out, q[:, :H * hd], kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
+                             n_splits=own, partials=partials, waves=4, chunk=chunk,
+                             tok_list=torch.tensor(rows, dtype=torch.int32, device=DEV), n_tokens=len(rows))
+        assert torch.equal(out[rows], outs[0][rows]), f"request {s_} alone"
+
+
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("splits", [2, 4, 7, 8])
 @pytest.mark.parametrize("case_id", [0, 1, 2, 3, 5, 6, 7])
