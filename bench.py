@@ -400,6 +400,19 @@ def main():
                 points[f"decode_b{args.batch}_page16"] = round(t, 1)
                 points[f"decode_b{args.batch}_page16_ms_per_step"] = round(pms_b, 4)
                 del small_pages
+            # the headline batch in the engine's two other modes: replies that do not depend on the batch, and the 32-bit path
+            others = []
+            if not args.batch_invariant and short == "bf16":
+                others.append((f"decode_b{args.batch}_batch_invariant", args.dtype, True))
+            if short == "bf16":
+                others.append((f"decode_b{args.batch}_fp32", "float32", False))
+            del engine
+            for name, dtype, invariant in others:
+                other = make_engine(d, dtype, args.batch, ctx, page_size=args.page_size, batch_invariant=invariant)
+                t, pms_b, _ = decode_run(other, cfg, args.batch, args.prompt, k, w)
+                points[name] = round(t, 1)
+                points[name + "_ms_per_step"] = round(pms_b, 4)
+                del other
             out["points"] = points
     print(json.dumps(out))
     return 0
