@@ -418,3 +418,39 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
             tt.check_against_plain(got, reqs, refs, TOL[dtype], f"{cfg} {label} {dtype}", family="drawn")
             core.manager.check()
             del core
+
+
+def test_random_workloads_through_the_scheduler(tmp_path):
+    """Sixty workloads drawn from a seed, each with its own budgets (positions a page, pages, live
+    requests, tokens a step, tokens a portion, graphs on or off), most of them too tight for the
+    requests at hand, so that prompts are cut, pages run out and requests are preempted and taken up
+    again: in float32 every greedy token is the plain implementation's choice, every request gets
+    its number of tokens, and no page is lost. (The preemptions are counted: the draw must bring some.)"""
+    from liyab_amd import Engine, SamplingParams
+    from liyab_amd.weights import write_random_model
+
+    cfg = dict(drawn_config(2), n_positions=160)
+    write_random_model(str(tmp_path), cfg, 77)
+    config, tensors = plain.read_model(str(tmp_path))
+    preemptions = 0
+    for seed in range(60):
+        rng = np.random.default_rng(5000 + seed)
+        prompts = [tt.random_tokens(seed * 100 + i, int(rng.integers(1, 90)), cfg["vocab_size"]) for i in range(int(rng.integers(1, 9)))]
+        n_new = int(rng.integers(1, 40))
+        page = int(rng.choice([4, 8, 16]))
+        need_one = -(-(max(len(p) for p in prompts) + n_new) // page)
+        kw = dict(page_size=page, num_pages=int(rng.integers(need_one, need_one * 4 + 2)), max_num_seqs=int(rng.integers(1, 7)),
+                  max_batched_tokens=int(rng.integers(8, 200)), prefill_chunk=int(rng.integers(2, 64)), use_graphs=bool(rng.integers(0, 2)))
+        engine = Engine(str(tmp_path), dtype="float32", **kw)
+        engine.stop_at_eos = False
+        results = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new))
+        for i, (prompt, res) in enumerate(zip(prompts, results)):
+            assert len(res.tokens) == n_new, (seed, kw, i)
+            ref = plain.forward(config, tensors, prompt + res.tokens[:-1])
+            for j, t in enumerate(res.tokens):
+                row = ref[len(prompt) - 1 + j]
+                assert row[t] >= row.max() - 1e-5 * np.abs(row).max(), (seed, kw, i, j, t, int(np.argmax(row)))
+        engine.core.manager.check()
+        assert all(engine.core.manager.pages_in_use(g.index) == 0 for g in engine.core.manager.groups)
+        preemptions += engine.scheduler.stats.preemptions
+    assert preemptions > 20
