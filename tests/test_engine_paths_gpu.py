@@ -317,3 +317,34 @@ def test_batch_invariant_replies_are_the_same_alone_and_among_eight(small_widths
         alone = [engine.generate(p, sp) for p in prompts]
         for i, (a, b) in enumerate(zip(together, alone)):
             assert a.tokens == b.tokens, f"prompt {i}: the reply among eight differs from the reply alone"
+
+
+# ---------------------------------------------------------------------------
+# contexts of thousands of positions
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_contexts_of_thousands_of_positions(dtype, tmp_path):
+    """A GPT-2 with 4,100 positions (257 pages of 16 a request): block tables, context buckets,
+    attention's splits and the prefill's walk over keys at four times GPT-2's own context. A
+    request of 4,100 tokens and one of 2,500, most of each in one step and the last 32 one by
+    one, in portions of up to 2,048 tokens, and mixed; every wanted row against the plain
+    implementation. (That a far key is found among thousands, which random weights would
+    average away, is the kernels' own test: test_attention_finds_one_far_key.)"""
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 2, "n_embd": 64, "n_head": 2, "n_inner": 96, "vocab_size": 300,
+           "n_positions": 4100, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    write_random_model(str(tmp_path), cfg, 31)
+    config, tensors = plain.read_model(str(tmp_path))
+    weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+    reqs = {"long": tt.random_tokens(1, 4100, 300), "mid": tt.random_tokens(2, 2500, 300)}
+    refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+    sparse = lambda steps: [dict(s, entries=[(r, t, w if len(t) < 64 else w[-3:]) for r, t, w in s["entries"]]) for s in steps]  # noqa: E731
+    for label, steps in (("bulk+tail", tt.schedule_bulk_tail(reqs)), ("portions", sparse(tt.schedule_portions(reqs, (2048, 7, 1000, 2, 300)))),
+                         ("mixed", sparse(tt.schedule_mixed(reqs, seed=4, decode_tail=6, portions=(700, 9, 1500, 64))))):
+        core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, refs, TOL[dtype], f"4,100 positions {label} {dtype}", family="long context")
+        core.manager.check()
+        del core

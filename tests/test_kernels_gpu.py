@@ -567,11 +567,13 @@ def test_attention_prefill(ops, case_id, window, tile, ksplit):
     close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, "prefill")
 
 
-def test_attention_prefill_finds_one_far_key(ops):
-    """A portion's queries each with one outstanding key, at page and block edges."""
+@pytest.mark.parametrize("T,targets", [(700, [0, 15, 16, 31, 32, 255, 256, 511, 559, 560, 561, 600, 640, 687, 698, 699]),
+                                       (5000, [0, 17, 1023, 1024, 2047, 2048, 3000, 4095, 4096, 4097, 4859, 4860, 4900, 4959, 4998, 4999])])
+def test_attention_prefill_finds_one_far_key(ops, T, targets):
+    """A portion's queries each with one outstanding key, at page and block edges; in a context of
+    700 positions and in one of 5,000 (313 pages)."""
     H = Hkv = 2
-    hd, page, T, nq = 64, 16, 700, 140
-    targets = [0, 15, 16, 31, 32, 255, 256, 511, 559, 560, 561, 600, 640, 687, 698, 699]
+    hd, page, nq = 64, 16, 140
     case = paged_case(1, [T], [nq], H, Hkv, hd, page, torch.bfloat16, seed=3)
     k = case["ks"][0]
     for n, target in enumerate(targets):
@@ -589,20 +591,34 @@ def test_attention_prefill_finds_one_far_key(ops):
     close(out, ref, 8e-3, "prefill far keys")
 
 
-@pytest.mark.parametrize("kernel", ["generic", "decode"])
-def test_attention_finds_one_far_key(ops, kernel):
+@pytest.mark.parametrize("T,targets", [(700, (0, 15, 16, 17, 255, 256, 511, 512, 687, 688, 698, 699)),
+                                       (5000, (0, 255, 256, 2047, 2048, 4095, 4096, 4863, 4864, 4998, 4999))])
+@pytest.mark.parametrize("kernel", ["generic", "decode", "decode by position", "decode walking its splits"])
+def test_attention_finds_one_far_key(ops, kernel, T, targets):
     """Random values average a wrong key away; here one key's score stands out, at a page's
-    first and last slot, in the first page and the last, and the output must be its value row."""
+    first and last slot, in the first page and the last, at the edges of splits, and the output
+    must be its value row; in a context of 700 positions and in one of 5,000."""
     H = Hkv = 2
-    hd, page, T = 64, 16, 700
-    for target in (0, 15, 16, 17, 255, 256, 511, 512, 687, 688, 698, 699):
+    hd, page = 64, 16
+    if kernel == "decode walking its splits" and T > 16 * 256:
+        pytest.skip("one workgroup walks at most 16 splits")
+    for target in targets:
         case = paged_case(1, [T], [1], H, Hkv, hd, page, torch.bfloat16, seed=target)
         qv = case["q"][0, :hd].float()
         k = case["ks"][0]
         k[target, 0] = (qv * 4).to(torch.bfloat16)  # head 0: score ~ 4 |q|^2 ~ 250, all others ~ N(0, 8)
         lp, off = divmod(target, page)
         case["kc"][case["bt"][0, lp], 0, off] = k[target, 0]
-        out = run_attention(ops, case, H, hd, 1.0, 0, kernel, splits=3 if kernel == "decode" else 1)
+        if kernel.startswith("decode "):
+            dev = lambda x: x.to(DEV)  # noqa: E731
+            splits = -(-T // 256) if kernel == "decode by position" else 1
+            out = torch.zeros(1, H * hd, dtype=torch.bfloat16, device=DEV)
+            ops.attention_decode(out, dev(case["q"])[:, :H * hd], dev(case["kc"]), dev(case["vc"]), dev(case["bt"]),
+                                 torch.zeros(1, dtype=torch.int32, device=DEV), torch.tensor([T - 1], dtype=torch.int32, device=DEV),
+                                 n_head=H, scale=1.0, n_splits=splits, waves=4, chunk=256,
+                                 partials=torch.empty(H * splits * (hd + 4), device=DEV) if splits > 1 else None)
+        else:
+            out = run_attention(ops, case, H, hd, 1.0, 0, kernel, splits=(3 if T < 1000 else 11) if kernel == "decode" else 1)
         want = case["vs"][0][target, 0].float()
         assert torch.allclose(out[0, :hd].float().cpu(), want, atol=2e-2), f"{kernel}: key {target} was not found"
 
