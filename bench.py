@@ -267,6 +267,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has, if needed")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--positions", type=int, default=0, help="a longer context than the size's own (the position table grows), e.g. 8192 with --prompt 7000")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill of 2,048 tokens (for profiling)")
     ap.add_argument("--prefill-tokens", default="", help="e.g. 512,2048,8192: best-of-5 prefill tokens a second per length, "
@@ -297,6 +298,8 @@ def main():
     full_layers = cfg["n_layer"]
     if args.layers:
         cfg["n_layer"] = args.layers
+    if args.positions:
+        cfg["n_positions"] = args.positions
     ctx = cfg["n_positions"]
     steps = max(1, min(args.steps, ctx - args.prompt - args.warmup))
     short = "bf16" if args.dtype == "bfloat16" else "fp32"

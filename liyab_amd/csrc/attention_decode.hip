@@ -244,19 +244,35 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
 template <typename T>
 __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
                                        const float* __restrict__ partials, int n_head, int hd, int n_splits) {
+    // The splits' maxima and sums go to LDS first, a lane a split, and the values are fetched
+    // eight splits at a time before they are used: the sums below are one chain in split order,
+    // and a load at a time inside it would cost its latency once a split.
+    __shared__ float sm[64], sl[64];
     const int slot = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
-    if (e >= hd) return;
     const int t = tok_list != nullptr ? tok_list[slot] : slot;
     const float* p = partials + (static_cast<int64_t>(slot) * n_head + h) * n_splits * (hd + 4);
+    for (int z = e; z < n_splits; z += blockDim.x) {
+        sm[z] = p[z * (hd + 4) + hd];
+        sl[z] = p[z * (hd + 4) + hd + 1];
+    }
+    __syncthreads();
+    if (e >= hd) return;
     float M = -INFINITY;
-    for (int z = 0; z < n_splits; ++z) M = fmaxf(M, p[z * (hd + 4) + hd]);
+    for (int z = 0; z < n_splits; ++z) M = fmaxf(M, sm[z]);
     float sum = 0.0f, o = 0.0f;
-    for (int z = 0; z < n_splits; ++z) {
-        const float m = p[z * (hd + 4) + hd];
-        if (m == -INFINITY) continue;
-        const float w = exp_for<T>(m - M);
-        sum = fmaf(w, p[z * (hd + 4) + hd + 1], sum);
-        o = fmaf(w, p[z * (hd + 4) + e], o);
+    for (int z0 = 0; z0 < n_splits; z0 += 8) {
+        float a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = p[min(z0 + u, n_splits - 1) * (hd + 4) + e];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (z0 + u >= n_splits) break;
+            const float m = sm[z0 + u];
+            if (m == -INFINITY) continue;
+            const float w = exp_for<T>(m - M);
+            sum = fmaf(w, sl[z0 + u], sum);
+            o = fmaf(w, a[u], o);
+        }
     }
     out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = from_float<T>(o / sum);
 }
@@ -358,7 +374,7 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
 extern "C" int liyab_attention_merge(void* out, int out_dtype, int64_t out_stride, const float* partials, int n, int n_head,
                                      int hd, int n_splits, hipStream_t stream) {
     LIYAB_REQUIRE(out && partials, "attention_merge: null pointer");
-    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_head <= 65535 && hd > 0 && hd <= 1024 && n_splits >= 1, "attention_merge: bad sizes");
+    LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_head <= 65535 && hd > 0 && hd <= 1024 && n_splits >= 1 && n_splits <= 64, "attention_merge: bad sizes (at most 64 splits)");
     LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * hd, "attention_merge: the row stride is shorter than heads x head size");
     LIYAB_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "attention_merge: unknown dtype %d", out_dtype);
     if (n == 0) return 0;
