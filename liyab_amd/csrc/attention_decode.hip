@@ -251,6 +251,10 @@ __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, 
     const int slot = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
     const int t = tok_list != nullptr ? tok_list[slot] : slot;
     const float* p = partials + (static_cast<int64_t>(slot) * n_head + h) * n_splits * (hd + 4);
+    const int ec = min(e, hd - 1);
+    float a[8];  // the first eight splits' values are on their way while the maxima and sums go through LDS
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = p[min(u, n_splits - 1) * (hd + 4) + ec];
     for (int z = e; z < n_splits; z += blockDim.x) {
         sm[z] = p[z * (hd + 4) + hd];
         sl[z] = p[z * (hd + 4) + hd + 1];
@@ -261,9 +265,10 @@ __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, 
     for (int z = 0; z < n_splits; ++z) M = fmaxf(M, sm[z]);
     float sum = 0.0f, o = 0.0f;
     for (int z0 = 0; z0 < n_splits; z0 += 8) {
-        float a[8];
+        if (z0 > 0) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a[u] = p[min(z0 + u, n_splits - 1) * (hd + 4) + e];
+            for (int u = 0; u < 8; ++u) a[u] = p[min(z0 + u, n_splits - 1) * (hd + 4) + e];
+        }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             if (z0 + u >= n_splits) break;
