@@ -15,8 +15,8 @@
 // running maximum and sum of a query need one exchange with the lane 32 apart
 // instead of a reduction over 32 lanes. The accumulators then serve, rounded to
 // bfloat16, directly as the second operand of O^T = V^T P^T (contraction over
-// the keys); V is transposed once on its way into LDS (2-byte writes by the
-// staging threads), so that every wave reads its operand as 8-byte pieces.
+// the keys); V lies in LDS as it lies in the pages, and a wave reads its operand, four keys
+// of one dimension a lane, through gfx950's transposing read.
 // Exponentials are taken against a reference value that follows the running
 // maximum from below by at most 2^8: the outputs are rescaled only when a
 // query's maximum jumps past that, which is rare, instead of at every block.
@@ -38,6 +38,14 @@ namespace liyab {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+// Four 16-bit values through the transposing read of LDS: see where it is used.
+__device__ __forceinline__ uint2 tr_read4(const bf16_t* p) {
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s* lds_v4s;
+    const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(p));
+    return __builtin_bit_cast(uint2, v);
+}
 
 union QFrag {
     u32x4 u;
@@ -62,9 +70,10 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     constexpr int AP_DEPTH = kDepth / NS;  // the same bytes in flight whatever a step holds
     constexpr int STEP_KEYS = AP_KEYS * KS * NS;  // keys staged a step
     constexpr int STAGE = STEP_KEYS * LDK;
-    // values are kept transposed, [dimension][key of the step], rows padded by 4 keys: the 8-byte
-    // reads of 32 lanes (32 dimensions, one group of 4 keys) then fall in 64 different banks
-    constexpr int LDV = STEP_KEYS + 4, VSTAGE = HDP * LDV;
+    // values lie as the keys do, [key of the step][dimension]; the product's operand wants four
+    // keys of one dimension a lane, which the transposing read gives (ds_read_b64_tr_b16: 16 lanes
+    // that point at 4 keys x 16 dimensions get them back as 16 dimensions x 4 keys)
+    constexpr int VSTAGE = STAGE;
     // two stages of keys and of values (the next step's load while this one is used); after the
     // walk the same memory carries the partial results of the waves with ks > 0
     constexpr int PARTIAL = DB * 16 * 64 + 2 * 64;  // floats a wave: outputs, then maximum and sum
@@ -155,10 +164,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 const bool ok = kp >= k_lo && kp <= k_hi && col < hd;
                 const u32x4 zero = {0, 0, 0, 0};
                 *reinterpret_cast<u32x4*>(&Kb[buf * STAGE + key * LDK + col]) = ok ? fk[i] : zero;
-                QFrag vt;
-                vt.u = ok ? fv[i] : zero;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) Vb[buf * VSTAGE + (col + e) * LDV + key] = vt.h[e];
+                *reinterpret_cast<u32x4*>(&Vb[buf * VSTAGE + key * LDK + col]) = ok ? fv[i] : zero;
             }
         }
     };
@@ -177,7 +183,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
         fetch(kb_step + AP_DEPTH * STEP_KEYS, rk[ring], rv[ring]);  // this set's keys are in LDS already
         const int kb0w = kb_step + ks * NS * AP_KEYS;  // this wave's first block of the step; its NS blocks are consecutive
         const bf16_t* Ks = Kb + cur * STAGE + ks * NS * AP_KEYS * LDK;
-        const bf16_t* Vs = Vb + cur * VSTAGE + ks * NS * AP_KEYS;
+        const bf16_t* Vs = Vb + cur * VSTAGE + ks * NS * AP_KEYS * LDK;
         if (wave_has && kb0w <= wave_last) {
             // S^T[key][query] = sum_d K[key][d] Q[query][d], a block a stream. Every slab of the
             // padded head dimension, without a branch (queries and staged keys are zero past the head
@@ -266,10 +272,12 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                 for (int z = 0; z < NS; ++z)
 #pragma unroll
                     for (int s2 = 0; s2 < 2; ++s2) {
-                        // this lane: dimension 32 d + ql, keys 16 s2 + 4 g2 + {0..3} and the same + 8 of the stream's block
-                        const bf16_t* vrow = Vs + (32 * d + ql) * LDV + z * AP_KEYS + 16 * s2 + 4 * g2;
-                        vf[z][s2].u[0] = *reinterpret_cast<const uint2*>(vrow);
-                        vf[z][s2].u[1] = *reinterpret_cast<const uint2*>(vrow + 8);
+                        // this lane gets: dimension 32 d + ql, keys 16 s2 + 4 g2 + {0..3} and the same + 8 of the
+                        // stream's block. It points at: of its 16 lanes' 4 keys x 16 dimensions, key (lane % 16) / 4,
+                        // dimensions 4 (lane % 4) .. + 3.
+                        const bf16_t* vat = Vs + (z * AP_KEYS + 16 * s2 + 4 * g2 + (lane % 16) / 4) * LDK + 32 * d + 16 * ((lane % 32) / 16) + 4 * (lane % 4);
+                        vf[z][s2].u[0] = tr_read4(vat);
+                        vf[z][s2].u[1] = tr_read4(vat + 8 * LDK);
                     }
 #pragma unroll
                 for (int s2 = 0; s2 < 2; ++s2)
