@@ -643,7 +643,7 @@ def test_argmax_ties_go_to_the_lowest_id(ops, rows, V):
     assert out.tolist() == rnd(rows, V, seed=4).argmax(dim=1).tolist()
 
 
-@pytest.mark.parametrize("V", [1000, 50257, 60000, 70001])
+@pytest.mark.parametrize("V", [1000, 50257, 53250, 60000, 70001])
 def test_sampler_against_the_plain_sampler(ops, V):
     """Temperature, top-k and top-p per row against the plain implementation's rules, at
     vocabularies that take each of the sampling kernels (the row in registers with a one-wave
@@ -676,7 +676,7 @@ def test_sampler_against_the_plain_sampler(ops, V):
                 assert probs[got[r]] > 0 and np.abs(cdf - u[r]).min() < 1e-5, (V, r, params[r], got[r], want)
 
 
-@pytest.mark.parametrize("V", [3000, 50257, 65533])
+@pytest.mark.parametrize("V", [3000, 50257, 53250, 65533])
 def test_top_p_over_many_candidates_keeps_exactly_the_nucleus(ops, V):
     """Top-p alone (and with a top-k too wide for one wave) at rows made so that a wrong cut shows
     in the draws: a few heavy ids over a light floor, the cut falling between them, inside a run
