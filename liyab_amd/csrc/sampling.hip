@@ -621,7 +621,123 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     // ---- top-k: the k-th largest key, and how many of its ties are kept ----
     uint32_t tau_k = 0;
     int ties_k = 0x7fffffff;
+    // the bin of a key: its logit's distance under the largest, in kBins steps over the kMassBits powers
+    // of two that a mass can lie under the largest one's (a monotone function of the key)
+    auto bin_of = [&](uint32_t key) {
+        const float below = (lmax - key_value(key)) * inv_t;  // powers of two under the largest mass, >= 0
+        return static_cast<int>(fminf(below * (static_cast<float>(kBins) / kMassBits), static_cast<float>(kBins - 1)));
+    };
+    bool k_found = false;
     if (use_k) {
+        // by bins, as top-p below: the keys are counted in bins, one wave finds the bin that holds the
+        // k-th largest, that bin's keys alone are gathered, and the wave picks among them. A bin with
+        // more keys than the pool leaves it to the counting passes over the whole row.
+        uint32_t* bin_count = reinterpret_cast<uint32_t*>(bin_mass);
+        __syncthreads();
+        for (int i = tid; i < kBins + kBins / kBinPad; i += THREADS) bin_count[i] = 0u;
+        if (tid == 0) { bins_ok = 0; n_pool = 0; }
+        __syncthreads();
+        // (the last bin takes every key from 2^-44 of the largest mass down, often most of the row: those are
+        // counted in a register and added once a wave, not one atomic each on the same word)
+        int last_bin = 0;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            const uint32_t key = again(keys[j]);
+            if (key != 0u) {
+                const int b = bin_of(key);
+                if (b == kBins - 1) ++last_bin;
+                else atomicAdd(&bin_count[bin_slot(b)], 1u);
+            }
+        }
+        last_bin = wave_sum_i(last_bin);
+        if (lane == 0 && last_bin != 0) atomicAdd(&bin_count[bin_slot(kBins - 1)], static_cast<uint32_t>(last_bin));
+        __syncthreads();
+        if (wave == 0) {
+            constexpr int PER_LANE = kBins / kWave;
+            int mine_sum = 0;
+#pragma unroll
+            for (int i = 0; i < PER_LANE; ++i) mine_sum += static_cast<int>(bin_count[bin_slot(lane * PER_LANE + i)]);
+            int incl = mine_sum;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                const int o = __shfl_up(incl, d, kWave);
+                if (lane >= d) incl += o;
+            }
+            const unsigned long long reached = __ballot(incl >= k);
+            if (reached != 0ull && lane == __ffsll(static_cast<long long>(reached)) - 1) {
+                int cum = incl - mine_sum;
+                for (int i = 0; i < PER_LANE; ++i) {
+                    const int next = cum + static_cast<int>(bin_count[bin_slot(lane * PER_LANE + i)]);
+                    if (next >= k) {
+                        bin_star = lane * PER_LANE + i;
+                        bins_above = static_cast<unsigned long long>(cum);
+                        bins_ok = 1;
+                        break;
+                    }
+                    cum = next;
+                }
+            }
+        }
+        __syncthreads();
+        if (bins_ok != 0) {
+            const int star = bin_star;
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const uint32_t key = again(keys[j]);
+                if (key != 0u && bin_of(key) == star) {
+                    const int at = atomicAdd(&n_pool, 1);  // the order of arrival does not matter: only keys count here
+                    if (at < kPool) pool_key[at] = key;
+                }
+            }
+            __syncthreads();
+            const int n = n_pool;
+            if (n <= kPool) {
+                if (wave == 0) {
+                    constexpr int PER = kPool / kWave;
+                    const int want = k - static_cast<int>(bins_above);  // the k-th largest of the row is the want-th largest of this bin
+                    uint32_t pk[PER];
+                    uint32_t lo = 0xffffffffu, hi = 0u;
+#pragma unroll
+                    for (int i = 0; i < PER; ++i) {
+                        const int e = lane + kWave * i;
+                        pk[i] = e < n ? pool_key[e] : 0u;
+                        if (e < n) { lo = min(lo, pk[i]); hi = max(hi, pk[i]); }
+                    }
+#pragma unroll
+                    for (int off = kWave / 2; off > 0; off >>= 1) {
+                        lo = min(lo, static_cast<uint32_t>(__shfl_xor(static_cast<int>(lo), off, kWave)));
+                        hi = max(hi, static_cast<uint32_t>(__shfl_xor(static_cast<int>(hi), off, kWave)));
+                    }
+                    const int open_bits = lo == hi ? 0 : 32 - __clz(lo ^ hi);
+                    uint32_t t = open_bits >= 32 ? 0u : (hi >> open_bits) << open_bits;
+                    for (int bit = open_bits - 1; bit >= 0; --bit) {
+                        const uint32_t cand = t | (1u << bit);
+                        int c = 0;
+#pragma unroll
+                        for (int i = 0; i < PER; ++i)
+                            if (i * kWave < n) c += __popcll(__ballot(pk[i] >= cand));
+                        if (c >= want) t = cand;
+                    }
+                    int above = 0;
+#pragma unroll
+                    for (int i = 0; i < PER; ++i)
+                        if (i * kWave < n) above += __popcll(__ballot(pk[i] > t));
+                    if (lane == 0) {
+                        found_tau = t;
+                        found_ties = want - above;
+                    }
+                }
+                __syncthreads();
+                tau_k = found_tau;
+                ties_k = found_ties;
+                k_found = true;
+            }
+        }
+        __syncthreads();
+        if (tid == 0) n_pool = 0;  // (the pool serves top-p next)
+        __syncthreads();
+    }
+    if (use_k && !k_found) {
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = tau_k | (1u << bit);
             int c = 0;
@@ -663,10 +779,6 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
         // A bin with more keys than the pool holds (thousands of nearly equal logits), or nothing
         // to cut, leaves it to the bisection.
         const unsigned long long tie_mass = use_k ? static_cast<unsigned long long>(ties_k) * fixed_mass(tau_k, lmax, inv_t) : 0ull;
-        auto bin_of = [&](uint32_t key) {
-            const float below = (lmax - key_value(key)) * inv_t;  // powers of two under the largest mass, >= 0
-            return static_cast<int>(fminf(below * (static_cast<float>(kBins) / kMassBits), static_cast<float>(kBins - 1)));
-        };
         for (int i = tid; i < kBins + kBins / kBinPad; i += THREADS) bin_mass[i] = 0ull;
         if (tid == 0) bins_ok = 0;
         __syncthreads();
