@@ -477,7 +477,7 @@ sample_registers_kernel(int* __restrict__ out, const float* __restrict__ logits,
     uint32_t bits[(EPT + 31) / 32];
     // is id j of this thread kept? (PLAIN: every element of the row is)
     // (the word of bits is read afresh each time, for the same reason: no lane mask an id is kept between the passes)
-    auto is_kept = [&](int j) { return PLAIN ? keys[j] != 0u : ((again(bits[j / 32]) >> (j % 32)) & 1u) != 0u; };
+    auto is_kept = [&](int j) { return PLAIN ? again(keys[j]) != 0u : ((again(bits[j / 32]) >> (j % 32)) & 1u) != 0u; };
     if constexpr (!PLAIN) {
     // ---- one wave among at most 64 candidates in cand_key / cand_id: nucleus cut and draw ----
     auto wave_finish = [&]() {
