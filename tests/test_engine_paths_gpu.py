@@ -348,3 +348,31 @@ def test_contexts_of_thousands_of_positions(dtype, tmp_path):
         tt.check_against_plain(got, reqs, refs, TOL[dtype], f"4,100 positions {label} {dtype}", family="long context")
         core.manager.check()
         del core
+
+
+# ---------------------------------------------------------------------------
+# layers far wider than GPT-2's own
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layers_of_width_4096(dtype, tmp_path):
+    """Width 4,096, 32 heads of 128, a feed-forward of 16,384: inner dimensions past what the
+    kernel with the norm folded in takes (2,048), more output features than the streaming
+    kernels take (8,192), heads of 128. Whole, most in one step with a tail token by token,
+    and mixed, against the plain implementation."""
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 2, "n_embd": 4096, "n_head": 32, "n_inner": 16384, "vocab_size": 3000,
+           "n_positions": 200, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    write_random_model(str(tmp_path), cfg, 5)
+    config, tensors = plain.read_model(str(tmp_path))
+    weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+    reqs = {f"w{i}": tt.random_tokens(40 + i, n, 3000) for i, n in enumerate([200, 37, 3, 90])}
+    refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+    for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=3, decode_tail=6)),
+                         ("bulk+tail", tt.schedule_bulk_tail(reqs, tail=8))):
+        core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, refs, TOL[dtype], f"width 4,096 {label} {dtype}", family="sizes:wide")
+        core.manager.check()
+        del core
