@@ -38,9 +38,12 @@ SMALL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 
          "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "layer_norm_epsilon": 1e-5,
          "activation_function": "gelu_new", "tie_word_embeddings": True}
 # GPT-2's other sizes, for --size: the layer sizes and, with them, the number of layers
-WEIGHT_SEEDS = {"small": 10, "medium": 20, "xl": 30}
+# ("wide": no GPT-2 of anybody's, but the architecture at layer sizes where a decode step is bound by the weights' bytes, not by
+# its chain of kernels: 403 MB of matrices a layer; run it with --layers 8 or so)
+WEIGHT_SEEDS = {"small": 10, "medium": 20, "xl": 30, "wide": 40}
 SIZES = {"small": {}, "medium": {"n_layer": 24, "n_embd": 1024, "n_head": 16, "n_inner": 4096},
-         "xl": {"n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400}}
+         "xl": {"n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400},
+         "wide": {"n_layer": 32, "n_embd": 4096, "n_head": 32, "n_inner": 16384}}
 
 
 def weight_bytes(cfg, elt):
@@ -263,7 +266,7 @@ def main():
     ap.add_argument("--steps", type=int, default=504)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--size", default="small", choices=sorted(SIZES), help="GPT-2 small's sizes (the default), medium's or XL's")
+    ap.add_argument("--size", default="small", choices=sorted(SIZES), help="GPT-2 small's sizes (the default), medium's or XL's; or layers of width 4,096")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has, if needed")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt", type=int, default=512)

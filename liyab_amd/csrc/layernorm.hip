@@ -138,6 +138,70 @@ layernorm_wave_kernel(T* __restrict__ out, const float* __restrict__ x, const fl
         if (lane + kWave * j < nv) store_row4<T>(o + 4 * (lane + kWave * j), (v[j] - mean) * scale * gw[j] + gb[j]);
 }
 
+// The same for wider rows (d a multiple of 4, at most THREADS * 4 * MAXV): a workgroup a row,
+// the row in its threads' registers, sums across the waves through LDS.
+template <typename T, int THREADS, int MAXV, bool PARTS>
+__global__ void __launch_bounds__(THREADS)
+layernorm_block_kernel(T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+                       const float* __restrict__ b, const int* __restrict__ rows, int d, float eps, PartSums ps) {
+    __shared__ float red[THREADS / kWave];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int64_t src = rows != nullptr ? rows[r] : r;
+    const float* row0 = x + src * d;
+    const int nv = d / 4;
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f}, one = {1.0f, 1.0f, 1.0f, 1.0f};
+    f32x4 v[MAXV], gw[MAXV], gb[MAXV];
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int i = min(tid + THREADS * j, nv - 1);  // past the row: its last piece again, unused
+        v[j] = reinterpret_cast<const f32x4*>(row0)[i];
+        gw[j] = w != nullptr ? reinterpret_cast<const f32x4*>(w)[i] : one;
+        gb[j] = b != nullptr ? reinterpret_cast<const f32x4*>(b)[i] : zero;
+    }
+    if constexpr (PARTS) {
+        // the further planes in their order, two planes' loads in flight together
+        constexpr int PB = 2;
+        for (int q0 = 1; q0 < ps.n_parts; q0 += PB) {
+            f32x4 plane[PB][MAXV];
+#pragma unroll
+            for (int u = 0; u < PB; ++u) {
+                const float* row = row0 + min(q0 + u, ps.n_parts - 1) * ps.stride;
+#pragma unroll
+                for (int j = 0; j < MAXV; ++j) plane[u][j] = reinterpret_cast<const f32x4*>(row)[min(tid + THREADS * j, nv - 1)];
+            }
+#pragma unroll
+            for (int u = 0; u < PB; ++u)
+#pragma unroll
+                for (int j = 0; j < MAXV; ++j)
+                    if (q0 + u < ps.n_parts) v[j] += plane[u][j];
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j)
+        if (tid + THREADS * j < nv) s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+    const float mean = block_sum<THREADS>(s, red) / static_cast<float>(d);
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j)
+        if (tid + THREADS * j < nv) {
+            const f32x4 dev = v[j] - mean;
+            ss += (dev[0] * dev[0] + dev[1] * dev[1]) + (dev[2] * dev[2] + dev[3] * dev[3]);
+        }
+    const float scale = 1.0f / sqrtf(block_sum<THREADS>(ss, red) / static_cast<float>(d) + eps);
+    T* o = out + static_cast<int64_t>(r) * d;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j)
+        if (tid + THREADS * j < nv) store_row4<T>(o + 4 * (tid + THREADS * j), (v[j] - mean) * scale * gw[j] + gb[j]);
+}
+
+template <typename T, int THREADS>
+void launch_block(T* out, const float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
+                  const PartSums& ps, hipStream_t stream) {
+    if (ps.n_parts > 1) layernorm_block_kernel<T, THREADS, 4, true><<<n, THREADS, 0, stream>>>(out, x, w, b, rows, d, eps, ps);
+    else layernorm_block_kernel<T, THREADS, 4, false><<<n, THREADS, 0, stream>>>(out, x, w, b, rows, d, eps, ps);
+}
+
 // out[i] = planes[0][i] + planes[1][i] + ..., added up in that order (the norm kernels' order).
 __global__ void __launch_bounds__(256) sum_parts_kernel(float* out, const float* planes, int64_t total, PartSums ps) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -155,24 +219,28 @@ void launch_wave(T* out, const float* x, const float* w, const float* b, const i
     else layernorm_wave_kernel<T, MAXV, false><<<grid, 256, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
 }
 
-// Whether the kernel with a wave per row takes these operands (the only one that adds planes up).
-static bool wave_takes(const void* out, const float* x, const float* w, const float* b, int d, int64_t stride) {
+// Whether the kernels that keep a row in registers take these operands (the only ones that add planes up):
+// a wave a row up to a width of 2,048, a workgroup a row beyond.
+constexpr int kWaveWidth = 2048, kBlockWidth = 16384;
+static bool registers_take(const void* out, const float* x, const float* w, const float* b, int d, int64_t stride) {
     auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    return d % 4 == 0 && d <= 2048 && al16(out) && al16(x) && al16(w) && al16(b) && stride % 4 == 0;
+    return d % 4 == 0 && d <= kBlockWidth && al16(out) && al16(x) && al16(w) && al16(b) && stride % 4 == 0;
 }
 
 template <typename T>
 int launch_layernorm(T* out, const float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
                      const PartSums& ps, hipStream_t stream) {
-    if (wave_takes(out, x, w, b, d, ps.stride)) {
-        if (d <= 256) launch_wave<T, 1>(out, x, w, b, rows, n, d, eps, ps, stream);
+    if (registers_take(out, x, w, b, d, ps.stride)) {
+        if (d > 4096) launch_block<T, 1024>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else if (d > kWaveWidth) launch_block<T, 256>(out, x, w, b, rows, n, d, eps, ps, stream);
+        else if (d <= 256) launch_wave<T, 1>(out, x, w, b, rows, n, d, eps, ps, stream);
         else if (d <= 512) launch_wave<T, 2>(out, x, w, b, rows, n, d, eps, ps, stream);
         else if (d <= 768) launch_wave<T, 3>(out, x, w, b, rows, n, d, eps, ps, stream);
         else if (d <= 1024) launch_wave<T, 4>(out, x, w, b, rows, n, d, eps, ps, stream);
         else launch_wave<T, 8>(out, x, w, b, rows, n, d, eps, ps, stream);
         return check_launch("layernorm");
     }
-    LIYAB_REQUIRE(ps.n_parts <= 1, "layernorm: rows in %d planes need a width that is a multiple of 4, at most 2048 (got %d), and 16-byte alignment",
+    LIYAB_REQUIRE(ps.n_parts <= 1, "layernorm: rows in %d planes need a width that is a multiple of 4, at most 16384 (got %d), and 16-byte alignment",
                   ps.n_parts, d);
     if (d <= 256) layernorm_kernel<T, 64><<<n, 64, 0, stream>>>(out, x, w, b, rows, d, eps);
     else layernorm_kernel<T, 256><<<n, 256, 0, stream>>>(out, x, w, b, rows, d, eps);
@@ -197,7 +265,7 @@ extern "C" int liyab_layernorm(void* out, int out_dtype, const float* x, const f
 
 // The same over rows given as a sum of planes: row r is planes[0][r] + planes[1][r] + ...
 // (n_parts planes [x_rows, d], part_stride floats apart), added in that order. d must be a
-// multiple of 4, at most 2048, and the operands 16-byte aligned (liyab_sum_parts first otherwise).
+// multiple of 4, at most 16,384, and the operands 16-byte aligned (liyab_sum_parts first otherwise).
 extern "C" int liyab_layernorm_parts(void* out, int out_dtype, const float* planes, int n_parts, int64_t part_stride,
                                      int x_rows, const float* w, const float* b, const int* rows, int n, int d, float eps,
                                      hipStream_t stream) {

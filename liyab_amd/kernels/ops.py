@@ -228,7 +228,7 @@ def _planes(x: torch.Tensor, what: str):
 
 def norm_takes_planes(d: int) -> bool:
     """Whether the norm kernel adds planes up as it loads a row of this width (sum_parts first otherwise)."""
-    return d % 4 == 0 and d <= 2048
+    return d % 4 == 0 and d <= 16384
 
 
 def layernorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],

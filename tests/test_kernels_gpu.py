@@ -50,7 +50,8 @@ def test_embed_and_add_rows(ops, dtype, n, d):
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n,d,eps", [(1, 64, 1e-5), (9, 96, 1e-6), (40, 1600, 1e-5), (3, 777, 1e-3), (5, 768, 1e-5),
-                                     (70, 260, 1e-5), (6, 1028, 1e-6), (7, 2048, 1e-5), (2, 2052, 1e-5)])
+                                     (70, 260, 1e-5), (6, 1028, 1e-6), (7, 2048, 1e-5), (2, 2052, 1e-5), (4, 4096, 1e-5), (3, 5120, 1e-6),
+                                     (2, 16384, 1e-5), (2, 16388, 1e-5), (3, 4098, 1e-5)])
 def test_layernorm(ops, out_dtype, n, d, eps):
     x = rnd(n + 3, d, scale=3.0) + 1.5
     w, b = rnd(d, seed=2) + 1.0, rnd(d, seed=3)
@@ -71,7 +72,8 @@ def test_layernorm(ops, out_dtype, n, d, eps):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,d,parts", [(1, 64, 1), (9, 96, 4), (16, 768, 4), (5, 1600, 2), (7, 2048, 5), (6, 200, 16), (70, 768, 3)])
+@pytest.mark.parametrize("n,d,parts", [(1, 64, 1), (9, 96, 4), (16, 768, 4), (5, 1600, 2), (7, 2048, 5), (6, 200, 16), (70, 768, 3),
+                                       (5, 4096, 3), (2, 8192, 4), (3, 2052, 2)])
 def test_layernorm_over_rows_in_planes(ops, out_dtype, n, d, parts):
     """Rows given as a sum of planes: the norm adds the planes up, in their order, as it loads a
     row, also over gathered rows; sum_parts alone does the same sum (into a tensor of its own or
