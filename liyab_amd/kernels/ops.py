@@ -690,9 +690,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
         return
     if mfma_takes(a, w):
         M, N = a.shape[0], w.shape[0]
-        if 12 < M <= 128 and N >= 16384 and a.shape[1] % 64 == 0:
+        if 12 < M <= 128 and N >= 16384 and a.shape[1] % 64 == 0 and (N + 127) // 128 >= compute_units():
             # a vocabulary's worth of output features: large tiles re-read the tokens least
-            # (16 rows: 22.5 against 25.1 us for 768 -> 50,257; 64 rows: 27.9 against 32.9)
+            # (16 rows: 22.5 against 25.1 us for 768 -> 50,257; 64 rows: 27.9 against 32.9); with fewer such tiles
+            # than compute units they stream too slowly (4,096 -> 16,384 at 64 rows: 128 tiles, 65 us)
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=8)
         elif ((M > 32 or (M > 16 and N * a.shape[1] >= 6 << 20)) and a.shape[1] % 64 == 0 and N >= 2048
               and (M + 63) // 64 * ((N + 31) // 32) <= compute_units()):
