@@ -505,11 +505,18 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
                   "gemm_mfma_dl: operands must be 16-byte aligned");
     EpiParams epi = *epi_in;
     if (int rc = check_epilogue(epi, M, N)) return rc;
-    // measured on {256..2048} x {768, 2304, 3072} x {768, 3072}: 64 x 64 tiles, three workgroups a
-    // CU, win or tie nearly everywhere; a long K likes one more stage in flight; a large output
+    // measured on {256..8192} x {768 .. 16,384} x {768 .. 16,384}: 64 x 64 tiles, three workgroups a
+    // CU, win or tie for small outputs; a long K likes one more stage in flight; a large output
     // (2,048 x 2,304 and up) likes 128 x 128 tiles, two stages deep, on eight waves (16.9 us against
     // 17.3 for 2,048 x 2,304 x 768, 18.0 against 22.6 for 2,048 x 3,072 x 768)
-    if (tile == 0) tile = K >= 2048 ? 6 : (static_cast<long>(M) * N >= 2048L * 2048L ? 8 : 2);
+    // A large output takes the 128 x 128 tiles whatever K (2,048 x 16,384 x 4,096: 0.85 PFLOP/s against 0.46 in
+    // tiles of 64 x 64), a somewhat smaller one with a long K too (2,048 x 1,600 x 6,400: 79 against 88 us); the
+    // fourth stage pays while the tiles of 64 x 64 are few enough for its LDS (4,096 x 768 x 3,072, 768 tiles:
+    // 36 us with three stages, 49 with four).
+    if (tile == 0) {
+        const long out = static_cast<long>(M) * N, tiles64 = static_cast<long>((M + 63) / 64) * ((N + 63) / 64);
+        tile = (out >= 2048L * 2048L || (out >= 2560L * 1024L && K >= 4096)) ? 8 : ((K >= 2048 && tiles64 < 640) ? 6 : 2);
+    }
     switch (tile) {
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
