@@ -44,7 +44,7 @@ def test_attention_split_plan(ops):
 def test_what_the_folded_norm_takes(ops):
     assert ops.skinny_ln_takes(1, 64) and ops.skinny_ln_takes(32, 2048)
     assert not ops.skinny_ln_takes(33, 768) and not ops.skinny_ln_takes(8, 2056) and not ops.skinny_ln_takes(8, 100)
-    assert ops.norm_takes_planes(768) and not ops.norm_takes_planes(777) and not ops.norm_takes_planes(4096)
+    assert ops.norm_takes_planes(768) and not ops.norm_takes_planes(777) and ops.norm_takes_planes(16384) and not ops.norm_takes_planes(16388)
 
 
 def test_attention_tile_of_a_step():
