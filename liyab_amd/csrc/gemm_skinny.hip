@@ -13,8 +13,8 @@
 // read once, straight from global memory into registers, 16 bytes a lane,
 // one trip ahead of the multiplies; the tokens' rows come from L2 (every
 // workgroup reads all of them: few, wide tiles of N would starve most CUs).
-// K must be a multiple of 8. The order of the sum depends on K and the split
-// only, never on M.
+// K must be a multiple of 8. The order of the sum depends on the output feature, K and the
+// split only, never on M.
 //
 // The product may be cut over K into parts (blockIdx.z), each part's sums going to its own
 // plane of 32-bit sums; the first plane may take the bias and the rows the product is to be
@@ -84,8 +84,21 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
             }
         }
     };
+    // How K goes to the waves. As a rule a trip of the workgroup is UPT * ksplit consecutive
+    // units, one wave after the other, and the next trip the next such stretch. Where rows lie
+    // a multiple of 32 KB apart (K a multiple of 16,384), the sixteen rows of a workgroup, and
+    // every workgroup's, begin in the same few memory channels, and workgroups in step crowd
+    // those: there a wave walks a block of consecutive trips of its own, and a workgroup starts
+    // blockIdx.x mod trips trips into its blocks and goes round past their end (16,384 ->
+    // 4,096 in a decode step: 34.3 -> 28.3 us; at rows of 8 KB the same walk is no faster in
+    // a step, though up to 12 % faster alone). The order of a sum depends on the output
+    // feature, K and the split only, never on M.
+    const bool blocks = K % 16384 == 0;
+    const int trips = max(1, (units + UPT * ksplit - 1) / (UPT * ksplit));
+    int trip = blocks ? static_cast<int>(blockIdx.x % trips) : 0;
+    auto unit_of = [&](int t) { return blocks ? (wave * trips + t) * UPT : (t * ksplit + wave) * UPT; };
     Frag wc[UPT][NT][2];
-    load_w(wave * UPT, wc);
+    load_w(unit_of(trip), wc);
     // what the epilogue will read for this thread's first output (bias, residual) is asked for
     // now: after the sums it would be one more trip to memory on the critical path
     const int e_m = m0 + 16 * ((tid / 256) / NT) + (tid % 256) / 16, e_n = n0 + 16 * ((tid / 256) % NT) + tid % 16;
@@ -126,7 +139,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
         }
     };
     Frag xc[UPT][MT][2];
-    load_x(wave * UPT, xc);
+    load_x(unit_of(trip), xc);
 
     floatx4 acc[MT][NT];
 #pragma unroll
@@ -147,11 +160,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     };
     // every trip but the last asks for the next trip's operands before it multiplies; the last
     // one is peeled off, so no trip asks for (and then waits for) operands nobody uses
-    int u0 = wave * UPT;
-    for (; u0 + UPT * ksplit < units; u0 += UPT * ksplit) {
+    for (int left = trips - 1; left > 0; --left) {
+        trip = trip + 1 == trips ? 0 : trip + 1;
         Frag wn[UPT][NT][2], xn[UPT][MT][2];
-        load_w(u0 + UPT * ksplit, wn);
-        load_x(u0 + UPT * ksplit, xn);
+        load_w(unit_of(trip), wn);
+        load_x(unit_of(trip), xn);
         multiply();
 #pragma unroll
         for (int p = 0; p < UPT; ++p) {

@@ -123,8 +123,15 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
             f[p][1].u = piece(wrow, k + 32, k_end);
         }
     };
+    // K goes to the waves as in gemm_skinny_kernel (trips of consecutive units, or, where rows
+    // lie a multiple of 32 KB apart, a block of trips a wave begun blockIdx.x mod trips trips
+    // in): the same bits
+    const bool blocks = K % 16384 == 0;
+    const int trips = max(1, (units + 2 * WAVES - 1) / (2 * WAVES));
+    int trip = blocks ? static_cast<int>(blockIdx.x % trips) : 0;
+    auto unit_of = [&](int t) { return blocks ? (wave * trips + t) * 2 : (t * WAVES + wave) * 2; };
     Frag wc[2][2];
-    load_w(wave * 2, wc);
+    load_w(unit_of(trip), wc);
     const int e_m = 16 * (tid / 256) + (tid % 256) / 16, e_n = n0 + tid % 16;  // tile tid / 256 of rows
     const bool e_mine = tid < MT * 256 && e_m < M && e_n < N;
     const bool based = base.planes != nullptr && blockIdx.z == 0;
@@ -167,10 +174,11 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
             }
         }
     };
-    int u0 = wave * 2;
-    for (; u0 + 2 * WAVES < units; u0 += 2 * WAVES) {
+    for (int left = trips - 1; left > 0; --left) {
+        const int u0 = unit_of(trip);
+        trip = trip + 1 == trips ? 0 : trip + 1;
         Frag wn[2][2];
-        load_w(u0 + 2 * WAVES, wn);
+        load_w(unit_of(trip), wn);
         multiply(u0);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -178,7 +186,7 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
             wc[p][1] = wn[p][1];
         }
     }
-    multiply(u0);  // a wave past the end of the part holds zeros
+    multiply(unit_of(trip));  // a wave past the end of the part holds zeros
     // acc[r][c] = partial C^T[n = 4 g + c][m = 16 r + i]; kept [tile][m][n] per wave, added up in wave order
 #pragma unroll
     for (int r = 0; r < MT; ++r)
