@@ -13,7 +13,10 @@ namespace liyab {
 
 // An id below zero is a reference: -1 - id indexes `last_tokens`, where the sampler left the
 // token a request drew in the step before (the host may not have seen it yet).
-template <typename T>
+// WIDE: rows whose width is a multiple of 16 bytes' worth of elements are read 16 bytes a lane,
+// all of a lane's loads asked for before the first is used (one element a lane and trip, a
+// row of 4,096 took 14 us of waiting for one load after the other).
+template <typename T, bool WIDE>
 __global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ tok, const T* __restrict__ pos,
                              const int* __restrict__ ids, const int* __restrict__ positions, int d, float scale,
                              const int* __restrict__ last_tokens) {
@@ -23,10 +26,30 @@ __global__ void embed_kernel(float* __restrict__ x, const T* __restrict__ tok, c
     const T* trow = tok + id * d;
     const T* prow = pos != nullptr ? pos + static_cast<int64_t>(positions[t]) * d : nullptr;
     float* out = x + static_cast<int64_t>(t) * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = to_float<T>(trow[i]) * scale;
-        if (prow != nullptr) v += to_float<T>(prow[i]);
-        out[i] = v;
+    if constexpr (WIDE) {
+        constexpr int V = 16 / sizeof(T);
+        struct alignas(16) Piece {
+            T e[V];
+        };
+        for (int i = threadIdx.x * V; i < d; i += blockDim.x * V) {
+            const Piece a = *reinterpret_cast<const Piece*>(trow + i);
+            Piece b = a;
+            if (prow != nullptr) b = *reinterpret_cast<const Piece*>(prow + i);
+            float v[V];
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                v[j] = to_float<T>(a.e[j]) * scale;
+                if (prow != nullptr) v[j] += to_float<T>(b.e[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < V; j += 4) *reinterpret_cast<float4*>(out + i + j) = make_float4(v[j], v[j + 1], v[j + 2], v[j + 3]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < d; i += blockDim.x) {
+            float v = to_float<T>(trow[i]) * scale;
+            if (prow != nullptr) v += to_float<T>(prow[i]);
+            out[i] = v;
+        }
     }
 }
 
@@ -110,13 +133,19 @@ extern "C" int liyab_embed(float* x, const void* tok, const void* pos, int dtype
     LIYAB_REQUIRE(pos == nullptr || positions != nullptr, "embed: a position table needs positions");
     LIYAB_REQUIRE(d > 0 && n >= 0, "embed: bad sizes n=%d d=%d", n, d);
     if (n == 0) return 0;
-    const int threads = d >= 256 ? 256 : 64;
+    auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool wide = d % (dtype == kF32 ? 4 : 8) == 0 && aligned(x) && aligned(tok) && aligned(pos);
+    auto launch = [&](auto* table, auto* positions_table) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(table)>>;
+        const int lanes = wide ? d / static_cast<int>(16 / sizeof(T)) : d;
+        const int threads = lanes > 512 ? 1024 : (lanes > 256 ? 512 : (lanes > 64 ? 256 : 64));
+        if (wide) embed_kernel<T, true><<<n, threads, 0, stream>>>(x, table, positions_table, ids, positions, d, scale, last_tokens);
+        else embed_kernel<T, false><<<n, threads, 0, stream>>>(x, table, positions_table, ids, positions, d, scale, last_tokens);
+    };
     if (dtype == kF32) {
-        embed_kernel<float><<<n, threads, 0, stream>>>(x, static_cast<const float*>(tok), static_cast<const float*>(pos),
-                                                       ids, positions, d, scale, last_tokens);
+        launch(static_cast<const float*>(tok), static_cast<const float*>(pos));
     } else if (dtype == kBF16) {
-        embed_kernel<bf16_t><<<n, threads, 0, stream>>>(x, static_cast<const bf16_t*>(tok),
-                                                        static_cast<const bf16_t*>(pos), ids, positions, d, scale, last_tokens);
+        launch(static_cast<const bf16_t*>(tok), static_cast<const bf16_t*>(pos));
     } else {
         return fail(1, "embed: unknown dtype %d", dtype);
     }

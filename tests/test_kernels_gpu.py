@@ -32,7 +32,7 @@ def close(got, want, tol, what=""):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,d", [(1, 64), (7, 100), (33, 1600), (5, 4096 + 24)])
+@pytest.mark.parametrize("n,d", [(1, 64), (7, 100), (33, 1600), (5, 4096 + 24), (3, 4096), (2, 777), (4, 8200), (9, 768)])
 def test_embed_and_add_rows(ops, dtype, n, d):
     V, P = 321, 77
     table, pos = rnd(V, d, dtype=dtype), rnd(P, d, dtype=dtype, seed=1)
