@@ -817,18 +817,27 @@ def prefill_takes(hd: int) -> bool:
 
 
 def decode_plan(n_tokens: int, n_head: int, context_bucket: int):
-    """(splits of the keys, waves per workgroup), from measurements at 12 heads of 64: with many
-    (token, head) pairs a workgroup of 4 waves per pair is fastest, with a few hundred one of 8
-    (us a decode step at batch 24 / 32 / 40 with 4, 8 and 16 waves: 610 595 654 / 648 633 692 /
-    706 698 755; at batch 48 and more 4 waves win by a little); with few, 16 waves per pair,
-    merged in LDS, beat cutting the keys across workgroups plus a merge kernel up to a few
-    thousand keys; beyond that the keys are also split across workgroups."""
+    """(splits of the keys, waves per workgroup) for tokens whose attention the kernel finishes
+    itself (several splits: plus the merge kernel). `context_bucket`: the most keys a token has,
+    rounded up. From measurements at 12 to 32 heads of 64 and 128, 1 to 8 tokens and 300 to
+    4,000 keys (us, attention and merge): with many (token, head) pairs a workgroup of 4 waves
+    a pair is fastest, with a few hundred one of 8 (a decode step at batch 24 / 32 / 40 with 4,
+    8 and 16 waves: 610 595 654 / 648 633 692 / 706 698 755; 200 pairs at 544 / 2,000 keys: 7.1
+    / 19.7 with 8 waves, 8.9 / 20.0 with 16). With fewer pairs than would fill the chip the keys
+    are cut across workgroups of 4 waves, into 4, 8 or 16 splits of 128 keys or more, while
+    pairs x splits stay within the chip's 256 compute units (32 pairs of 128 dimensions at
+    1,000 / 2,000 / 4,000 keys: 7.5 / 10.6 / 18.4 in 8 splits against 11.8 / 19.1 / 33.1 uncut
+    on 16 waves; 12 pairs of 64: 6.9 / 7.8 / 9.7 against 8.7 / 11.8 / 18.6). Two splits never
+    beat 8 waves uncut. Uncut, 16 waves a pair pay from 4,000 keys on only."""
     pairs = max(1, n_tokens * n_head)
     if pairs >= 512 or context_bucket <= 256:
         return 1, 4
-    if pairs >= 256:
-        return 1, 8
-    return max(1, min(context_bucket // 2048, 32)), 16
+    splits = 1
+    while splits < 16 and pairs * splits * 2 <= 256 and context_bucket // (splits * 2) >= 128:
+        splits *= 2
+    if splits >= 4:
+        return splits, 4
+    return 1, (16 if context_bucket >= 4096 and pairs < 256 else 8)
 
 
 def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int):
@@ -879,7 +888,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
             and out.stride(0) % 8 == 0)
 
     def decode(tok_list, n):
-        splits, waves = decode_plan(n, n_head, plan.context_bucket)
+        splits, waves = decode_plan(n, n_head, min(plan.context_bucket, window) if window > 0 else plan.context_bucket)
         partials = None
         if splits > 1:
             partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32)
