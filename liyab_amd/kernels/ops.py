@@ -586,7 +586,16 @@ def tiled_k_parts(M: int, N: int, K: int) -> int:
     if K % 64 != 0 or M <= 32 or _invariant:
         return 1
     if M <= 64:
-        return 4 if K >= 3072 and N <= 2048 else 1
+        if N <= 2048:
+            return 4 if K >= 3072 else 1
+        # more output features: tiles of 64 x 64 (every tile reads all the rows: 32 x 32 tiles read
+        # them twice as often as the weights), cut while tiles x parts stay within the chip (us at 64
+        # rows, alone: 16,384 -> 4,096 42.2 whole in 32 x 32 tiles, 32.3 in 64 x 64 and 4 parts; 4,096
+        # -> 4,096 13.5 and 9.7; 8,192 -> 8,192 34.8 and 31.6 in 2 parts)
+        tiles, parts = (N + 63) // 64, 1
+        while parts < 4 and tiles * parts * 2 <= 256 and K // 64 // (parts * 2) >= 8:  # (256: the compute units of the part this was measured on)
+            parts *= 2
+        return parts
     # several tiles of rows (a prompt's portion): 64 x 64 tiles, cut until they cover the chip,
     # a part keeping 256 of K or more
     tiles = (M + 63) // 64 * ((N + 63) // 64)

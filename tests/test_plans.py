@@ -14,8 +14,8 @@ def test_parts_of_k_are_whole_and_none_is_empty(ops):
     """A product cut over K: every part holds whole units of 64 and at least one of them, for
     every shape the rules answer for."""
     for M in (1, 3, 8, 16, 17, 24, 32, 33, 48, 64, 65, 128, 200, 512, 2048):
-        for N in (16, 100, 768, 1024, 1600, 2304, 4800, 50257):
-            for K in (8, 64, 72, 192, 768, 1024, 1600, 3072, 4096, 6400, 8192):
+        for N in (16, 100, 768, 1024, 1600, 2304, 4096, 4800, 8192, 16384, 50257):
+            for K in (8, 64, 72, 192, 768, 1024, 1600, 3072, 4096, 6400, 8192, 16384):
                 units = (K + 63) // 64
                 for parts in (ops.k_parts(M, N, K), ops.tiled_k_parts(M, N, K)):
                     assert 1 <= parts <= 16
@@ -39,6 +39,31 @@ def test_attention_split_plan(ops):
                 assert ops.att_parts_takes(n_tokens, splits, 64)
     assert ops.decode_split_plan(1, 12, 256)[0] == 2 and ops.decode_split_plan(1, 12, 1024)[0] == 8
     assert ops.decode_split_plan(16, 12, 1024)[0] == 4
+
+
+def test_attention_plan_of_tokens_that_finish_themselves(ops):
+    """Decode attention that merges its own splits: 1, 4, 8 or 16 splits (two never pay), a split
+    keeping 128 keys or more of the longest context, pairs x splits within 256 workgroups; cut
+    keys go on 4 waves, uncut ones on 4, 8 or 16."""
+    for n_tokens in (1, 2, 4, 8, 9, 17, 32, 64, 300):
+        for n_head in (1, 3, 12, 25, 32):
+            for bucket in (64, 256, 512, 1024, 2048, 4096, 8192, 131072):
+                splits, waves = ops.decode_plan(n_tokens, n_head, bucket)
+                assert splits in (1, 4, 8, 16) and waves in (4, 8, 16)
+                if splits > 1:
+                    assert waves == 4 and bucket // splits >= 128 and n_tokens * n_head * splits <= 256
+    assert ops.decode_plan(1, 32, 1024) == (8, 4) and ops.decode_plan(1, 12, 4096) == (16, 4)
+    assert ops.decode_plan(8, 25, 1024) == (1, 8) and ops.decode_plan(4, 25, 4096) == (1, 16)
+    assert ops.decode_plan(64, 12, 1024) == (1, 4) and ops.decode_plan(1, 12, 256) == (1, 4)
+
+
+def test_tiled_parts_of_one_tile_of_rows(ops):
+    """33 to 64 rows added to the stream: few output features in 4 parts from an inner size of
+    3,072 on; many output features while 64 x 64 tiles x parts stay within 256 workgroups."""
+    assert ops.tiled_k_parts(64, 768, 3072) == 4 and ops.tiled_k_parts(64, 768, 768) == 1
+    assert ops.tiled_k_parts(64, 4096, 16384) == 4 and ops.tiled_k_parts(40, 4096, 4096) == 4
+    assert ops.tiled_k_parts(64, 8192, 8192) == 2 and ops.tiled_k_parts(64, 16384, 4096) == 1
+    assert ops.tiled_k_parts(32, 4096, 16384) == 1
 
 
 def test_what_the_folded_norm_takes(ops):
