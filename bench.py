@@ -207,7 +207,7 @@ def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
     from liyab_amd.engine import StepItem
 
     rng = np.random.default_rng(seed)
-    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in prompt_lens]
+    prompts = [rng.integers(0, cfg["vocab_size"], n) for n in prompt_lens]  # arrays of ids, as the scheduler hands portions over
     best = float("inf")
     for it in range(repeat + 2):
         for i in range(len(prompts)):

