@@ -353,26 +353,54 @@ def test_contexts_of_thousands_of_positions(dtype, tmp_path):
 # ---------------------------------------------------------------------------
 # layers far wider than GPT-2's own
 # ---------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def width_4096_model(tmp_path_factory):
+    """One model folder of width 4,096 for the tests below (writing it takes most of their time)."""
+    from liyab_amd.weights import write_random_model
+
+    d = str(tmp_path_factory.mktemp("width4096"))
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 2, "n_embd": 4096, "n_head": 32, "n_inner": 16384, "vocab_size": 3000,
+           "n_positions": 640, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    write_random_model(d, cfg, 5)
+    return (d,) + tuple(plain.read_model(d))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_layers_of_width_4096(dtype, tmp_path):
+def test_layers_of_width_4096(dtype, width_4096_model):
     """Width 4,096, 32 heads of 128, a feed-forward of 16,384: inner dimensions past what the
     kernel with the norm folded in takes (2,048), more output features than the streaming
     kernels take (8,192), heads of 128. Whole, most in one step with a tail token by token,
     and mixed, against the plain implementation."""
     from liyab_amd.engine import EngineCore
-    from liyab_amd.weights import write_random_model
 
-    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 2, "n_embd": 4096, "n_head": 32, "n_inner": 16384, "vocab_size": 3000,
-           "n_positions": 200, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
-    write_random_model(str(tmp_path), cfg, 5)
-    config, tensors = plain.read_model(str(tmp_path))
+    d, config, tensors = width_4096_model
     weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
     reqs = {f"w{i}": tt.random_tokens(40 + i, n, 3000) for i, n in enumerate([200, 37, 3, 90])}
     refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
     for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=3, decode_tail=6)),
                          ("bulk+tail", tt.schedule_bulk_tail(reqs, tail=8))):
-        core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        core = EngineCore(d, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
         got = tt.run_schedule(core, steps)
         tt.check_against_plain(got, reqs, refs, TOL[dtype], f"width 4,096 {label} {dtype}", family="sizes:wide")
         core.manager.check()
         del core
+
+
+def test_few_heads_over_many_keys_finish_their_own_splits(width_4096_model):
+    """One request of 600 positions at 32 heads of 128, its tail token by token: the projection
+    of this width is not cut over its inner dimension, so nobody merges attention's splits for
+    it, and with 32 (token, head) pairs the step cuts the keys into 8 splits and merges them
+    itself (ops.decode_plan)."""
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.kernels import ops
+
+    d, config, tensors = width_4096_model
+    assert ops.decode_plan(1, 32, 1024) == (8, 4) and ops.k_parts(1, 4096, 4096) == 1
+    weights = plain.round_weights_to_bf16(tensors)
+    reqs = {"deep": tt.random_tokens(77, 600, 3000)}
+    refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+    steps = tt.schedule_bulk_tail(reqs, tail=12)
+    core = EngineCore(d, dtype="bfloat16", page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=2)
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, refs, TOL["bfloat16"], "width 4,096, 600 positions, tail token by token", family="sizes:wide")
+    core.manager.check()
