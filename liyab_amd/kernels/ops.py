@@ -722,8 +722,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, tile=17 if small else 16)
         elif M <= 16 or (M <= 64 and N <= 8192):
             # few tokens: stream the weights (for a huge N and more than 16 tokens the tiled
-            # kernel's shared loads beat every workgroup re-reading the tokens)
-            gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=0)
+            # kernel's shared loads beat every workgroup re-reading the tokens); 11 to 16 tokens and
+            # very many output features in strips of 64, which read the tokens a quarter as often (16
+            # rows, alone: 4,096 -> 16,384 31.6 against 36.4 us, -> 12,288 25.3 against 28.5; at 8 rows
+            # and at 6,400 features strips of 16 win)
+            gemm_skinny(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv, wide=1 if 10 < M <= 16 and N >= 12288 else 0)
         elif a.shape[1] % 64 == 0:
             gemm_mfma_dl(a, w, bias, out=out, residual=residual, epilogue=epilogue, kv=kv)
         else:
