@@ -574,8 +574,8 @@ def skinny_parts_takes(M: int, N: int, K: int) -> bool:
 
 
 def tiled_k_parts(M: int, N: int, K: int) -> int:
-    """Into how many parts of K the tiled product of more than 32 rows is best cut when it is
-    added to the residual stream (1: not at all). Several tiles of rows, few output features and
+    """Into how many parts of K the tiled product of more than 32 rows (of more than 16, with many
+    output features) is best cut when it is added to the residual stream (1: not at all). Several tiles of rows, few output features and
     a long K (a prompt's portion through the feed-forward's second product: 128 x 768 x 3,072 is
     24 tiles of 64 x 64, each walking the whole of K in 18.7 us): cut until the tiles cover the
     chip. One tile of rows (33 to 64): the 64 x 32 tiles are few and each walks the whole of K;
@@ -583,16 +583,19 @@ def tiled_k_parts(M: int, N: int, K: int) -> int:
     1,600 19.8 and 8.2. In a decode step the next readers pay for the planes, though: inner
     dimensions from 3,072 gain, in 4 parts (ms a step at 64 rows, whole and cut: GPT-2 small's
     sizes 0.806 and 0.797, medium's 1.767 and 1.715; XL's 5.19 and 4.90)."""
-    if K % 64 != 0 or M <= 32 or _invariant:
+    if K % 64 != 0 or M <= 16 or _invariant:
         return 1
     if M <= 64:
         if N <= 2048:
-            return 4 if K >= 3072 else 1
-        # more output features: tiles of 64 x 64 (every tile reads all the rows: 32 x 32 tiles read
-        # them twice as often as the weights), cut while tiles x parts stay within the chip (us at 64
-        # rows, alone: 16,384 -> 4,096 42.2 whole in 32 x 32 tiles, 32.3 in 64 x 64 and 4 parts; 4,096
-        # -> 4,096 13.5 and 9.7; 8,192 -> 8,192 34.8 and 31.6 in 2 parts)
-        tiles, parts = (N + 63) // 64, 1
+            return 4 if K >= 3072 and M > 32 else 1
+        # more output features: the largest tiles that take the rows in one, 32 x 32 up to 32 rows and
+        # 64 x 64 beyond (every tile reads all the rows: at 64 rows, 32 x 32 tiles read them twice as
+        # often as the weights), cut while tiles x parts stay within the chip (us alone, whole as it
+        # was and cut: 64 rows, 16,384 -> 4,096 42.2 and 32.3 in 4 parts, 4,096 -> 4,096 13.5 and 9.7,
+        # 8,192 -> 8,192 34.8 and 31.6 in 2 parts; 32 rows, 16,384 -> 4,096 39.7 and 27.8 in 2 parts,
+        # 4,096 -> 4,096 12.3 and 9.6, 8,192 -> 8,192 27.3 whole)
+        side = 32 if M <= 32 else 64
+        tiles, parts = (N + side - 1) // side, 1
         while parts < 4 and tiles * parts * 2 <= 256 and K // 64 // (parts * 2) >= 8:  # (256: the compute units of the part this was measured on)
             parts *= 2
         return parts

@@ -98,8 +98,11 @@ def linear_deferred(a, w: torch.Tensor, bias: Optional[torch.Tensor], ctx, name:
         # 3,072 -> 768 in four parts: 6.5 against 7.5 us in 64 x 64 tiles), 64 x 64 tiles beyond
         few = (M + 63) // 64 * ((w.shape[0] + 31) // 32) * parts <= ops.compute_units()
         fewer = (M + 31) // 32 * ((w.shape[0] + 31) // 32) * parts <= ops.compute_units()  # 32 x 32 tiles each on a compute unit of its own
-        many = M <= 64 and w.shape[0] > 2048  # one tile of rows, many output features: 64 x 64 (ops.tiled_k_parts)
-        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=6 if many else (17 if fewer else (16 if M <= 64 or few else 6)))
+        if M <= 64 and w.shape[0] > 2048:  # one tile of rows, many output features: the largest tile that takes the rows (ops.tiled_k_parts)
+            tile = 17 if M <= 32 else 6
+        else:
+            tile = 17 if fewer else (16 if M <= 64 or few else 6)
+        ops.gemm_mfma_dl_parts(a, w, planes, bias=bias, base=base, tile=tile)
     else:
         ops.gemm_skinny_parts(a, w, planes, bias=bias, base=base)
     return SplitStream(planes, stream.home if split else stream)

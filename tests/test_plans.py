@@ -24,7 +24,7 @@ def test_parts_of_k_are_whole_and_none_is_empty(ops):
                 if ops.k_parts(M, N, K) > 1:
                     assert M <= 32 and K % 8 == 0
                 if ops.tiled_k_parts(M, N, K) > 1:
-                    assert M > 32 and K % 64 == 0
+                    assert M > 16 and (M > 32 or N > 2048) and K % 64 == 0
 
 
 def test_attention_split_plan(ops):
@@ -63,7 +63,8 @@ def test_tiled_parts_of_one_tile_of_rows(ops):
     assert ops.tiled_k_parts(64, 768, 3072) == 4 and ops.tiled_k_parts(64, 768, 768) == 1
     assert ops.tiled_k_parts(64, 4096, 16384) == 4 and ops.tiled_k_parts(40, 4096, 4096) == 4
     assert ops.tiled_k_parts(64, 8192, 8192) == 2 and ops.tiled_k_parts(64, 16384, 4096) == 1
-    assert ops.tiled_k_parts(32, 4096, 16384) == 1
+    assert ops.tiled_k_parts(32, 4096, 16384) == 2 and ops.tiled_k_parts(17, 4096, 4096) == 2 and ops.tiled_k_parts(24, 8192, 8192) == 1
+    assert ops.tiled_k_parts(16, 4096, 16384) == 1 and ops.tiled_k_parts(32, 768, 3072) == 1
 
 
 def test_what_the_folded_norm_takes(ops):
