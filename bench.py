@@ -85,7 +85,9 @@ def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
     engine.stop_at_eos = False
     for i in range(batch):
         prompt = rng.integers(0, cfg["vocab_size"], prompt_len).tolist()
-        engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1), rid=f"b{batch}-{i}")
+        # (requests that go on for some steps past the timed ones: a request about to reach its last
+        # token is waited for, not run ahead of, and that wait is no part of a decode step)
+        engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8), rid=f"b{batch}-{i}")
     while any(r.remaining > 1 or not r.generated for r in engine.scheduler.running) or engine.scheduler.waiting:
         engine.step()  # prompts, until every request is decoding
     for _ in range(warmup):
