@@ -62,6 +62,15 @@ struct PartsParams {
 // 8 different pieces: the piece index is XORed with (row / 2) % 8.
 __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 
+// Dynamic LDS of a workgroup: the operand stages, or, where bfloat16 outputs leave through LDS as whole
+// rows, the waves' padded output tiles if those take more (tiles of 256 x 256: 144 KB against 128).
+template <int BM, int BN, int DSTAGES, int WM, int WN, int WK>
+constexpr size_t dl_lds_bytes(size_t out_bytes) {
+    const size_t stages = static_cast<size_t>(DSTAGES) * WK * (BM + BN) * 64 * 2;
+    const size_t staging = out_bytes == 2 ? static_cast<size_t>(WM * WN * WK) * (BM / WM) * (BN / WN + 8) * 2 : 0;
+    return stages > staging ? stages : staging;
+}
+
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1, int SETS = 1>
 __global__ void __launch_bounds__(64 * WM * WN * WK)
 gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int M, int N, int K,
@@ -257,7 +266,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
         // cache lines, where the accumulators' own layout would write 16 bytes of 32 different
         // rows with every instruction (measured: 5.7 of 19.7 us on a 2,048 x 2,304 product).
         constexpr int RM = BM / WM, CN = BN / WN, LDO = CN + 8;  // padded rows, 16-byte aligned
-        static_assert(WAVES * RM * LDO <= DSTAGES * STAGE, "the output staging must fit the operand stages");
+        static_assert(WAVES * RM * LDO * 2 <= dl_lds_bytes<BM, BN, DSTAGES, WM, WN, WK>(2), "the output staging must fit the dynamic LDS the launcher asks for");
         if (columns_inside && vec_ok > 1) {
             lds_barrier();  // everyone is done reading the last operand stage
             bf16_t* tile = lds + wave * RM * LDO;
@@ -415,7 +424,8 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
 template <int BM, int BN, int DSTAGES, typename OutT, int EPI, int WM = 2, int WN = 2, int WK = 1, int SETS = 1>
 int launch_dl_as(const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
     const int grid = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
-    const size_t smem = static_cast<size_t>(DSTAGES) * WK * (BM + BN) * DBK * sizeof(bf16_t);
+    constexpr size_t smem = dl_lds_bytes<BM, BN, DSTAGES, WM, WN, WK>(sizeof(OutT));
+    static_assert(smem <= 160 * 1024, "a workgroup's LDS");
     auto kern = gemm_mfma_dl_kernel<BM, BN, DSTAGES, OutT, EPI, WM, WN, WK, SETS>;
     static bool ready = false;  // once per instantiation, outside any stream capture's first use
     if (!ready) {
@@ -495,6 +505,24 @@ using namespace liyab;
 // its own chain of load, barrier, fragments and products, not on the loads in flight); 0 = chosen from
 // the shape. (Measured and dropped: 128x128 on four waves, 128x64, 128x192, and deeper rings under
 // 128x128, whose LDS leaves one workgroup a compute unit, so that 288 tiles take two rounds.)
+// The epilogues that tiles of 256 x 256 are compiled with: into the residual stream, plain 32-bit
+// outputs, and bfloat16 outputs plain, through the tanh GELU or into the cache's pages.
+static bool dl_takes_256(const EpiParams& epi) {
+    if (epi.mode == kEpiResidual) return true;
+    if (epi.out_dtype == kF32) return epi.mode == kEpiNone;
+    return epi.mode == kEpiNone || epi.mode == kEpiGeluTanh || epi.mode == kEpiQkvPaged;
+}
+
+static int launch_dl_256(const void* a, int64_t lda, const void* w, int M, int N, int K, const EpiParams& epi, hipStream_t stream) {
+    auto* pa = static_cast<const bf16_t*>(a);
+    auto* pw = static_cast<const bf16_t*>(w);
+    if (epi.mode == kEpiResidual) return launch_dl_as<256, 256, 2, float, kEpiResidual, 2, 4>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.out_dtype == kF32) return launch_dl_as<256, 256, 2, float, kEpiNone, 2, 4>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.mode == kEpiGeluTanh) return launch_dl_as<256, 256, 2, bf16_t, kEpiGeluTanh, 2, 4>(pa, lda, pw, M, N, K, epi, stream);
+    if (epi.mode == kEpiQkvPaged) return launch_dl_as<256, 256, 2, bf16_t, kEpiQkvPaged, 2, 4>(pa, lda, pw, M, N, K, epi, stream);
+    return launch_dl_as<256, 256, 2, bf16_t, kEpiNone, 2, 4>(pa, lda, pw, M, N, K, epi, stream);
+}
+
 extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int M, int N, int K, int tile,
                                   const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(a && w && epi_in, "gemm: null operand");
@@ -513,14 +541,26 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
     // tiles of 64 x 64), a somewhat smaller one with a long K too (2,048 x 1,600 x 6,400: 79 against 88 us); the
     // fourth stage pays while the tiles of 64 x 64 are few enough for its LDS (4,096 x 768 x 3,072, 768 tiles:
     // 36 us with three stages, 49 with four).
+    // Tiles of 256 x 256 (half the operand bytes a product of 128 x 128 tiles brings in from L2, which is
+    // what bounds those) where they cover most of the chip: 0.9-1.09 PFLOP/s against 0.76-0.84 at widths
+    // of 4,096 to 16,384 (4,096 x 4,096 x 16,384: 507 against 721 us), and from 2,048 x 6,400 x 1,600 on
+    // (66 against 77 us); a short K pays its fill and its epilogue more often (8,192 x 3,072 x 768: 83
+    // against 80 us, 16,384 rows: 130 against 150).
     if (tile == 0) {
         const long out = static_cast<long>(M) * N, tiles64 = static_cast<long>((M + 63) / 64) * ((N + 63) / 64);
-        tile = (out >= 2048L * 2048L || (out >= 2560L * 1024L && K >= 4096)) ? 8 : ((K >= 2048 && tiles64 < 640) ? 6 : 2);
+        const long tiles256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
+        if (tiles256 >= 200 && (K >= 1536 || tiles256 >= 768) && dl_takes_256(epi)) tile = 15;
+        else tile = (out >= 2048L * 2048L || (out >= 2560L * 1024L && K >= 4096)) ? 8 : ((K >= 2048 && tiles64 < 640) ? 6 : 2);
     }
     switch (tile) {
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
         case 6: return launch_dl<64, 64, 4>(a, lda, w, M, N, K, epi, stream);
         case 8: return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
+        case 15:
+            // 256 x 256 on eight waves of 128 x 64: with the epilogues that are compiled in (the others
+            // would spill its 128 accumulation registers a lane) and tiles of 128 x 128 otherwise
+            if (dl_takes_256(epi)) return launch_dl_256(a, lda, w, M, N, K, epi, stream);
+            return launch_dl<128, 128, 2, 4, 2>(a, lda, w, M, N, K, epi, stream);
         case 16: return launch_dl<64, 32, 3, 2, 1, 4>(a, lda, w, M, N, K, epi, stream);
         case 17: return launch_dl<32, 32, 3, 1, 1, 4>(a, lda, w, M, N, K, epi, stream);
         // 102, 106, 108: the tiles of 2, 6 and 8 with four sums by unit of K, whose results are those of 16 and 17 bit for bit

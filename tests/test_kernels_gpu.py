@@ -224,10 +224,10 @@ def test_gemm_float32(ops, M, N, K, epilogue):
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
-                                    "dl2", "dl6", "dl8", "dl16", "dl17"])
+                                    "dl2", "dl6", "dl8", "dl15", "dl16", "dl17"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
-                                                 (500, 300, 128), (129, 193, 192), (20, 4800, 1600)])
+                                                 (500, 300, 128), (129, 193, 192), (20, 4800, 1600), (600, 520, 256), (1030, 770, 128)])
 def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
     a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
     tiles = {"mfma128": 1, "mfma64": 2, "mfma128x64": 3}
@@ -785,8 +785,8 @@ def test_tiles_of_every_shape_give_a_row_the_same_bits(ops, K):
             assert torch.equal(out, full[108][rows]), f"rows {rows} in tiles {tile}"
 
 
-@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "dl16", "auto"])
-@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64)])
+@pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "dl15", "dl16", "auto"])
+@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64), (700, 6, 3, 64, 128, 16)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
     """Queries to a dense buffer, keys and values straight into shuffled cache slots, against
     the plain product followed by the scatter kernel."""
