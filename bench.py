@@ -5,6 +5,7 @@
     python bench.py --prefill-tokens 512,2048,8192   # prefill tokens a second per length
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
     python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
+    python bench.py --product 4096,4096,16384,8,15   # one product in tiles of 128 x 128 and of 256 x 256
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -142,6 +143,35 @@ def workload_run(engine, cfg, prompts, params_of, label):
             "generated": generated, "prompt_tokens": prompt_tokens,
             "preemptions": sum(r.stats.preemptions for r in results),
             "roofline_frac": round(bytes_read / dt / 1e9 / HBM_PEAK_GBS, 4)}, [r.tokens for r in results]
+
+
+def product_run(M, N, K, tiles, device="cuda:0", reps=30):
+    """One product a[M, K] . w[N, K]^T + bias in bfloat16 (outputs bfloat16), as the tiled matrix-core
+    kernel runs it in the tiles named (0: the kernel's own choice; 2 and 6: 64 x 64, 8: 128 x 128,
+    15: 256 x 256): microseconds and TFLOP/s each."""
+    import torch
+
+    from liyab_amd.kernels import ops
+
+    dev = torch.device(device)
+    a = torch.randn(M, K, device=dev).bfloat16()
+    w = (torch.randn(N, K, device=dev) * 0.02).bfloat16()
+    bias = torch.randn(N, device=dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    runs = []
+    for tile in tiles:
+        for _ in range(3):
+            ops.gemm_mfma_dl(a, w, bias, out=out, tile=tile)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            ops.gemm_mfma_dl(a, w, bias, out=out, tile=tile)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        runs.append({"tile": tile, "us": round(us, 1), "tflops": round(2.0 * M * N * K / us / 1e6, 1)})
+    return {"metric": "one product, bfloat16", "M": M, "N": N, "K": K, "runs": runs}
 
 
 def link_floor(device="cuda:0", links=100):
@@ -285,6 +315,7 @@ def main():
                          "tokens each; xl64: GPT-2 XL's sizes, 64 requests with prompts of 256 tokens decoding to 1,024, greedy and at temperature 1")
     ap.add_argument("--page-size", type=int, default=64, help="positions a cache page (default 64; the engine's own default is 16)")
     ap.add_argument("--batch-invariant", action="store_true", help="kernels chosen from sizes and positions only (reproducible bfloat16 replies)")
+    ap.add_argument("--product", default="", help="M,N,K[,tile,...]: time one bfloat16 product in the tiled kernel's tiles (0: its own choice, 6: 64 x 64, 8: 128 x 128, 15: 256 x 256)")
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -294,6 +325,10 @@ def main():
 
     from liyab_amd.weights import write_random_model
 
+    if args.product:
+        sizes = [int(x) for x in args.product.split(",")]
+        print(json.dumps(product_run(sizes[0], sizes[1], sizes[2], sizes[3:] or [0])))
+        return 0
     if args.link_floor:
         print(json.dumps(link_floor()))
         return 0

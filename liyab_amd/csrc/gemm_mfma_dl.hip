@@ -96,11 +96,27 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
     // Workgroups go to the 8 XCDs round-robin, each XCD with an L2 of its own. Tile t of the
     // row-major tile order goes to the XCD that holds the tiles around it, so that an XCD's
     // tiles share a few row blocks of `a` and its L2 holds them beside all of `w`.
-    const int tiles_n = (N + BN - 1) / BN, n_tiles = tiles_n * ((M + BM - 1) / BM);
+    // An XCD takes a stretch of the row-major tile order: a band of rows. While `w` is small that is
+    // the best order: the XCD reads `w` once, and its rows of `a` are what its own workgroups of the
+    // product before wrote (a prefill step's products all run over the same bands of tokens, so an
+    // XCD's activations stay in its L2). With a large `w` the workgroups that run side by side on an
+    // XCD, one row of tiles and all of `w`'s columns, share nothing of `w`, and every row of tiles
+    // reads all of it again from memory (4,096 x 4,096 x 16,384 in 128 x 128 tiles: 3.9 GB of L2
+    // misses for 0.27 GB of operands, at the memory's own speed): there the XCD's stretch goes in
+    // groups of GM rows of tiles, down the rows first, so that its workgroups form a block of GM
+    // rows by a few columns (half the misses; 721 -> 611 us). The bound between the two, 12 MB of
+    // `w`: GPT-2 small's prefill of 2,048 tokens is 6 % slower in groups (its second feed-forward
+    // product 24.2 -> 28.9 us), XL's of 8,192 tokens 6 % faster, width 4,096's 6 %.
+    const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM, n_tiles = tiles_n * tiles_m;
     const int xcd = blockIdx.x % 8, base = n_tiles / 8, rem = n_tiles % 8;
     const int tile_id = xcd * base + min(xcd, rem) + blockIdx.x / 8;
-    int m0 = (tile_id / tiles_n) * BM;
-    const int n0 = (tile_id % tiles_n) * BN;
+    constexpr int GM = BM >= 128 ? 4 : 8;
+    const bool groups = static_cast<int64_t>(N) * K > (6 << 20);
+    const int per_group = groups ? GM * tiles_n : tiles_n;  // (plain rows: groups of one row of tiles)
+    const int group = tile_id / per_group, first_m = group * (groups ? GM : 1), in_group = tile_id - group * per_group;
+    const int gm = groups ? min(GM, tiles_m - first_m) : 1;
+    int m0 = (first_m + in_group % gm) * BM;
+    const int n0 = (in_group / gm) * BN;
     const int li = lane % 32, g = lane / 32;
 
     // this lane's part in a wave-load: row lane / 8 of the 8, LDS piece position lane % 8
@@ -541,16 +557,19 @@ extern "C" int liyab_gemm_mfma_dl(const void* a, int64_t lda, const void* w, int
     // tiles of 64 x 64), a somewhat smaller one with a long K too (2,048 x 1,600 x 6,400: 79 against 88 us); the
     // fourth stage pays while the tiles of 64 x 64 are few enough for its LDS (4,096 x 768 x 3,072, 768 tiles:
     // 36 us with three stages, 49 with four).
-    // Tiles of 256 x 256 (half the operand bytes a product of 128 x 128 tiles brings in from L2, which is
-    // what bounds those) where they cover most of the chip: 0.9-1.09 PFLOP/s against 0.76-0.84 at widths
-    // of 4,096 to 16,384 (4,096 x 4,096 x 16,384: 507 against 721 us), and from 2,048 x 6,400 x 1,600 on
-    // (66 against 77 us); a short K pays its fill and its epilogue more often (8,192 x 3,072 x 768: 83
-    // against 80 us, 16,384 rows: 130 against 150).
+    // Tiles of 256 x 256 (half the operand bytes a product of 128 x 128 tiles brings in from L2) where
+    // K is long and they fill whole rounds over the chip's 256 compute units, one a unit: 0.93-1.1
+    // PFLOP/s against 0.8-0.95 at widths of 4,096 to 16,384 (4,096 x 4,096 x 16,384: 502 against 611
+    // us); with 384 tiles (a round and a half), or a K of 1,600 and more than one round (8,192 x 6,400 x
+    // 1,600: 289 against 248 us), the 128 x 128 tiles, two a unit, win. (Alone and added to the residual
+    // stream, 2,048 x 2,304 x 768 runs 19.8 us in 64 x 64 tiles and 23.4 in 128 x 128; in a prefill
+    // step, writing keys and values into their pages or through the GELU, the large tiles win.)
     if (tile == 0) {
         const long out = static_cast<long>(M) * N, tiles64 = static_cast<long>((M + 63) / 64) * ((N + 63) / 64);
-        const long tiles256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
-        if (tiles256 >= 200 && (K >= 1536 || tiles256 >= 768) && dl_takes_256(epi)) tile = 15;
-        else tile = (out >= 2048L * 2048L || (out >= 2560L * 1024L && K >= 4096)) ? 8 : ((K >= 2048 && tiles64 < 640) ? 6 : 2);
+        const long tiles256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256), rounds = (tiles256 + 255) / 256;
+        if ((K >= 2048 || (K >= 1536 && rounds == 1)) && tiles256 >= 200 && tiles256 * 100 >= rounds * 256 * 78 && dl_takes_256(epi)) tile = 15;
+        else if (out >= 2048L * 2048L || (out >= 2560L * 1024L && K >= 4096)) tile = 8;
+        else tile = (K >= 2048 && tiles64 < 640) ? 6 : 2;
     }
     switch (tile) {
         case 2: return launch_dl<64, 64, 3>(a, lda, w, M, N, K, epi, stream);
