@@ -600,11 +600,13 @@ def tiled_k_parts(M: int, N: int, K: int) -> int:
             parts *= 2
         return parts
     # several tiles of rows (a prompt's portion): 64 x 64 tiles, cut until they cover the chip,
-    # a part keeping 256 of K or more
+    # a part keeping 256 of K or more; in two parts while two workgroups a compute unit hold them
+    # (ms a step of 768 / 1,024 tokens whole and in two parts: GPT-2 small's sizes 1.00 and 0.99 /
+    # 1.13 and 1.12, medium's 2.32 and 2.16 / 2.54 and 2.47; XL's at 512 tokens 6.11 and 5.88)
     tiles = (M + 63) // 64 * ((N + 63) // 64)
     nk = K // 64
     parts = 1
-    while parts < TILED_MAX_PARTS and tiles * parts * 2 <= 256 and nk // (parts * 2) >= 4:
+    while parts < TILED_MAX_PARTS and tiles * parts * 2 <= (512 if parts == 1 else 256) and nk // (parts * 2) >= 4:
         parts *= 2
     return parts
 
