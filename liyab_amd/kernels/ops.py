@@ -869,7 +869,11 @@ def decode_split_plan(n_tokens: int, n_head: int, context_bucket: int):
     splits = 1
     while splits < most and context_bucket // (2 * splits) >= 128:
         splits *= 2
-    return splits, 4
+    # very long contexts of one or two requests: 8 splits of 4 waves leave most of the chip idle and
+    # each walks thousands of keys; 16 waves a split walk them four times as fast (us, 12 pairs of 64
+    # at 8,000 / 16,000 / 30,000 keys: 14.5 / 25.1 / 41.2 on 4 waves, 11.7 / 17.0 / 23.6 on 16; from
+    # 48 pairs on 4 waves win)
+    return splits, (16 if pairs <= 32 and context_bucket // splits >= 1024 else 4)
 
 
 # pairs up to which 4 and 2 splits are taken (beyond 16 tokens splits lost: us a step at batch 17 / 24 / 32

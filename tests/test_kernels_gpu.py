@@ -495,10 +495,11 @@ def test_attention_splits_by_position(ops, case_id, dtype, window):
         assert torch.equal(out[rows], outs[0][rows]), f"request {s_} alone"
 
 
+@pytest.mark.parametrize("waves", [4, 16])
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("splits", [2, 4, 7, 8])
 @pytest.mark.parametrize("case_id", [0, 1, 2, 3, 5, 6, 7])
-def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window):
+def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window, waves):
     """Attention that leaves each (token, head) pair's keys in splits, and the projection cut
     over its inner dimension that merges them as it loads them: the planes add up to rows +
     attention . W^T + bias; the merge kernel gives attention's output from the same splits.
@@ -514,7 +515,7 @@ def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window)
     partials = torch.full((n, H, splits, hd + 4), float("nan"), device=DEV)
     untouched = torch.full((n, H * hd), 7.0, dtype=torch.bfloat16, device=DEV)
     ops.attention_decode(untouched, q[:, :H * hd], kc, vc, bt, tok_seq, tok_pos, n_head=H, scale=scale, window=window,
-                         n_splits=splits, partials=partials, waves=4, leave_splits=True)
+                         n_splits=splits, partials=partials, waves=waves, leave_splits=True)
     assert (untouched == 7.0).all()
     want = attention_reference(case, H, Hkv, hd, scale, window)
     merged = torch.empty(n, H * hd, dtype=torch.bfloat16, device=DEV)

@@ -32,13 +32,15 @@ def test_attention_split_plan(ops):
     longest context, workgroups of 4 waves; one split when the context is short."""
     for n_tokens in (1, 2, 8, 9, 16, 17, 32):
         for n_head in (1, 3, 12, 25):
-            for bucket in (256, 512, 1024, 2048, 8192):
+            for bucket in (256, 512, 1024, 2048, 8192, 32768):
                 splits, waves = ops.decode_split_plan(n_tokens, n_head, bucket)
-                assert splits in (1, 2, 4, 8) and waves == 4
+                assert splits in (1, 2, 4, 8) and waves in (4, 16)
+                assert waves == 4 or (n_tokens * n_head <= 32 and bucket // splits >= 1024)
                 assert splits == 1 or bucket // splits >= 128
                 assert ops.att_parts_takes(n_tokens, splits, 64)
     assert ops.decode_split_plan(1, 12, 256)[0] == 2 and ops.decode_split_plan(1, 12, 1024)[0] == 8
     assert ops.decode_split_plan(16, 12, 1024)[0] == 4
+    assert ops.decode_split_plan(1, 12, 32768) == (8, 16) and ops.decode_split_plan(8, 12, 32768) == (8, 4)
 
 
 def test_attention_plan_of_tokens_that_finish_themselves(ops):
