@@ -53,7 +53,7 @@ def test_attention_plan_of_tokens_that_finish_themselves(ops):
                 splits, waves = ops.decode_plan(n_tokens, n_head, bucket)
                 assert splits in (1, 4, 8, 16) and waves in (4, 8, 16)
                 if splits > 1:
-                    assert waves == 4 and bucket // splits >= 128 and n_tokens * n_head * splits <= 256
+                    assert waves == (8 if bucket // splits >= 1024 else 4) and bucket // splits >= 128 and n_tokens * n_head * splits <= 256
     assert ops.decode_plan(1, 32, 1024) == (8, 4) and ops.decode_plan(1, 12, 4096) == (16, 4)
     assert ops.decode_plan(8, 25, 1024) == (1, 8) and ops.decode_plan(4, 25, 4096) == (1, 16)
     assert ops.decode_plan(64, 12, 1024) == (1, 4) and ops.decode_plan(1, 12, 256) == (1, 4)
