@@ -227,7 +227,7 @@ def test_gemm_float32(ops, M, N, K, epilogue):
                                     "dl2", "dl6", "dl8", "dl15", "dl16", "dl17"])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(300, 264, 1600), (2, 50257 // 16, 64), (8, 130, 3072), (16, 2304, 768), (3, 40, 200), (17, 100, 64), (40, 333, 768), (64, 257, 1600),
-                                                 (500, 300, 128), (129, 193, 192), (20, 4800, 1600), (600, 520, 256), (1030, 770, 128)])
+                                                 (500, 300, 128), (129, 193, 192), (20, 4800, 1600), (600, 520, 256), (1030, 770, 128), (5, 100, 16384)])
 def test_gemm_bfloat16(ops, M, N, K, epilogue, kernel):
     a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
     tiles = {"mfma128": 1, "mfma64": 2, "mfma128x64": 3}
