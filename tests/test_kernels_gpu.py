@@ -544,6 +544,32 @@ def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window,
             assert torch.equal(planes, two)
 
 
+def test_projection_over_splits_with_rows_32_kb_apart(ops):
+    """Heads x head size = 16,384: the weights' rows lie 32 KB apart, where the streaming kernels
+    walk K in blocks from a place of each workgroup's own; the kernel that merges attention's
+    splits as it loads them must still give the bits of the merge followed by the plain product."""
+    M, H, S, hd, N = 3, 128, 2, 128, 40
+    g = torch.Generator().manual_seed(3)
+    partials = torch.randn(M, H, S, hd + 4, generator=g)
+    partials[..., hd] = torch.randn(M, H, S, generator=g) * 2  # the splits' maxima
+    partials[..., hd + 1] = torch.rand(M, H, S, generator=g) * 50 + 1  # and sums
+    partials = partials.to(DEV)
+    merged = torch.empty(M, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_merge(merged, partials)
+    w, bias = rnd(N, H * hd, seed=1, scale=0.05, dtype=torch.bfloat16), rnd(N, seed=2)
+    base = rnd(M, N, seed=8, scale=3.0)
+    with pytest.raises(Exception, match="do not fit LDS"):  # whole rows of 16,384 are refused, not mangled
+        ops.gemm_att_parts(partials, w, torch.empty(1, M, N, device=DEV), bias=bias, base=base)
+    for parts in (2, 4):
+        planes = torch.full((parts, M, N), float("nan"), device=DEV)
+        ops.gemm_att_parts(partials, w, planes, bias=bias, base=base)
+        want = merged.double() @ w.double().t() + bias.double() + base.double()
+        close(planes.double().sum(0), want, 1e-5, f"projection over splits at K = 16,384, {parts} parts")
+        two = torch.empty_like(planes)
+        ops.gemm_skinny_parts(merged, w, two, bias=bias, base=base, ksplit=8)
+        assert torch.equal(planes, two)
+
+
 PREFILL_CASES = [
     # ctx_lens, q_lens, H, Hkv, hd, page
     ([1, 17, 300], [1, 17, 300], 4, 4, 16, 16),
