@@ -160,7 +160,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __re
     };
     // every trip but the last asks for the next trip's operands before it multiplies; the last
     // one is peeled off, so no trip asks for (and then waits for) operands nobody uses
-    for (int left = trips - 1; left > 0; --left) {
+    // (dealt trip by trip, a wave whose unit of the last trip lies past the end of K stops a trip
+    // early: it would ask for the rows' last bytes again, as every such wave would, and drop them)
+    const int my_trips = blocks ? trips : max(1, (units - wave * UPT + UPT * ksplit - 1) / (UPT * ksplit));
+    for (int left = my_trips - 1; left > 0; --left) {
         trip = trip + 1 == trips ? 0 : trip + 1;
         Frag wn[UPT][NT][2], xn[UPT][MT][2];
         load_w(unit_of(trip), wn);

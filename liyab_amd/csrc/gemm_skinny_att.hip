@@ -174,7 +174,8 @@ gemm_att_parts_kernel(Splits att, const bf16_t* __restrict__ w, int M, int N, in
             }
         }
     };
-    for (int left = trips - 1; left > 0; --left) {
+    const int my_trips = blocks ? trips : max(1, (units - wave * 2 + 2 * WAVES - 1) / (2 * WAVES));  // (as gemm_skinny_kernel stops a wave early)
+    for (int left = my_trips - 1; left > 0; --left) {
         const int u0 = unit_of(trip);
         trip = trip + 1 == trips ? 0 : trip + 1;
         Frag wn[2][2];
