@@ -575,8 +575,8 @@ def skinny_parts_takes(M: int, N: int, K: int) -> bool:
 
 def tiled_k_parts(M: int, N: int, K: int) -> int:
     """Into how many parts of K the tiled product of more than 32 rows (of more than 16, with many
-    output features) is best cut when it is added to the residual stream (1: not at all). Several tiles of rows, few output features and
-    a long K (a prompt's portion through the feed-forward's second product: 128 x 768 x 3,072 is
+    output features) is best cut when it is added to the residual stream (1: not at all).
+    Several tiles of rows, few output features and a long K (a prompt's portion through the feed-forward's second product: 128 x 768 x 3,072 is
     24 tiles of 64 x 64, each walking the whole of K in 18.7 us): cut until the tiles cover the
     chip. One tile of rows (33 to 64): the 64 x 32 tiles are few and each walks the whole of K;
     cut over K they cover the chip: alone, at 64 rows, 3,072 -> 768 takes 8.2 us whole (the streaming kernel) and 4.9 in 8 parts, 6,400 ->
