@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|xl] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--size small|medium|large|xl|wide] [--layers L]
     python bench.py --sequences 1,2,4,8 [-n 128]     # together against in turns, and whether replies are the same
     python bench.py --prefill-tokens 512,2048,8192   # prefill tokens a second per length
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
@@ -41,8 +41,9 @@ SMALL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 
 # GPT-2's other sizes, for --size: the layer sizes and, with them, the number of layers
 # ("wide": no GPT-2 of anybody's, but the architecture at layer sizes where a decode step is bound by the weights' bytes, not by
 # its chain of kernels: 403 MB of matrices a layer; run it with --layers 8 or so)
-WEIGHT_SEEDS = {"small": 10, "medium": 20, "xl": 30, "wide": 40}
+WEIGHT_SEEDS = {"small": 10, "medium": 20, "large": 25, "xl": 30, "wide": 40}
 SIZES = {"small": {}, "medium": {"n_layer": 24, "n_embd": 1024, "n_head": 16, "n_inner": 4096},
+         "large": {"n_layer": 36, "n_embd": 1280, "n_head": 20, "n_inner": 5120},
          "xl": {"n_layer": 48, "n_embd": 1600, "n_head": 25, "n_inner": 6400},
          "wide": {"n_layer": 32, "n_embd": 4096, "n_head": 32, "n_inner": 16384}}
 
@@ -298,7 +299,7 @@ def main():
     ap.add_argument("--steps", type=int, default=504)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--size", default="small", choices=sorted(SIZES), help="GPT-2 small's sizes (the default), medium's or XL's; or layers of width 4,096")
+    ap.add_argument("--size", default="small", choices=sorted(SIZES), help="GPT-2 small's sizes (the default), medium's, large's or XL's; or layers of width 4,096")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has, if needed")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt", type=int, default=512)

@@ -306,6 +306,11 @@ SIZES = {
     # GPT-2 XL's layer sizes (width 1600, 25 heads, feed-forward 6400), two layers, a small vocabulary
     "xl_layers": dict(n_layer=2, n_embd=1600, n_head=25, n_inner=6400, vocab_size=3001, n_positions=512, seed=30,
                       lens=[200, 33, 90]),
+    # GPT-2 medium's and large's layer sizes (widths 1,024 and 1,280: 16 and 20 units of 64 to a row), two layers each
+    "medium_layers": dict(n_layer=2, n_embd=1024, n_head=16, n_inner=4096, vocab_size=2999, n_positions=512, seed=20,
+                          lens=[150, 40, 9]),
+    "large_layers": dict(n_layer=2, n_embd=1280, n_head=20, n_inner=5120, vocab_size=3003, n_positions=512, seed=25,
+                         lens=[170, 35, 64]),
     # three heads of 48 in a width of 144, a vocabulary that is no multiple of anything
     "odd": dict(n_layer=2, n_embd=144, n_head=3, n_inner=200, vocab_size=777, n_positions=640, seed=5,
                 lens=[600, 45, 170]),
@@ -340,7 +345,7 @@ def sized_models(tmp_path_factory):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", list(SIZES))
 def test_real_widths_whole_and_mixed(name, dtype, sized_models):
-    """GPT-2 small's full sizes, XL's layer sizes and an odd geometry: whole prompts and a
+    """GPT-2 small's full sizes, medium's, large's and XL's layer sizes and an odd geometry: whole prompts and a
     mixed schedule with pages used again, against the plain implementation."""
     d, reqs, refs = sized_models(name)
     for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=1, decode_tail=6))):
