@@ -76,7 +76,7 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
                         int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
-                        int n_splits, int chunk, float* __restrict__ partials) {
+                        int n_splits, int chunk, float* __restrict__ partials, int num_pages) {
     constexpr int KPP = 64 / LPK;  // keys per wave and pass
     __shared__ float lds2[2][AD_WAVES][LPK][10];  // the waves' sums, for the first wave to merge; two of them in turn, so that one barrier a split is enough
     const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
@@ -90,8 +90,11 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
     __shared__ int sbt[AD_MAX_BLOCKS];
     const int seq = rows_are_requests ? t : tok_seq[t];
     const int* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
-    for (int i = tid; i < max_blocks; i += 64 * AD_WAVES) sbt[i] = bt[i];
-    const int pos = tok_pos[t];
+    // (an id outside the caches' pages, an unmapped -1 or a wrong word, becomes a page that exists:
+    // whatever a table holds, no fetch leaves the caches)
+    for (int i = tid; i < max_blocks; i += 64 * AD_WAVES) sbt[i] = min(max(bt[i], 0), num_pages - 1);
+    // (a position past the block table's reach would index the staged ids out of range)
+    const int pos = static_cast<int>(min(static_cast<int64_t>(max(tok_pos[t], 0)), static_cast<int64_t>(max_blocks) * page_size - 1));
     const int hkv = h / (n_head / n_kv_head);
     // lanes past the head dimension read column 0 and multiply it by a zero query
     const int col = active ? c * 8 : 0;
@@ -287,7 +290,7 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
                             const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq,
                             const int* tok_pos, int n, float scale, int window, int n_head, int n_kv_head, int hd,
                             int page_size, int n_splits, int chunk, int waves, int rows_are_requests, float* partials,
-                            int leave_splits, hipStream_t stream) {
+                            int leave_splits, int num_pages, hipStream_t stream) {
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
         if ((1 << b) == page_size) page_shift = b;
@@ -301,15 +304,15 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
         if (waves == 4)                                                                                              \
             attention_decode_kernel<T, L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
         else if (waves == 8)                                                                                         \
             attention_decode_kernel<T, L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
         else                                                                                                         \
             attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
-                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials); \
+                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
     } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);
@@ -337,11 +340,13 @@ using namespace liyab;
 // dtype: the element type of out, q and the caches (bfloat16 or 32-bit floats). chunk: 0 = each
 // split an equal share of the token's keys; > 0 = split z takes keys [z * chunk, (z + 1) * chunk)
 // of the token's (n_splits * chunk must cover the longest context: keys beyond are not read).
+// num_pages: the pages the caches hold; page ids of the block tables are brought into [0, num_pages).
 extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                       const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
                                       const int* tok_seq, const int* tok_pos, int n, float scale, int window,
                                       int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
-                                      int rows_are_requests, float* partials, int leave_splits, hipStream_t stream) {
+                                      int rows_are_requests, float* partials, int leave_splits, int num_pages, hipStream_t stream) {
+    LIYAB_REQUIRE(num_pages > 0, "attention_decode: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
     LIYAB_REQUIRE(dtype == kBF16 || dtype == kF32, "attention_decode: unknown dtype %d", dtype);
     LIYAB_REQUIRE(!leave_splits || n_splits > 1, "attention_decode: splits are left only when there are several");
@@ -368,10 +373,10 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     if (dtype == kF32)
         return launch_attention_decode<float>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
                                               tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
-                                              rows_are_requests, partials, leave_splits, stream);
+                                              rows_are_requests, partials, leave_splits, num_pages, stream);
     return launch_attention_decode<bf16_t>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
                                            tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
-                                           rows_are_requests, partials, leave_splits, stream);
+                                           rows_are_requests, partials, leave_splits, num_pages, stream);
 }
 
 // out[m, h * hd + e] = the splits of (m, h) merged in split order: for splits that

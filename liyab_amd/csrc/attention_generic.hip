@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(ATT_THREADS)
 attention_generic_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
                          const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ block_tables,
                          int max_blocks, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale,
-                         int window, int n_head, int n_kv_head, int hd, int page_size) {
+                         int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages) {
     extern __shared__ float smem[];
     float* qs = smem;                    // [hd]
     float* sc = qs + hd;                 // [ATT_THREADS]
@@ -32,7 +32,7 @@ attention_generic_kernel(T* __restrict__ out, int64_t out_stride, const T* __res
 
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int wave = tid / kWave, lane = tid % kWave;
-    const int pos = tok_pos[t];
+    const int pos = static_cast<int>(min(static_cast<int64_t>(max(tok_pos[t], 0)), static_cast<int64_t>(max_blocks) * page_size - 1));  // within the table's reach
     const int* bt = block_tables + static_cast<int64_t>(tok_seq[t]) * max_blocks;
     const int hkv = h / (n_head / n_kv_head);
     const int first = window > 0 ? max(0, pos - window + 1) : 0;
@@ -49,7 +49,7 @@ attention_generic_kernel(T* __restrict__ out, int64_t out_stride, const T* __res
         const int j = j0 + tid;
         float s = -INFINITY;
         if (j <= pos) {
-            const int64_t page = bt[j / page_size];
+            const int64_t page = min(max(bt[j / page_size], 0), num_pages - 1);  // whatever the table holds, a page of the caches
             const T* kr = kc + ((page * n_kv_head + hkv) * page_size + j % page_size) * hd;
             float dot = 0.0f;
             for (int i = 0; i < hd; ++i) dot = fmaf(to_float<T>(kr[i]), qs[i], dot);
@@ -80,7 +80,7 @@ attention_generic_kernel(T* __restrict__ out, int64_t out_stride, const T* __res
             const int len = min(ATT_THREADS, pos - j0 + 1);
             for (int jj = g; jj < len; jj += G) {
                 const int jv = j0 + jj;
-                const int64_t page = bt[jv / page_size];
+                const int64_t page = min(max(bt[jv / page_size], 0), num_pages - 1);
                 const T* vr = vc + ((page * n_kv_head + hkv) * page_size + jv % page_size) * hd;
                 acc = fmaf(sc[jj], to_float<T>(vr[e]), acc);
             }
@@ -103,8 +103,9 @@ using namespace liyab;
 extern "C" int liyab_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                        const void* vc, int dtype, const int* block_tables, int max_blocks,
                                        const int* tok_seq, const int* tok_pos, int n, float scale, int window,
-                                       int n_head, int n_kv_head, int hd, int page_size, hipStream_t stream) {
+                                       int n_head, int n_kv_head, int hd, int page_size, int num_pages, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention: null pointer");
+    LIYAB_REQUIRE(num_pages > 0, "attention: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE(n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention: bad sizes");
     LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention: %d query heads are no multiple of %d key/value heads", n_head,
                   n_kv_head);
@@ -120,12 +121,12 @@ extern "C" int liyab_attention_generic(void* out, int64_t out_stride, const void
         attention_generic_kernel<float><<<grid, ATT_THREADS, smem, stream>>>(
             static_cast<float*>(out), out_stride, static_cast<const float*>(q), q_stride, static_cast<const float*>(kc),
             static_cast<const float*>(vc), block_tables, max_blocks, tok_seq, tok_pos, scale, window, n_head, n_kv_head,
-            hd, page_size);
+            hd, page_size, num_pages);
     } else if (dtype == kBF16) {
         attention_generic_kernel<bf16_t><<<grid, ATT_THREADS, smem, stream>>>(
             static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride,
             static_cast<const bf16_t*>(kc), static_cast<const bf16_t*>(vc), block_tables, max_blocks, tok_seq, tok_pos,
-            scale, window, n_head, n_kv_head, hd, page_size);
+            scale, window, n_head, n_kv_head, hd, page_size, num_pages);
     } else {
         return fail(1, "attention: unknown dtype %d", dtype);
     }

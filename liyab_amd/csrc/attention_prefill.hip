@@ -63,7 +63,7 @@ __global__ void __launch_bounds__(64 * QG * KS)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
-                         int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift) {
+                         int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift, int num_pages) {
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
     constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
@@ -86,7 +86,9 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     // heads vary fastest: the work list has the longest tiles first, and workgroups start in the
     // grid's order, so that every head's longest tile starts before anybody's short one
     const int* wk = work + 4 * blockIdx.y;
-    const int seq = wk[0], row0 = wk[1], pos0 = wk[2], nq = wk[3];
+    // (queries and positions within what the tile and the block table hold, whatever the list says)
+    const int seq = wk[0], row0 = wk[1], nq = min(max(wk[3], 1), 32 * QG);
+    const int pos0 = static_cast<int>(min(static_cast<int64_t>(max(wk[2], 0)), static_cast<int64_t>(max_blocks) * page_size - nq));
     const int h = blockIdx.x;
     const int hkv = h / (n_head / n_kv_head);
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -139,7 +141,8 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     // put into LDS): a load under a branch would have to be waited for where the branch ends.
     __shared__ int sbt[AP_MAX_BLOCKS];
     const int first_page = k_lo / page_size, n_pages = k_hi / page_size - first_page + 1;
-    for (int i = tid; i < n_pages; i += THREADS) sbt[i] = bt[first_page + i];  // the host has checked that they fit
+    // (the host has checked that they fit; an id outside the caches' pages becomes one that exists)
+    for (int i = tid; i < n_pages; i += THREADS) sbt[i] = min(max(bt[first_page + i], 0), num_pages - 1);
     __syncthreads();
     auto fetch = [&](int kb, u32x4 (&fk)[PER], u32x4 (&fv)[PER]) {
 #pragma unroll
@@ -369,11 +372,13 @@ using namespace liyab;
 
 // work: n_tiles x (request index, first row, first position, queries <= tile), int32; tile = 64 or 128
 // queries (2 or 4 groups of 32); ksplit = 1, 2 or 4 waves share a query group's keys (128-query tiles: 1 or 2).
+// num_pages: the pages the caches hold; page ids of the block tables are brought into [0, num_pages).
 extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                        const void* vc, const int* block_tables, int max_blocks, const int* work,
                                        int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
-                                       int page_size, hipStream_t stream) {
+                                       int page_size, int num_pages, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
+    LIYAB_REQUIRE(num_pages > 0, "attention_prefill: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
     LIYAB_REQUIRE(n_head % n_kv_head == 0 && n_head <= 65535, "attention_prefill: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
     LIYAB_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0, "attention_prefill: head size %d is not a multiple of 16 in 16..128", hd);
@@ -400,7 +405,7 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     auto* pv = static_cast<const bf16_t*>(vc);
 #define LIYAB_RUN(D, Q, S)                                                                                          \
     attention_prefill_kernel<D, Q, S, (D <= 2 && Q == 4 && S <= 2) ? 2 : 1><<<grid, 64 * Q * S, 0, stream>>>(                          \
-        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift)
+        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift, num_pages)
 #define LIYAB_RUN4(D) LIYAB_RUN(D, 2, 4)
 #define LIYAB_SKIP4(D) (void)0  // four stages of 128 keys do not fit LDS at these head sizes (refused above)
 #define LIYAB_GO(D, FOUR)                           \

@@ -69,10 +69,10 @@ __global__ void add_rows_kernel(float* __restrict__ x, const T* __restrict__ tab
 template <typename T>
 __global__ void kv_write_kernel(T* __restrict__ kc, T* __restrict__ vc, const T* __restrict__ src, int64_t src_stride,
                                 int k_off, int v_off, const int* __restrict__ slots, int n_kv_head, int hd,
-                                int page_size) {
+                                int page_size, uint32_t num_slots) {
     const int t = blockIdx.x;
     const int64_t slot = slots[t];
-    if (slot < 0) return;
+    if (static_cast<uint64_t>(slot) >= num_slots) return;  // no slot (-1), or none of these caches
     const int64_t page = slot / page_size;
     const int off = static_cast<int>(slot % page_size);
     const T* row = src + static_cast<int64_t>(t) * src_stride;
@@ -169,8 +169,10 @@ extern "C" int liyab_add_rows(float* x, const void* table, int dtype, const int*
 }
 
 extern "C" int liyab_kv_write(void* kc, void* vc, const void* src, int dtype, int64_t src_stride, int k_off, int v_off,
-                              const int* slots, int n, int n_kv_head, int hd, int page_size, hipStream_t stream) {
+                              const int* slots, int n, int n_kv_head, int hd, int page_size, int num_pages, hipStream_t stream) {
     LIYAB_REQUIRE(kc && vc && src && slots, "kv_write: null pointer");
+    LIYAB_REQUIRE(num_pages > 0 && static_cast<int64_t>(num_pages) * page_size < (int64_t{1} << 31), "kv_write: the caches hold %d pages", num_pages);
+    const uint32_t num_slots = static_cast<uint32_t>(num_pages) * static_cast<uint32_t>(page_size);
     LIYAB_REQUIRE(n >= 0 && n_kv_head > 0 && hd > 0 && page_size > 0, "kv_write: bad sizes");
     LIYAB_REQUIRE(k_off >= 0 && v_off >= 0 && k_off + n_kv_head * hd <= src_stride && v_off + n_kv_head * hd <= src_stride,
                   "kv_write: column offsets %d/%d with %d values do not fit a row of %lld", k_off, v_off, n_kv_head * hd,
@@ -180,11 +182,11 @@ extern "C" int liyab_kv_write(void* kc, void* vc, const void* src, int dtype, in
     if (dtype == kF32) {
         kv_write_kernel<float><<<n, threads, 0, stream>>>(static_cast<float*>(kc), static_cast<float*>(vc),
                                                           static_cast<const float*>(src), src_stride, k_off, v_off,
-                                                          slots, n_kv_head, hd, page_size);
+                                                          slots, n_kv_head, hd, page_size, num_slots);
     } else if (dtype == kBF16) {
         kv_write_kernel<bf16_t><<<n, threads, 0, stream>>>(static_cast<bf16_t*>(kc), static_cast<bf16_t*>(vc),
                                                            static_cast<const bf16_t*>(src), src_stride, k_off, v_off,
-                                                           slots, n_kv_head, hd, page_size);
+                                                           slots, n_kv_head, hd, page_size, num_slots);
     } else {
         return fail(1, "kv_write: unknown dtype %d", dtype);
     }

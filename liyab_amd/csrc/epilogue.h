@@ -32,6 +32,7 @@ struct EpiParams {
     const int* slots;         // [M]: page * page_size + offset
     int q_dim, kv_dim, hd, n_kv_head, page_size;
     int exact;                // erf in double (32-bit path)
+    uint32_t num_slots;       // pages x page_size of the caches: a slot outside [0, num_slots) is not written
 };
 
 // `MODE` >= 0 fixes the epilogue at compile time (straight-line code in the kernels' store
@@ -63,7 +64,7 @@ __device__ __forceinline__ void epilogue_store_biased(const EpiParams& p, int m,
                 const bool is_v = n >= p.q_dim + p.kv_dim;
                 const int c = n - p.q_dim - (is_v ? p.kv_dim : 0);
                 const int64_t slot = p.slots[m];
-                if (slot < 0) return;
+                if (static_cast<uint64_t>(slot) >= p.num_slots) return;  // no slot (-1), or none of these caches
                 const int64_t page = slot / p.page_size;
                 const int off = static_cast<int>(slot % p.page_size);
                 const int64_t dst = ((page * p.n_kv_head + c / p.hd) * p.page_size + off) * p.hd + c % p.hd;
@@ -78,10 +79,11 @@ __device__ __forceinline__ void epilogue_store_biased(const EpiParams& p, int m,
 
 // The paged QKV epilogue for kernels whose lanes hold several rows of one column: what depends
 // on the row (its slot's place in the pages) is computed once per row, ahead of the stores.
-// Element offset of row m's slot for head 0, dimension 0; -1 for a token without a slot.
+// Element offset of row m's slot for head 0, dimension 0; -1 for a token without a slot (or with
+// one past the caches' pages: a wrong word in the slots must not become a store outside them).
 __device__ __forceinline__ int64_t qkv_row_base(const EpiParams& p, int m) {
     const int64_t slot = p.slots[m];
-    if (slot < 0) return -1;
+    if (static_cast<uint64_t>(slot) >= p.num_slots) return -1;
     return (slot / p.page_size) * (static_cast<int64_t>(p.n_kv_head) * p.page_size * p.hd) + (slot % p.page_size) * p.hd;
 }
 // What depends on the column: -1 for a query column, else the offset of (head, dimension)
@@ -112,6 +114,8 @@ inline int check_epilogue(const EpiParams& p, int M, int N) {
         LIYAB_REQUIRE(p.q_dim > 0 && p.kv_dim > 0 && p.hd > 0 && p.page_size > 0 && p.n_kv_head * p.hd == p.kv_dim &&
                           p.q_dim + 2 * p.kv_dim == N && p.ldo >= p.q_dim,
                       "gemm: the paged QKV epilogue's sizes do not fit N = %d", N);
+        LIYAB_REQUIRE(p.num_slots > 0 && p.num_slots % static_cast<uint32_t>(p.page_size) == 0,
+                      "gemm: the paged QKV epilogue needs the caches' slots (pages x page size), got %u", p.num_slots);
     } else {
         LIYAB_REQUIRE(p.mode >= kEpiNone && p.mode <= kEpiGeluErf, "gemm: unknown epilogue %d", p.mode);
         LIYAB_REQUIRE(p.out != nullptr && p.ldo >= N, "gemm: needs an output of row stride >= N");

@@ -316,7 +316,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                     const int slot = epi.slots[min(mw + (t * 64 + lane) / CHUNKS, M - 1)];
                     const int page = page_shift >= 0 ? slot >> page_shift : slot / epi.page_size;
                     const int off = slot - page * epi.page_size;
-                    row_base[t] = slot < 0 ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
+                    row_base[t] = static_cast<uint32_t>(slot) >= epi.num_slots ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
                 }
             }
 #pragma unroll
@@ -353,7 +353,7 @@ gemm_mfma_dl_kernel(const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __r
                 const int slot = epi.slots[m];
                 const int page = page_shift >= 0 ? slot >> page_shift : slot / epi.page_size;
                 const int off = slot - page * epi.page_size;
-                row_base = slot < 0 ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
+                row_base = static_cast<uint32_t>(slot) >= epi.num_slots ? -1 : static_cast<int64_t>(page) * epi.n_kv_head * epi.page_size * epi.hd + static_cast<int64_t>(off) * epi.hd;
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {

@@ -111,8 +111,8 @@ void* liyab_sched_create(void* manager, int max_num_seqs, int max_batched_tokens
     return new SchedulerHandle{Scheduler(static_cast<CacheManager*>(manager), max_num_seqs, max_batched_tokens, prefill_chunk), {}, {}, {}};
 }
 void liyab_sched_destroy(void* h) { delete static_cast<SchedulerHandle*>(h); }
-int liyab_sched_add(void* h, int n_prompt, int max_tokens, int* id) {
-    return static_cast<SchedulerHandle*>(h)->sched.add(n_prompt, max_tokens, id, &g_error);
+int liyab_sched_add(void* h, int n_prompt, int max_tokens, int priority, int* id) {
+    return static_cast<SchedulerHandle*>(h)->sched.add(n_prompt, max_tokens, priority, id, &g_error);
 }
 int liyab_sched_pressure(void* h) { return static_cast<SchedulerHandle*>(h)->sched.pressure() ? 1 : 0; }
 // The step's batch; it stays valid until the next call. counts: [batch, opened, preempted].
@@ -134,7 +134,7 @@ void liyab_sched_tokens(void* h, const int* ids, const int* is_stop, int n, int*
     for (int i = 0; i < n; ++i) reasons[i] = s.token(ids[i], is_stop[i] != 0);
 }
 int liyab_sched_finish(void* h, int id) { return static_cast<SchedulerHandle*>(h)->sched.finish(id, &g_error); }
-// what: 0 state, 1 computed, 2 pending, 3 generated, 4 preemptions, 5 slot
+// what: 0 state, 1 computed, 2 pending, 3 generated, 4 preemptions, 5 slot, 6 priority
 int liyab_sched_get(void* h, int id, int what) {
     const auto& s = static_cast<SchedulerHandle*>(h)->sched;
     if (id < 0) return -1;
@@ -145,6 +145,7 @@ int liyab_sched_get(void* h, int id, int what) {
         case 3: return s.n_generated(id);
         case 4: return s.preemptions(id);
         case 5: return s.slot(id);
+        case 6: return s.priority(id);
         default: return -1;
     }
 }

@@ -13,7 +13,7 @@ Scheduler::Scheduler(CacheManager* manager, int max_num_seqs, int max_batched_to
     : m_(manager), max_num_seqs_(std::min(max_num_seqs, manager->max_requests())), max_batched_tokens_(max_batched_tokens),
       prefill_chunk_(prefill_chunk) {}
 
-Status Scheduler::add(int n_prompt, int max_tokens, int* id, std::string* err) {
+Status Scheduler::add(int n_prompt, int max_tokens, int priority, int* id, std::string* err) {
     if (n_prompt <= 0) return fail(err, kInvalidArgument, "the prompt is empty");  // src/core/engine.cpp:3867-3871
     if (max_tokens <= 0) return fail(err, kInvalidArgument, "max_tokens must be positive");
     if (n_prompt >= m_->max_positions() + 1)
@@ -29,9 +29,13 @@ Status Scheduler::add(int n_prompt, int max_tokens, int* id, std::string* err) {
     Request r;
     r.n_prompt = n_prompt;
     r.max_tokens = max_tokens;
+    r.priority = priority;
     *id = next_id_++;
     reqs_.emplace(*id, r);
-    waiting_.push_back(*id);
+    // behind every waiting request of its own or a higher priority
+    auto at = waiting_.begin();
+    while (at != waiting_.end() && req(*at).priority >= priority) ++at;
+    waiting_.insert(at, *id);
     return kOk;
 }
 
@@ -76,7 +80,10 @@ Status Scheduler::preempt(int id, std::string* err) {
     r.state = kWaiting;
     r.preemptions += 1;
     stats_.preemptions += 1;
-    waiting_.push_front(id);
+    // ahead of every waiting request of its own or a lower priority
+    auto at = waiting_.begin();
+    while (at != waiting_.end() && req(*at).priority > r.priority) ++at;
+    waiting_.insert(at, id);
     return kOk;
 }
 
@@ -136,7 +143,7 @@ Status Scheduler::schedule(std::vector<Scheduled>* batch, std::vector<int>* open
         }
         if (count > 0 && r.state == kRunning) take(id, count);
     }
-    // admission, first come first served
+    // admission: the queue's order (priority, then first come first served)
     while (!waiting_.empty() && static_cast<int>(running_.size()) < max_num_seqs_ && budget > 0) {
         const int id = waiting_.front();
         Request& r = req(id);

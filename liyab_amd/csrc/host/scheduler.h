@@ -10,10 +10,14 @@
 //
 //   * every step first gives each decoding request its one token, then hands the rest of the
 //     token budget to prompt portions in order of admission (a portion is as small as the budget
-//     leaves, down to one token), then admits waiting requests first come, first served, while a
-//     request slot, budget and pages for the first portion are there;
+//     leaves, down to one token), then admits waiting requests, the higher priority first and
+//     first come, first served among equals, while a request slot, budget and pages for the
+//     first portion are there (the reference has two classes, foreground and background, and
+//     lets foreground requests go first: src/core/engine.cpp:1936-1945; here a priority is any
+//     integer, the larger the sooner, and it orders admission only);
 //   * when a request cannot get its pages, the most recently admitted running request is
-//     preempted: its pages and slot go back, it returns to the head of the waiting queue and is
+//     preempted: its pages and slot go back, it returns to the waiting queue ahead of every
+//     request of its own or a lower priority and is
 //     recomputed from its prompt plus what it has generated. A request is never preempted for
 //     its own sake by a later one, and a request that could not fit the pool alone is refused
 //     on arrival.
@@ -52,8 +56,9 @@ class Scheduler {
 public:
     Scheduler(CacheManager* manager, int max_num_seqs, int max_batched_tokens, int prefill_chunk);
 
-    // A new request of n_prompt tokens that may generate max_tokens; its id goes to *id.
-    Status add(int n_prompt, int max_tokens, int* id, std::string* err);
+    // A new request of n_prompt tokens that may generate max_tokens; its id goes to *id. It
+    // waits behind every request of its own or a higher priority.
+    Status add(int n_prompt, int max_tokens, int priority, int* id, std::string* err);
     bool has_unfinished() const { return !waiting_.empty() || !running_.empty(); }
     // Whether the request's pending token is its last whatever it turns out to be.
     bool draining(int id) const;
@@ -79,6 +84,7 @@ public:
     int n_generated(int id) const { const Request* r = find(id); return r ? r->n_generated : 0; }
     int preemptions(int id) const { const Request* r = find(id); return r ? r->preemptions : 0; }
     int slot(int id) const { const Request* r = find(id); return r ? r->slot : -1; }
+    int priority(int id) const { const Request* r = find(id); return r ? r->priority : 0; }
     int n_requests() const { return static_cast<int>(reqs_.size()); }  // the unfinished ones
     const std::vector<int>& running() const { return running_; }
     const std::deque<int>& waiting() const { return waiting_; }
@@ -88,7 +94,7 @@ private:
     struct Request {
         int n_prompt, max_tokens;
         int n_generated = 0, pending = 0, computed = 0;
-        int state = kWaiting, slot = -1, preemptions = 0;
+        int state = kWaiting, slot = -1, preemptions = 0, priority = 0;
         int n_tokens() const { return n_prompt + n_generated + pending; }
         int remaining() const { return n_tokens() - computed; }
     };

@@ -51,7 +51,7 @@ static int run(unsigned seed, int n_steps) {
         while (pick(0, 3) == 0 && s.n_requests() < 12) {
             int id = -1;
             const int n_prompt = pick(1, max_positions + 3), max_tokens = pick(1, 40);
-            const Status st = s.add(n_prompt, max_tokens, &id, &err);
+            const Status st = s.add(n_prompt, max_tokens, static_cast<int>(rng() % 3) - 1, &id, &err);
             CHECK(st == kOk || st == kInvalidArgument || st == kOutOfPages, "seed %u: add: %s", seed, err.c_str());
         }
         // tokens of the step before reach the host before this one is scheduled, or lag one step

@@ -134,7 +134,10 @@ class Engine:
 
     # -- continuous batching ------------------------------------------------------
     def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
-                    rid: Optional[Hashable] = None) -> Hashable:
+                    rid: Optional[Hashable] = None, priority: int = 0) -> Hashable:
+        """`priority`: among waiting requests the larger is admitted first (first come, first
+        served among equals); the reference's foreground and background sequences
+        (include/liyab/engine.h:1034, 1088-1091) are two values of it."""
         params = params or SamplingParams()
         prompt = [int(t) for t in prompt_ids]
         V = self.core.vocab_size
@@ -146,7 +149,7 @@ class Engine:
             self._next_id += 1
         if rid in self._requests and self._requests[rid].state != "finished":
             raise InvalidArgument(f"request {rid!r} is still running")
-        r = Request(rid=rid, prompt=prompt, params=params, seed=params.resolved_seed())
+        r = Request(rid=rid, prompt=prompt, params=params, seed=params.resolved_seed(), priority=int(priority))
         self.scheduler.add(r)
         self._requests[rid] = r
         self._t_first.pop(rid, None)  # an id used before starts its clocks again

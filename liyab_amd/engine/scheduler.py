@@ -4,7 +4,7 @@ finishing, and what happens when pages run out.
 The decisions are native (`csrc/host/scheduler.{h,cpp}`, where the rules and
 their sources in the reference are written down: decoding requests first,
 then prompt portions under the token budget in order of admission, then
-first-come-first-served admission; when pages run out the most recently
+admission by priority, first come first served among equals; when pages run out the most recently
 admitted running request is preempted and recomputed later). This module
 is their Python face: `Request` objects carry what only the caller knows
 (the token ids, the sampling parameters), mirror the counters the native
@@ -47,6 +47,7 @@ class Request:
     arrival: int = 0
     pending: int = 0  # tokens sampled in steps whose result the host has not read yet (at most 1 when scheduling)
     sid: int = -1  # the native scheduler's id of this request
+    priority: int = 0  # the larger the sooner it is admitted; first come, first served among equals
     _prompt_ids: Optional[np.ndarray] = field(default=None, repr=False, compare=False)  # the prompt as an array, made when a portion is first asked for
 
     @property
@@ -146,7 +147,8 @@ class Scheduler:
     def add(self, request: Request) -> None:
         sid = ctypes.c_int(-1)
         try:
-            host.check(self._lib.liyab_sched_add(self._h, len(request.prompt), int(request.params.max_tokens), ctypes.byref(sid)))
+            host.check(self._lib.liyab_sched_add(self._h, len(request.prompt), int(request.params.max_tokens),
+                                                 int(request.priority), ctypes.byref(sid)))
         except Exception as e:
             raise type(e)(f"request {request.rid!r}: {e}") from None
         request.sid = sid.value
@@ -154,7 +156,18 @@ class Scheduler:
         request.arrival = self._arrivals
         self._arrivals += 1
         self._by_sid[sid.value] = request
-        self.waiting.append(request)
+        self._enqueue(request, behind_equals=True)
+
+    def _enqueue(self, request: Request, behind_equals: bool) -> None:
+        """Into the waiting queue where the native side puts it: behind every request of a higher
+        priority, and behind (a new request) or ahead of (a preempted one) those of its own."""
+        at = 0
+        for other in self.waiting:
+            if other.priority > request.priority or (behind_equals and other.priority == request.priority):
+                at += 1
+            else:
+                break
+        self.waiting.insert(at, request)
 
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
@@ -185,7 +198,7 @@ class Scheduler:
             r.computed = 0
             r.state = WAITING
             r.preemptions += 1
-            self.waiting.appendleft(r)
+            self._enqueue(r, behind_equals=False)
         host.check(rc)
         raw = self._raw
         opened = {self._opened[i] for i in range(n_opened)}

@@ -61,7 +61,7 @@ _SIGNATURES = {
     "liyab_cm_check": ([c_void_p], c_int),
     "liyab_sched_create": ([c_void_p, c_int, c_int, c_int], c_void_p),
     "liyab_sched_destroy": ([c_void_p], None),
-    "liyab_sched_add": ([c_void_p, c_int, c_int, IP], c_int),
+    "liyab_sched_add": ([c_void_p, c_int, c_int, c_int, IP], c_int),
     "liyab_sched_pressure": ([c_void_p], c_int),
     "liyab_sched_schedule": ([c_void_p, POINTER(POINTER(Scheduled)), POINTER(IP), POINTER(IP), IP], c_int),
     "liyab_sched_advance": ([c_void_p, POINTER(Scheduled), c_int], None),

@@ -28,7 +28,7 @@ class EpiParams(ctypes.Structure):
     _fields_ = [
         ("mode", c_int), ("out_dtype", c_int), ("bias", P), ("out", P), ("ldo", c_int64), ("residual", P),
         ("ldr", c_int64), ("kc", P), ("vc", P), ("slots", P), ("q_dim", c_int), ("kv_dim", c_int), ("hd", c_int),
-        ("n_kv_head", c_int), ("page_size", c_int), ("exact", c_int),
+        ("n_kv_head", c_int), ("page_size", c_int), ("exact", c_int), ("num_slots", c_uint32),
     ]
 
 
@@ -40,7 +40,7 @@ _SIGNATURES = {
     "liyab_add_rows": [P, P, c_int, P, c_int, c_int, P],
     "liyab_gather_rows": [P, c_int, P, P, c_int, c_int, P],
     "liyab_scale": [P, c_float, c_int64, P],
-    "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
+    "liyab_kv_write": [P, P, P, c_int, c_int64, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, P],
     "liyab_layernorm": [P, c_int, P, P, P, P, c_int, c_int, c_float, P],
     "liyab_layernorm_parts": [P, c_int, P, c_int, c_int64, c_int, P, P, P, c_int, c_int, c_float, P],
     "liyab_sum_parts": [P, c_int, c_int, P, c_int, c_int64, P],
@@ -51,14 +51,14 @@ _SIGNATURES = {
     "liyab_gemm_mfma_dl_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_skinny": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_generic": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_int, c_int,
-                                c_int, c_int, c_int, P],
+                                c_int, c_int, c_int, c_int, P],
     "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, P],
+                               c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, P],
     "liyab_attention_merge": [P, c_int, c_int64, P, c_int, c_int, c_int, c_int, P],
     "liyab_gemm_att_parts": [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_skinny_ln": [P, c_int, c_int64, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
     "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
-                                c_int, c_int, c_int, P],
+                                c_int, c_int, c_int, c_int, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
     "liyab_argmax_static_init": [],
     "liyab_argmax_static": [P, P, c_int64, c_int, c_int, P, P, P],

@@ -117,6 +117,17 @@ def _rows(t: torch.Tensor, what: str) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
 
 
+def _pages(k_cache: torch.Tensor, num_pages: Optional[int]) -> int:
+    """The number of pages a launcher is told the caches hold: all of them unless the caller
+    counts fewer (page ids and slots beyond that count are not followed by the kernels)."""
+    pages = k_cache.shape[0] if num_pages is None else int(num_pages)
+    if not 0 < pages <= k_cache.shape[0]:
+        raise KernelError(f"the caches hold {k_cache.shape[0]} pages, not {pages}")
+    if pages * k_cache.shape[2] >= 1 << 31:
+        raise KernelError(f"{pages} pages of {k_cache.shape[2]} positions: slots must fit 31 bits")
+    return pages
+
+
 def check_device() -> None:
     _lib.call("liyab_check_device")
 
@@ -292,10 +303,10 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 
 def kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, src: torch.Tensor, k_off: int, v_off: int,
-             slots: torch.Tensor) -> None:
+             slots: torch.Tensor, num_pages: Optional[int] = None) -> None:
     """Writes token t's keys src[t, k_off:k_off+Hkv*hd] and values to slot slots[t] of caches
-    laid out [pages, kv_heads, page_size, head_dim]. Slots are page * page_size + offset; the
-    caller has checked them against the cache's pages."""
+    laid out [pages, kv_heads, page_size, head_dim]. Slots are page * page_size + offset; a
+    slot outside the caches' `num_pages` (all of them by default) pages is not written."""
     _dev(k_cache, "k_cache")
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("kv_write: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
@@ -308,12 +319,12 @@ def kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, src: torch.Tensor, k_
     if k_off + hkv * hd > src.shape[1] or v_off + hkv * hd > src.shape[1]:
         raise KernelError("kv_write: column offsets pass the source's width")
     _lib.call("liyab_kv_write", k_cache.data_ptr(), v_cache.data_ptr(), src.data_ptr(), dtype_code(src.dtype), stride,
-              k_off, v_off, slots.data_ptr(), n, hkv, hd, page, _stream())
+              k_off, v_off, slots.data_ptr(), n, hkv, hd, page, _pages(k_cache, num_pages), _stream())
 
 
 def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
-                      scale: float, window: int = 0) -> None:
+                      scale: float, window: int = 0, num_pages: Optional[int] = None) -> None:
     """out[t, h*hd:(h+1)*hd] = softmax(scale * q_th . K[:pos_t+1]) V for the request tok_seq[t].
     q is [n, >= n_head*hd] (a view into a wider projection output is fine)."""
     n = out.shape[0]
@@ -333,7 +344,7 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     _i32(tok_pos, "tok_pos", n)
     _lib.call("liyab_attention_generic", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], tok_seq.data_ptr(),
-              tok_pos.data_ptr(), n, float(scale), int(window), n_head, hkv, hd, page, _stream())
+              tok_pos.data_ptr(), n, float(scale), int(window), n_head, hkv, hd, page, _pages(k_cache, num_pages), _stream())
 
 
 _argmax_scratch = {}
@@ -416,7 +427,8 @@ def _epilogue(a, w, bias, out, residual, epilogue, kv):
             raise KernelError("gemm: the residual epilogue needs a float32 residual [M, N]")
         e.residual, e.ldr = residual.data_ptr(), _rows(residual, "residual")
     elif epilogue == EPI_QKV_PAGED:
-        k_cache, v_cache, slots, q_dim = kv
+        k_cache, v_cache, slots, q_dim = kv[:4]
+        e.num_slots = _pages(k_cache, kv[4] if len(kv) > 4 else None) * k_cache.shape[2]
         if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
             raise KernelError("gemm: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
         _, hkv, page, hd = k_cache.shape
@@ -685,7 +697,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], *, out:
          residual: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, kv=None) -> None:
     """The product kernel for these operands: matrix cores for bfloat16 shapes they take,
     the plain tiled kernel for float32 and everything else. `kv` = (k_cache, v_cache, slots,
-    q_dim) with the paged QKV epilogue."""
+    q_dim[, num_pages]) with the paged QKV epilogue (a slot outside the caches' pages is not written)."""
     if _invariant and mfma_takes(a, w):
         # one family of kernels whatever the number of rows: their sum over k has one order for
         # every tile shape, so a row's bits do not depend on the rows beside it. K a multiple of 64:
@@ -747,7 +759,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      block_tables: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor, *, n_head: int,
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
-                     rows_are_requests: bool = False, leave_splits: bool = False, chunk: int = 0) -> None:
+                     rows_are_requests: bool = False, leave_splits: bool = False, chunk: int = 0,
+                     num_pages: Optional[int] = None) -> None:
     """Each token on its own over its request's cache (bfloat16, or float32 throughout), its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
     request t (every request brings one token), which saves the kernel a lookup. With
@@ -784,7 +797,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
     _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
               n, float(scale), int(window), n_head, hkv, hd, page, n_splits, int(chunk), waves, 1 if rows_are_requests else 0,
-              _ptr(partials), 1 if leave_splits else 0, _stream())
+              _ptr(partials), 1 if leave_splits else 0, _pages(k_cache, num_pages), _stream())
 
 
 def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
@@ -802,7 +815,7 @@ def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, work: torch.Tensor, n_tiles: int, *, n_head: int, scale: float,
-                      window: int = 0, tile: int = 128, ksplit: int = 1) -> None:
+                      window: int = 0, tile: int = 128, ksplit: int = 1, num_pages: Optional[int] = None) -> None:
     """Tiles of up to `tile` (64 or 128) consecutive queries of one request over its bfloat16
     cache, on the matrix cores; `ksplit` waves (1, 2, or 4 with tiles of 64) share the keys of
     32 queries. work: int32 [n_tiles, 4] = (request index, first row, first
@@ -823,7 +836,7 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     _i32(work, "work", 4 * n_tiles)
     _lib.call("liyab_attention_prefill", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
               block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), int(ksplit), float(scale), int(window),
-              n_head, hkv, hd, page, _stream())
+              n_head, hkv, hd, page, _pages(k_cache, num_pages), _stream())
 
 
 PREFILL_KSPLIT4_WORK = 256  # tiles x heads up to which four waves share a tile of 64 queries' keys
@@ -888,6 +901,16 @@ ATTENTION_MAX_HEAD_DIM = 256  # what the attention kernels take (attention_gener
 
 INVARIANT_CHUNK = 256  # keys a split where splits go by position alone
 INVARIANT_SPLIT_WORK = 1024  # (token, head, split) workgroups up to which such splits are launched side by side
+INVARIANT_MAX_SPLITS = 16  # what one workgroup walks in turn (attention_decode.hip: AD_LOOP_CHUNKS)
+
+
+def invariant_chunk(reach: int) -> int:
+    """Keys a split where splits go by position alone, for requests that reach at most `reach` keys:
+    INVARIANT_CHUNK, doubled until INVARIANT_MAX_SPLITS splits cover the reach."""
+    chunk = INVARIANT_CHUNK
+    while chunk * INVARIANT_MAX_SPLITS < reach:
+        chunk *= 2
+    return chunk
 
 
 def attention_takes(head_dim: int) -> bool:
@@ -926,15 +949,19 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         # in splits of INVARIANT_CHUNK from its first key on, merged in their order: the order of a
         # token's sums follows from its position alone, so its bits do not depend on the batch
         n = out.shape[0]
-        splits = max(1, -(-min(plan.context_bucket, window if window > 0 else plan.context_bucket) // INVARIANT_CHUNK))
+        # a split's keys follow from what a request can reach at most (the table's width, the window): a
+        # constant of the engine, never of the step; at most 16 splits, so that one workgroup can walk them
+        # all and the merge's arrays hold them (contexts past 4,096 keys take longer splits)
+        reach = block_tables.shape[1] * k_cache.shape[2] if window <= 0 else min(window, block_tables.shape[1] * k_cache.shape[2])
+        chunk = invariant_chunk(reach)
+        splits = max(1, -(-min(plan.context_bucket, reach) // chunk))
         # many tokens: a workgroup walks its token's splits in turn (the same bits: the kernel merges them
         # as the merge kernel does), which saves the splits' traffic and leaves the chip as full
-        reach = block_tables.shape[1] * k_cache.shape[2] if window <= 0 else min(window, block_tables.shape[1] * k_cache.shape[2])
-        if n * n_head * splits > INVARIANT_SPLIT_WORK and reach <= INVARIANT_CHUNK * 16:
+        if n * n_head * splits > INVARIANT_SPLIT_WORK:
             splits = 1
         partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32) if splits > 1 else None
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
-                         window=window, n_splits=splits, partials=partials, waves=4, chunk=INVARIANT_CHUNK,
+                         window=window, n_splits=splits, partials=partials, waves=4, chunk=chunk,
                          rows_are_requests=host.max_q_len == 1)
         return None
     if fast and plan.mode == "decode" and block_tables.shape[1] <= 2048:

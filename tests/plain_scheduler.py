@@ -31,6 +31,7 @@ class Request:
     preemptions: int = 0
     arrival: int = 0
     pending: int = 0  # tokens sampled in steps whose result the host has not read yet (at most 1 when scheduling)
+    priority: int = 0  # the larger the sooner it is admitted
 
     @property
     def tokens(self) -> List[int]:
@@ -111,7 +112,16 @@ class Scheduler:
         request.state = WAITING
         request.arrival = self._arrivals
         self._arrivals += 1
-        self.waiting.append(request)
+        self._enqueue(request, behind_equals=True)
+
+    def _enqueue(self, request, behind_equals: bool) -> None:
+        """Behind every waiting request of a higher priority, and behind (a new request) or ahead
+        of (a preempted one) those of its own: foreground before background as the reference
+        chooses a pass's requests (src/core/engine.cpp:1936-1945), first come first served among equals."""
+        queue = list(self.waiting)
+        keep = [o for o in queue if o.priority > request.priority or (behind_equals and o.priority == request.priority)]
+        assert queue[:len(keep)] == keep  # the queue is ordered by priority
+        self.waiting.insert(len(keep), request)
 
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
@@ -160,7 +170,7 @@ class Scheduler:
         r.state = WAITING
         r.preemptions += 1
         self.stats.preemptions += 1
-        self.waiting.appendleft(r)
+        self._enqueue(r, behind_equals=False)
 
     def schedule(self) -> List[Scheduled]:
         """Chooses this step's batch and opens/preempts requests accordingly.

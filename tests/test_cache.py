@@ -237,3 +237,67 @@ def test_native_manager_does_what_the_plain_one_does(seed):
             assert a.length(rid) == b.length(rid) == length and a.slot(rid) == b.slot(rid)
             assert [a.block_table(rid, g) for g in range(2)] == [b.block_table(rid, g) for g in range(2)]
             assert a.pages_needed(rid, length + 33) == b.pages_needed(rid, length + 33)
+
+
+@pytest.mark.parametrize("seed,page_size,window", [(0, 16, 0), (1, 4, 0), (2, 24, 0), (3, 8, 20), (4, 48, 100)])
+def test_a_steps_metadata_names_only_pages_and_slots_of_the_pool(seed, page_size, window):
+    """Random stories of requests through the step metadata's native layout (liyab_step_shape /
+    liyab_step_fill): every page id a block table carries to the device is -1 or a page of the
+    pool, every slot a position of a page of the pool, and the slot of a token is its page's
+    place in the table. The kernels follow these words without asking."""
+    import ctypes
+
+    from liyab_amd import host
+
+    rng = random.Random(seed)
+    num_pages, max_positions, vocab = 40, 300, 1000
+    groups = [(KVSpec(2, 16, 0), [0]), (KVSpec(2, 16, window), [1])] if window else [(KVSpec(2, 16, 0), [0, 1])]
+    m = CacheManager(groups, page_size=page_size, num_pages=num_pages, max_requests=6, max_positions=max_positions)
+    lib = host.lib()
+    ip = lambda a: a.ctypes.data_as(host.IP)  # noqa: E731
+    live, next_id, steps = {}, 0, 0
+    for _ in range(400):
+        if len(live) < 6 and (not live or rng.random() < 0.3):
+            m.open(next_id)
+            live[next_id] = 0
+            next_id += 1
+        batch = [r for r in live if rng.random() < 0.7] or [next(iter(live))]
+        q = [min(rng.choice([1, 1, 1, 2, 5, 17, 60]), max_positions - live[r]) for r in batch]
+        batch, q = [r for r, n in zip(batch, q) if n > 0], [n for n in q if n > 0]
+        if batch:
+            slots = np.array([m.slot(r) for r in batch], dtype=np.intc)
+            q_lens = np.array(q, dtype=np.intc)
+            try:
+                new_lengths = m.reserve_more(slots, q_lens)
+            except OutOfPages:
+                victim = rng.choice(list(live))
+                m.close(victim)
+                del live[victim]
+                continue
+            wants = np.zeros(len(batch), dtype=np.intc)
+            shape = host.StepShape()
+            host.check(lib.liyab_step_shape(m.handle, len(batch), ip(slots), ip(q_lens), ip(wants), ctypes.byref(shape)))
+            block = np.full(shape.total, -12345, dtype=np.int32)
+            tokens = np.array([rng.randrange(vocab) for _ in range(int(q_lens.sum()))], dtype=np.int64)
+            host.check(lib.liyab_step_fill(m.handle, ctypes.byref(shape), ip(slots), ip(q_lens),
+                                           tokens.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), ip(wants), ip(np.zeros(1, dtype=np.intc)),
+                                           vocab, block.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))))
+            S, N, W = len(batch), int(q_lens.sum()), shape.max_blocks
+            positions = block[shape.off_positions:shape.off_positions + N]
+            tok_seq = block[shape.off_tok_seq:shape.off_tok_seq + N]
+            assert positions.min() >= 0 and positions.max() < W * page_size
+            for g in range(shape.n_groups):
+                bt = block[shape.off_block_tables[g]:shape.off_block_tables[g] + S * W].reshape(S, W)
+                sl = block[shape.off_slots[g]:shape.off_slots[g] + N]
+                assert bt.min() >= -1 and bt.max() < num_pages
+                assert sl.min() >= 0 and sl.max() < num_pages * page_size
+                assert (sl == bt[tok_seq, positions // page_size] * page_size + positions % page_size).all()
+            m.commit_slots(slots, new_lengths)
+            for r, n in zip(batch, new_lengths):
+                live[r] = int(n)
+            steps += 1
+        for r in [r for r in live if live[r] >= max_positions or rng.random() < 0.03]:
+            m.close(r)
+            del live[r]
+        m.check()
+    assert steps > 200

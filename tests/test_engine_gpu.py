@@ -48,12 +48,12 @@ def reference(plain_models):
     return out
 
 
-def make_core(model_dir, dtype, max_tokens, page_size=16, poison=True):
+def make_core(model_dir, dtype, max_tokens, page_size=16, poison=True, num_pages=None):
     import torch
 
     from liyab_amd.engine import EngineCore
 
-    core = EngineCore(model_dir, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8)
+    core = EngineCore(model_dir, dtype=dtype, page_size=page_size, max_tokens=max_tokens, num_pages=num_pages, max_requests=8)
     if poison:  # free pages hold NaN: a kernel that reads past a request's length shows it
         for c in core.storage.layers.values():
             for t in c.rows.values():
@@ -114,6 +114,28 @@ def test_mixed_batches_with_pages_used_again(name, dtype, seed, model_dirs, refe
     tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"mixed {name} {dtype}")
     core.manager.check()
     assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", [("A", 24), ("B", 48), ("B", 3)])
+def test_mixed_batches_with_pages_that_are_no_power_of_two(name, page_size, dtype, model_dirs, reference):
+    """Pages of 24, 48 and 3 positions (the reference takes any page_tokens,
+    include/liyab/kv_cache.h:72-80): page and offset by division in every kernel that looks a
+    position up, with just the pages the schedule needs, so that they are used again."""
+    reqs = make_requests(name)
+    steps = tt.schedule_mixed(reqs, seed=3)
+    pages = tt.max_live_pages(steps, page_size)
+    assert pages < sum(-(-len(t) // page_size) for t in reqs.values())
+    core = make_core(model_dirs[name], dtype, None, page_size=page_size, num_pages=pages)
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"mixed, pages of {page_size}, {name} {dtype}", family="mixed")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+    # whole prompts through the tiled attention kernel, too
+    steps = tt.schedule_whole(reqs)
+    core = make_core(model_dirs[name], dtype, None, page_size=page_size, num_pages=tt.max_live_pages(steps, page_size))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL[dtype], f"whole, pages of {page_size}, {name} {dtype}", family="whole")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

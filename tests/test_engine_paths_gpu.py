@@ -24,15 +24,17 @@ def _near_argmax(ref_row, token, tol):
 # preemption and recomputation on the device
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("overlap", [False, True])
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_preempted_requests_are_recomputed_to_the_same_tokens(dtype, overlap, model_dirs, plain_models):
+@pytest.mark.parametrize("mode", DTYPES + ["bfloat16 batch-invariant"])
+def test_preempted_requests_are_recomputed_to_the_same_tokens(mode, overlap, model_dirs, plain_models):
     """Three prompts of 30 tokens that each grow to 74 positions (5 pages of 16) in a pool of 8
     pages: they cannot all stay, so the latest admitted is preempted, its pages go to the others
     and it is recomputed from its prompt plus what it had generated, through pages other
     requests have used. Greedy and seeded: the tokens are those of each request alone (in
-    32-bit also the plain implementation's), whatever was preempted when."""
+    32-bit also the plain implementation's), whatever was preempted when; in bfloat16 that holds
+    bit for bit in the batch-invariant mode, and within the tolerance of the plain choice otherwise."""
     from liyab_amd import Engine, SamplingParams
 
+    dtype, invariant = mode.split()[0], "invariant" in mode
     name = "B"
     cfg, _ = CONFIGS[name]
     config, tensors = plain_models[name]
@@ -42,7 +44,7 @@ def test_preempted_requests_are_recomputed_to_the_same_tokens(dtype, overlap, mo
     for sp in (SamplingParams(temperature=0.0, max_tokens=45),
                SamplingParams(temperature=0.8, top_k=0, top_p=1.0, seed=4, max_tokens=45)):
         tight = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=8, max_num_seqs=3, max_batched_tokens=64,
-                       prefill_chunk=32, overlap=overlap)
+                       prefill_chunk=32, overlap=overlap, batch_invariant=invariant)
         tight.stop_at_eos = False
         for c in tight.core.storage.layers.values():  # free pages hold NaN
             for t in c.rows.values():
@@ -55,17 +57,17 @@ def test_preempted_requests_are_recomputed_to_the_same_tokens(dtype, overlap, mo
         tight.core.manager.check()
         assert tight.core.step_fn.graph_replays > 0
         roomy = Engine(model_dirs[name], dtype=dtype, page_size=16, num_pages=64, max_num_seqs=3, max_batched_tokens=64,
-                       prefill_chunk=32, overlap=overlap)
+                       prefill_chunk=32, overlap=overlap, batch_invariant=invariant)
         roomy.stop_at_eos = False
         alone = [roomy.generate(p, sp) for p in prompts]
         assert roomy.scheduler.stats.preemptions == 0
         for prompt, a, b in zip(prompts, together, alone):
             assert len(a.tokens) == 45 and a.finish_reason == "length"
-            if dtype == "float32":
+            if dtype == "float32" or invariant:
                 assert a.tokens == b.tokens
-                if sp.temperature == 0.0:
+                if sp.temperature == 0.0 and dtype == "float32":
                     assert a.tokens == plain.generate_greedy(config, tensors, prompt, 45)
-            elif sp.temperature == 0.0:
+            if dtype == "bfloat16" and sp.temperature == 0.0:
                 # bfloat16: each token is the plain implementation's choice given the tokens before it,
                 # within the tolerance (a recomputed prompt goes through other kernels than single tokens)
                 ref = plain.forward(config, weights, prompt + a.tokens[:-1])
@@ -277,7 +279,9 @@ def test_batch_invariant_logits_have_the_same_bits_alone_and_together(small_widt
 
     d, cfg = small_widths_model
     V = cfg["vocab_size"]
-    reqs = {f"i{i}": tt.random_tokens(500 + i, n, V) for i, n in enumerate([150, 33, 9, 70, 260])}
+    # (the request of 950 tokens: its whole prompt walks four splits of 256 keys in one workgroup a
+    # token and head, its last tokens are launched in splits side by side)
+    reqs = {f"i{i}": tt.random_tokens(500 + i, n, V) for i, n in enumerate([150, 33, 9, 70, 260, 950])}
     runs = {}
     for label, steps in (("whole", tt.schedule_whole(reqs)), ("tail", tt.schedule_bulk_tail(reqs, tail=12)),
                          ("portions", tt.schedule_portions(reqs, (5, 2, 17, 3, 48, 2, 31, 7))),
@@ -298,6 +302,33 @@ def test_batch_invariant_logits_have_the_same_bits_alone_and_together(small_widt
     fast = tt.run_schedule(core, steps)
     worst = max(tt.rel_err(fast[rid][p], runs["whole"][rid][p]) for rid, toks in reqs.items() for p in range(len(toks)))
     assert 0 < worst <= TOL["bfloat16"]
+
+
+def test_float32_logits_have_the_same_bits_whole_and_token_by_token(small_widths_model):
+    """The 32-bit path at GPT-2 small's widths, a request of 950 tokens: whole (one workgroup a
+    token and head walks four splits of 256 keys), in portions, and its last tokens one by one
+    (the splits launched side by side) give the same bits, and the plain implementation's
+    logits within the 32-bit tolerance."""
+    from liyab_amd.engine import EngineCore
+
+    d, cfg = small_widths_model
+    config, tensors = plain.read_model(d)
+    reqs = {"f0": tt.random_tokens(700, 950, cfg["vocab_size"]), "f1": tt.random_tokens(701, 40, cfg["vocab_size"])}
+    sparse = lambda steps: [dict(s, entries=[(r, t, w[-4:]) for r, t, w in s["entries"]]) for s in steps]  # noqa: E731
+    runs = {}
+    for label, steps in (("whole", sparse(tt.schedule_whole(reqs))), ("tail", sparse(tt.schedule_bulk_tail(reqs, tail=6))),
+                         ("mixed", sparse(tt.schedule_mixed(reqs, seed=1, decode_tail=5, portions=(300, 9, 48))))):
+        core = EngineCore(d, dtype="float32", page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4)
+        runs[label] = tt.run_schedule(core, steps)
+        del core
+    refs = {rid: plain.forward(config, tensors, t) for rid, t in reqs.items()}
+    tt.check_against_plain(runs["whole"], reqs, refs, TOL["float32"], "float32, 950 tokens whole", family="sizes:small")
+    for label in ("tail", "mixed"):
+        tt.check_against_plain(runs[label], reqs, refs, TOL["float32"], f"float32, 950 tokens {label}", family="sizes:small")
+        for rid in reqs:
+            for p in set(runs[label][rid]) & set(runs["whole"][rid]):
+                assert np.array_equal(runs[label][rid][p], runs["whole"][rid][p]), f"{label}: request {rid} position {p}: other bits than whole"
+    assert set(runs["tail"]["f0"]) & set(runs["whole"]["f0"]) >= {946, 949}
 
 
 @pytest.mark.parametrize("overlap", [False, True])
@@ -348,6 +379,58 @@ def test_contexts_of_thousands_of_positions(dtype, tmp_path):
         tt.check_against_plain(got, reqs, refs, TOL[dtype], f"4,100 positions {label} {dtype}", family="long context")
         core.manager.check()
         del core
+
+
+@pytest.fixture(scope="module")
+def positions_16640_model(tmp_path_factory):
+    """A one-layer GPT-2 with 16,640 positions and its plain logits for one request that fills them
+    and one short one (the plain attention takes a while at this length: made once)."""
+    from liyab_amd.weights import write_random_model
+
+    d = str(tmp_path_factory.mktemp("positions16640"))
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 1, "n_embd": 32, "n_head": 2, "n_inner": 48, "vocab_size": 120,
+           "n_positions": 16640, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    write_random_model(d, cfg, 77)
+    config, tensors = plain.read_model(d)
+    reqs = {"deep": tt.random_tokens(5, 16640, 120), "short": tt.random_tokens(6, 300, 120)}
+    refs = {}
+    for dtype in DTYPES:
+        weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+        refs[dtype] = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+    return d, reqs, refs
+
+
+@pytest.mark.parametrize("mode,page_size", [("float32", 16), ("bfloat16", 16), ("bfloat16 batch-invariant", 16), ("float32", 8), ("bfloat16", 8)])
+def test_contexts_past_16384_keys_and_tables_past_2048_pages(mode, page_size, positions_16640_model):
+    """16,640 positions: past 16,384 keys the splits by position of the 32-bit path and of the
+    batch-invariant mode are longer than 256 keys, so that sixteen of them still cover a request
+    (a step of many tokens walks them in one workgroup, the last tokens are launched in splits);
+    with pages of 8 a request's block table holds 2,080 pages, more than the fast attention
+    kernels stage, and every step takes the plain kernel. A long request in portions of up to
+    2,048 tokens with its last tokens one by one beside a short request's, against the plain
+    implementation."""
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.kernels import ops
+
+    assert ops.invariant_chunk(16640) == 2048 and ops.invariant_chunk(1024) == 256 and ops.invariant_chunk(4097) == 512
+    d, reqs, refs = positions_16640_model
+    dtype = mode.split()[0]
+    deep, short = reqs["deep"], reqs["short"]
+    steps, at = [], 0
+    for n in (2048, 2048, 1500, 2048, 2048, 2048, 2048, 2048, 700):  # 16,636; the last four one by one
+        steps.append({"entries": [("deep", deep[at:at + n], [n - 2, n - 1])], "end": []})
+        at += n
+    steps.append({"entries": [("short", short[:296], [0, 295])], "end": []})
+    for i in range(4):
+        steps.append({"entries": [("deep", deep[at + i:at + i + 1], [0]), ("short", short[296 + i:297 + i], [0])],
+                      "end": ["deep", "short"] if i == 3 else []})
+    core = EngineCore(d, dtype=dtype, page_size=page_size, max_tokens=tt.max_live_tokens(steps), max_requests=2,
+                      batch_invariant="invariant" in mode)
+    assert core.manager.max_blocks == 16640 // page_size
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, refs[dtype], TOL[dtype], f"16,640 positions, pages of {page_size}, {mode}", family="long context")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
 
 
 # ---------------------------------------------------------------------------

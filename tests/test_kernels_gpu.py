@@ -417,6 +417,9 @@ ATT_CASES = [
     ([90, 31], [1, 1], 2, 2, 256, 16),
     ([50, 3], [4, 3], 3, 3, 80, 4),
     ([300, 40, 90], [8, 8, 8], 4, 2, 64, 16),
+    # pages that are no power of two: page and offset by division
+    ([130, 24, 49], [3, 1, 8], 3, 3, 32, 24),
+    ([200, 97], [1, 5], 4, 2, 64, 48),
 ]
 
 
@@ -498,7 +501,7 @@ def test_attention_splits_by_position(ops, case_id, dtype, window):
 @pytest.mark.parametrize("waves", [4, 16])
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("splits", [2, 4, 7, 8])
-@pytest.mark.parametrize("case_id", [0, 1, 2, 3, 5, 6, 7])
+@pytest.mark.parametrize("case_id", [0, 1, 2, 3, 5, 6, 7, 8, 9])
 def test_attention_splits_merged_by_the_projection(ops, case_id, splits, window, waves):
     """Attention that leaves each (token, head) pair's keys in splits, and the projection cut
     over its inner dimension that merges them as it loads them: the planes add up to rows +
@@ -579,6 +582,9 @@ PREFILL_CASES = [
     ([300], [300], 2, 1, 128, 16),
     ([90, 31], [31, 9], 2, 2, 80, 16),
     ([1024], [1024], 1, 1, 64, 16),
+    # pages that are no power of two
+    ([130, 24, 49], [100, 24, 40], 3, 3, 32, 24),
+    ([400, 97], [200, 97], 4, 2, 64, 48),
 ]
 
 
@@ -594,6 +600,112 @@ def test_attention_prefill(ops, case_id, window, tile, ksplit):
     out = run_attention(ops, case, H, hd, scale, window, "prefill", splits=tile, ksplit=ksplit)
     assert torch.isfinite(out.float()).all()
     close(out, attention_reference(case, H, Hkv, hd, scale, window), 8e-3, "prefill")
+
+
+def reference_from_pages(case, kc, vc, bt, H, Hkv, hd, page, scale, window=0):
+    """The plain formula over whatever pages a block table names (float64)."""
+    out = torch.zeros(case["n"], H * hd, dtype=torch.float64)
+    for t, (s, p) in enumerate(zip(case["tok_seq"], case["tok_pos"])):
+        first = max(0, p - window + 1) if window > 0 else 0
+        pos = torch.arange(first, p + 1)
+        pages, offs = bt[s, pos // page].long(), pos % page
+        for h in range(H):
+            hk = h // (H // Hkv)
+            k, v = kc[pages, hk, offs].double(), vc[pages, hk, offs].double()
+            w = torch.softmax((k @ case["q"][t, h * hd:(h + 1) * hd].double()) * scale, dim=0)
+            out[t, h * hd:(h + 1) * hd] = w @ v
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("kernel", ["generic", "decode", "decode in splits", "prefill"])
+def test_a_page_id_past_the_counted_pages_is_not_followed(ops, kernel, dtype):
+    """The caches hold eight pages more than the launcher is told of, and block tables name ids
+    in that slack (and a -1 in a place that is read): told the count, a kernel reads the last
+    counted page instead; told of all pages it reads the slack page. Either way every fetch
+    stays inside the caches: an id that a table should never hold costs a wrong number, not
+    the machine."""
+    if kernel == "prefill" and dtype != torch.bfloat16:
+        pytest.skip("the tiled kernel is bfloat16 only")
+    ctx_lens, q_lens, H, Hkv, hd, page = ([300, 70], [9, 40], 4, 2, 64, 16) if kernel == "prefill" else ([300, 70], [3, 1], 4, 2, 64, 16)
+    case = paged_case(len(ctx_lens), ctx_lens, q_lens, H, Hkv, hd, page, dtype, seed=11)
+    counted = case["kc"].shape[0]
+    g = torch.Generator().manual_seed(5)
+    kc = torch.cat([torch.nan_to_num(case["kc"].float(), nan=0.5), torch.randn(8, Hkv, page, hd, generator=g)]).to(dtype)
+    vc = torch.cat([torch.nan_to_num(case["vc"].float(), nan=-0.5), torch.randn(8, Hkv, page, hd, generator=g)]).to(dtype)
+    bt = case["bt"].clone()
+    bt[0, 2], bt[0, 7], bt[1, 1] = counted + 3, counted + 7, -1
+    case = dict(case, kc=kc, vc=vc, bt=bt)
+    scale = 0.7 / math.sqrt(hd)
+    tol = 8e-3 if dtype == torch.bfloat16 else 2e-6
+
+    def run(num_pages):
+        dev = lambda x: x.to(DEV)  # noqa: E731
+        q = dev(case["q"])[:, :H * hd]
+        tok_seq = torch.tensor(case["tok_seq"], dtype=torch.int32, device=DEV)
+        tok_pos = torch.tensor(case["tok_pos"], dtype=torch.int32, device=DEV)
+        out = torch.zeros(case["n"], H * hd, dtype=dtype, device=DEV)
+        kw = dict(n_head=H, scale=scale, num_pages=num_pages)
+        if kernel == "generic":
+            ops.attention_generic(out, q, dev(kc), dev(vc), dev(bt), tok_seq, tok_pos, **kw)
+        elif kernel == "prefill":
+            work = torch.tensor([0, 0, ctx_lens[0] - q_lens[0], q_lens[0], 1, q_lens[0], ctx_lens[1] - q_lens[1], q_lens[1]],
+                                dtype=torch.int32, device=DEV)
+            ops.attention_prefill(out, q, dev(kc), dev(vc), dev(bt), work, 2, tile=64, **kw)
+        else:
+            splits = 3 if kernel == "decode in splits" else 1
+            partials = torch.empty(case["n"] * H * splits * (hd + 4), device=DEV) if splits > 1 else None
+            ops.attention_decode(out, q, dev(kc), dev(vc), dev(bt), tok_seq, tok_pos, n_splits=splits, partials=partials, **kw)
+        assert torch.isfinite(out.float()).all()
+        return out
+
+    told = run(counted)
+    close(told, reference_from_pages(case, kc, vc, bt.clamp(0, counted - 1), H, Hkv, hd, page, scale), tol, "ids brought into the counted pages")
+    whole = run(None)
+    close(whole, reference_from_pages(case, kc, vc, bt.clamp(0, counted + 7), H, Hkv, hd, page, scale), tol, "every page counted")
+    assert not torch.equal(told, whole)
+    with pytest.raises(Exception, match="pages"):
+        run(counted + 9)
+
+
+@pytest.mark.parametrize("kernel", ["kv_write", "skinny", "dl", "mfma", "folded norm"])
+def test_a_slot_past_the_counted_pages_is_not_written(ops, kernel):
+    """Slots in the eight pages the launcher is not told of (and a -1) are skipped; told of all
+    pages, the same call writes them."""
+    M, H, Hkv, hd, K, page = 24, 3, 3, 32, 128, 8
+    q_dim, kv_dim = H * hd, Hkv * hd
+    N = q_dim + 2 * kv_dim
+    counted = 6
+    a, w, bias = rnd(M, K, dtype=torch.bfloat16), rnd(N, K, seed=1, scale=0.2, dtype=torch.bfloat16), rnd(N, seed=2)
+    slots = torch.randperm(counted * page)[:M].to(torch.int32)
+    slots[3], slots[10], slots[17] = counted * page, (counted + 8) * page - 1, -1
+    slots = slots.to(DEV)
+
+    def run(num_pages):
+        kc = torch.zeros(counted + 8, Hkv, page, hd, dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros_like(kc)
+        q = torch.zeros(M, q_dim, dtype=torch.bfloat16, device=DEV)
+        kw = dict(out=q, epilogue=ops.EPI_QKV_PAGED, kv=(kc, vc, slots, q_dim, num_pages))
+        if kernel == "kv_write":
+            full = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            ops.gemm_simple(a, w, bias, out=full)
+            ops.kv_write(kc, vc, full, q_dim, q_dim + kv_dim, slots, num_pages=num_pages)
+        elif kernel == "skinny":
+            ops.gemm_skinny(a, w, bias, **kw)
+        elif kernel == "dl":
+            ops.gemm_mfma_dl(a, w, bias, tile=2, **kw)
+        elif kernel == "mfma":
+            ops.gemm_mfma(a, w, bias, tile=2, **kw)
+        else:
+            x = rnd(M, K, scale=2.0, seed=4)
+            ops.gemm_skinny_ln(x, rnd(K, seed=5) + 1.0, rnd(K, seed=6), 1e-5, w, bias, **kw)
+        return kc, vc
+
+    for num_pages, written in ((counted, M - 3), (None, M - 1)):
+        kc, vc = run(num_pages)
+        for c in (kc, vc):
+            assert (c[:counted] != 0).any(dim=(1, 3)).sum().item() == M - 3  # the tokens with a slot in the counted pages
+            assert (c != 0).any(dim=(1, 3)).sum().item() == written
 
 
 @pytest.mark.parametrize("T,targets", [(700, [0, 15, 16, 31, 32, 255, 256, 511, 559, 560, 561, 600, 640, 687, 698, 699]),
@@ -813,7 +925,8 @@ def test_tiles_of_every_shape_give_a_row_the_same_bits(ops, K):
 
 
 @pytest.mark.parametrize("kernel", ["skinny", "mfma128", "mfma64", "dl2", "dl8", "dl15", "dl16", "auto"])
-@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64), (700, 6, 3, 64, 128, 16)])
+@pytest.mark.parametrize("M,H,Hkv,hd,K,page", [(5, 3, 3, 16, 64, 4), (40, 4, 2, 32, 128, 16), (200, 5, 5, 48, 192, 8), (130, 2, 1, 64, 64, 64), (700, 6, 3, 64, 128, 16),
+                                               (50, 3, 3, 32, 128, 24), (300, 4, 2, 64, 192, 48)])
 def test_gemm_paged_qkv_epilogue(ops, kernel, M, H, Hkv, hd, K, page):
     """Queries to a dense buffer, keys and values straight into shuffled cache slots, against
     the plain product followed by the scatter kernel."""

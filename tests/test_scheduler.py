@@ -92,6 +92,48 @@ def test_admission_first_come_first_served_and_slots():
     assert all(r.generated == alone(r.prompt, 4) for r in rs)
 
 
+def test_admission_by_priority_then_first_come_first_served():
+    """Among waiting requests the higher priority is admitted first, equals in order of arrival
+    (the reference lets foreground requests go before background ones, src/core/engine.cpp:1936-1945);
+    a preempted request waits ahead of its equals but behind a higher priority."""
+    def one_step(m, s):
+        batch = s.schedule()
+        m.reserve([(b.request.rid, b.first + b.count) for b in batch])
+        for b in batch:
+            m.commit(b.request.rid, b.first + b.count)
+        s.update(batch, {b.request.rid: 9 for b in batch if b.wants_logits})
+        m.check()
+        return [b.request.rid for b in batch]
+
+    m, s = setup(max_num_seqs=1)
+    for rid, pr in (("a", 0), ("b", 0), ("c", 2), ("d", -1), ("e", 2), ("f", 0)):
+        s.add(Request(rid, [1, 2, 3], SamplingParams(temperature=0, max_tokens=1), priority=pr))
+    assert [r.rid for r in s.waiting] == ["c", "e", "a", "b", "f", "d"]
+    order = []
+    while s.has_unfinished():
+        order += one_step(m, s)
+    assert order == ["c", "e", "a", "b", "f", "d"]
+    # two requests that cannot both grow to their end in 4 pages: the later one is preempted and
+    # waits ahead of its equal, behind the higher priority
+    m, s = setup(num_pages=4, max_num_seqs=2)
+    first = Request("first", [1] * 30, SamplingParams(temperature=0, max_tokens=30))
+    second = Request("second", [1] * 30, SamplingParams(temperature=0, max_tokens=30))
+    s.add(first)
+    s.add(second)
+    one_step(m, s)
+    s.add(Request("equal", [1] * 5, SamplingParams(temperature=0, max_tokens=2)))
+    s.add(Request("urgent", [1] * 5, SamplingParams(temperature=0, max_tokens=2), priority=1))
+    s.add(Request("later", [1] * 5, SamplingParams(temperature=0, max_tokens=2), priority=-3))
+    assert [r.rid for r in s.waiting] == ["urgent", "equal", "later"]
+    while second.preemptions == 0:
+        one_step(m, s)
+    # (the step that preempted it admitted the urgent one into the slot it left)
+    assert [r.rid for r in s.waiting] == ["second", "equal", "later"] and [r.rid for r in s.running] == ["first", "urgent"]
+    while s.has_unfinished():
+        one_step(m, s)
+    assert len(second.generated) == 30 and len(first.generated) == 30 and m.pages_in_use() == 0
+
+
 def test_stops_at_eos_and_at_the_last_position():
     m, s = setup(max_positions=32, eos=next_token(Request("p", [5, 6, 7], SamplingParams())))
     r = Request("a", [5, 6, 7], SamplingParams(temperature=0, max_tokens=10))
@@ -285,7 +327,7 @@ def test_native_scheduler_decides_as_the_plain_one(seed, lagged):
     arrivals = []
     for i in range(rng.randint(4, 9)):
         n = rng.randint(1, min(60, num_pages * page_size - 1))
-        arrivals.append((rng.randint(0, 25), f"q{i}", [rng.randrange(90) for _ in range(n)], rng.randint(1, 40)))
+        arrivals.append((rng.randint(0, 25), f"q{i}", [rng.randrange(90) for _ in range(n)], rng.randint(1, 40), rng.choice([0, 0, 0, 1, -1, 5])))
     eos = rng.choice([None, 7, 50])
 
     def drive(native):
@@ -306,8 +348,8 @@ def test_native_scheduler_decides_as_the_plain_one(seed, lagged):
 
         while s.has_unfinished() or inflight is not None or pending:
             while pending and pending[0][0] <= step:
-                _, rid, prompt, max_tokens = pending.pop(0)
-                r = make(rid, list(prompt), SamplingParams(temperature=0, max_tokens=max_tokens))
+                _, rid, prompt, max_tokens, priority = pending.pop(0)
+                r = make(rid, list(prompt), SamplingParams(temperature=0, max_tokens=max_tokens), priority=priority)
                 try:
                     s.add(r)
                     reqs.append(r)

@@ -94,6 +94,11 @@ def max_live_tokens(steps, round_to=64):
     return most
 
 
+def max_live_pages(steps, page_size):
+    """The most pages of `page_size` positions that live requests hold at any time."""
+    return max_live_tokens(steps, round_to=page_size) // page_size
+
+
 def run_schedule(core, steps):
     """Drives an EngineCore through `steps`; returns {rid: {position: float32 logits row}}."""
     from liyab_amd.engine import StepItem
