@@ -68,12 +68,13 @@ def prefill_flops(cfg, prompt_lens, logit_rows):
     return flops + 2.0 * logit_rows * d * V
 
 
-def make_engine(model_dir, dtype, batch, ctx, page_size=64, prefill_chunk=1024, batch_invariant=False):
+def make_engine(model_dir, dtype, batch, ctx, page_size=64, prefill_chunk=1024, batch_invariant=False, phases=False):
     from liyab_amd import Engine
 
     pages = batch * (-(-ctx // page_size)) + 4
     return Engine(model_dir, dtype=dtype, page_size=page_size, num_pages=pages, max_num_seqs=max(batch, 2),
-                  max_batched_tokens=max(2048, batch), prefill_chunk=prefill_chunk, ctx=ctx, batch_invariant=batch_invariant)
+                  max_batched_tokens=max(2048, batch), prefill_chunk=prefill_chunk, ctx=ctx, batch_invariant=batch_invariant,
+                  phases=phases)
 
 
 def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
@@ -104,10 +105,10 @@ def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
     elt = 2 if engine.core.dtype == torch.bfloat16 else 4
     # each timed step s reads the cache of positions [0, context + s] of every request
     kv_positions = sum(c * steps + steps * (steps + 1) // 2 for c in contexts)
-    bytes_per_step = weight_bytes(cfg, elt) + kv_positions * kv_bytes_per_position(cfg, elt) / steps
+    bytes_per_step = weight_bytes(cfg, elt) + kv_positions * kv_bytes_per_position(cfg, elt) / max(steps, 1)
     for r in list(engine.scheduler.running):
         engine.abort(r.rid)
-    return batch * steps / dt, dt * 1e3 / steps, bytes_per_step
+    return batch * steps / dt, dt * 1e3 / max(steps, 1), bytes_per_step
 
 
 def workload_run(engine, cfg, prompts, params_of, label):
@@ -318,6 +319,8 @@ def main():
     ap.add_argument("--batch-invariant", action="store_true", help="kernels chosen from sizes and positions only (reproducible bfloat16 replies)")
     ap.add_argument("--product", default="", help="M,N,K[,tile,...]: time one bfloat16 product in the tiled kernel's tiles (0: its own choice, 6: 64 x 64, 8: 128 x 128, 15: 256 x 256)")
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
+    ap.add_argument("--phases", action="store_true", help="device milliseconds per phase of the forward pass (embed, attention, dense_ffn, lm_head) a decode step "
+                    "and a prefill of 2,048 tokens, as the reference's command line prints them (tools/liyab_cli.cpp:198-211); steps run kernel by kernel, without graphs")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -356,7 +359,7 @@ def main():
 
             layers_note = {"n_layer": cfg["n_layer"], "n_layer_full": full_layers}
             if args.workload == "medium16":
-                # BASELINE's workload for GPT-2 medium's sizes: 16 requests, prompt lengths uniform in [64, 1024) and ids
+                # the continuous-batching workload at GPT-2 medium's sizes: 16 requests, prompt lengths uniform in [64, 1024) and ids
                 # from seed 21, continuously batched with portions of 256, 128 greedy tokens each (capped at the positions)
                 rng = np.random.default_rng(21)
                 lens = rng.integers(64, 1024, 16).tolist()
@@ -370,7 +373,7 @@ def main():
                                   "dtype": short, "data": "synthetic", "page_size": args.page_size, **layers_note,
                                   "prompt_lens": lens, "runs": runs}))
             else:
-                # BASELINE's workload for GPT-2 XL's sizes: 64 requests, prompts of 256 ids from seed 31, decoding to 1,024
+                # the batch-64 workload at GPT-2 XL's sizes: 64 requests, prompts of 256 ids from seed 31, decoding to 1,024
                 # positions, greedy and at temperature 1
                 rng = np.random.default_rng(31)
                 prompts = [rng.integers(0, cfg["vocab_size"], 256).tolist() for _ in range(64)]
@@ -397,6 +400,25 @@ def main():
             return 0
         if args.sequences:
             print(json.dumps(sequences_run(engine, cfg, [int(x) for x in args.sequences.split(",")], args.prompt, args.n)))
+            return 0
+        if args.phases:
+            timed = make_engine(d, args.dtype, max(args.batch, 2), ctx, page_size=args.page_size, batch_invariant=args.batch_invariant, phases=True)
+            k = min(steps, 64)
+            decode_run(timed, cfg, args.batch, args.prompt, 4, 2)  # every kernel has run once
+            timed.phases_ms(reset=True)
+            tps, ms, _ = decode_run(timed, cfg, args.batch, args.prompt, k, 0, seed=12)
+            whole = timed.phases_ms(reset=True)  # the prompts of the run, too: taken off below
+            prefill_run(timed, cfg, [1024, 1024], repeat=1)
+            prefill = timed.phases_ms(reset=True)
+            per = lambda table, n: {name: round(v / n, 4) for name, v in table.items()}  # noqa: E731
+            # the prompts of the decode run went through the same timer: one step of `batch` prompts of args.prompt tokens
+            timed.phases_ms(reset=True)
+            decode_run(timed, cfg, args.batch, args.prompt, 0, 0, seed=12)
+            prompts_only = timed.phases_ms(reset=True)
+            decode = {name: max(whole.get(name, 0.0) - prompts_only.get(name, 0.0), 0.0) for name in whole}
+            print(json.dumps({"metric": f"device ms per phase (GPT-2 {args.size} sizes, {short}; steps launched kernel by kernel)",
+                              "decode_step": {"batch": args.batch, "steps": k, "phases_ms": per(decode, k), "ms_per_step_wall": round(ms, 4)},
+                              "prefill_2048": {"phases_ms": per(prefill, 3)}}))
             return 0
         if args.prefill_only:
             ptps, pms = prefill_run(engine, cfg, [1024, 1024], repeat=20)
