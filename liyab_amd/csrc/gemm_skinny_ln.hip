@@ -151,10 +151,15 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
     // that every wave runs the same loads). Its loads go first and the wave's share of the weights
     // and its bias right after: counted in order, a wait for the row does not wait for the weights,
     // which come from further away and arrive while the norm is computed.
-    norm_row(min(wave, M - 1), wave < M, [&]() {
+    auto ask_weights = [&]() {
         load_w(wave * 2, wc);
         e_bias = (e_mine && epi.bias != nullptr) ? epi.bias[e_n] : 0.0f;
-    });
+    };
+    // (a wave past the last row asks for its weights only: a compute unit takes 64 bytes a cycle from
+    // its cache, and eight waves that each ask for a row in four planes and the norm's two vectors
+    // are 147 KB, six times the workgroup's weights)
+    if (wave < M) norm_row(wave, true, ask_weights);
+    else ask_weights();
     for (int m = wave + LN_WAVES; m < M; m += LN_WAVES) norm_row(m, true, []() {});
     lds_barrier();  // the weights may still be on their way
 
