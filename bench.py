@@ -260,6 +260,40 @@ def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
     return n / best, best * 1e3
 
 
+def ttft_run(engine, cfg, prompt_len=512, repeat=6, seed=14):
+    """An idle engine and one prompt, each time of a length the engine has not seen (so that the
+    step is launched kernel by kernel, not replayed from a graph): milliseconds until step() has
+    launched everything (the host's share), the step's kernels on the device (events around it),
+    and until the first token is on the host. Best of `repeat`."""
+    import numpy as np
+    import torch
+
+    from liyab_amd import SamplingParams
+
+    rng = np.random.default_rng(seed)
+    engine.stop_at_eos = False
+    host = device = total = float("inf")
+    for it in range(repeat + 2):
+        prompt = rng.integers(0, cfg["vocab_size"], prompt_len - it).tolist()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        rid = engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=1))
+        e0.record()
+        engine.step()
+        e1.record()
+        t1 = time.perf_counter()
+        while engine.has_unfinished():
+            engine.step()
+        engine.flush()
+        t2 = time.perf_counter()
+        torch.cuda.synchronize()
+        engine.release(rid)
+        if it >= 2:
+            host, device, total = min(host, (t1 - t0) * 1e3), min(device, e0.elapsed_time(e1)), min(total, (t2 - t0) * 1e3)
+    return {"prompt_len": prompt_len, "host_ms": round(host, 4), "device_ms": round(device, 4), "ms": round(total, 4)}
+
+
 def sequences_run(engine, cfg, counts, prompt_len, n_new, seed=13):
     """Several sequences generated together against the same sequences one after the other, as
     the reference's liyab-seq-bench reports them (tools/liyab_seq_bench.cpp:1-32): total tokens
@@ -448,6 +482,7 @@ def main():
             flops = prefill_flops(cfg, lens, len(lens))
             out["prefill"] = {"value": round(ptps, 1), "tokens": sum(lens), "ms": round(pms, 4),
                               "frac": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)}
+            out["ttft"] = ttft_run(engine, cfg, min(args.prompt, ctx - 16))
             # every point over at least 64 steps after at least 3 of its own shape, whatever --steps says: fewer do
             # not outlast the first sight of a shape (an eager run, then a capture)
             points = {}

@@ -18,6 +18,7 @@
 // (more splits when few tokens are in flight), which moves results by
 // rounding only. Scores, exponentials and sums are 32-bit.
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

@@ -13,6 +13,7 @@
 // read at the cache's precision. It serves the true 32-bit path and any
 // head size up to 256 on the bfloat16 path.
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

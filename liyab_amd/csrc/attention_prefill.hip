@@ -32,6 +32,7 @@
 // other, so their chains overlap, and the streams are merged once at the end (in registers, then
 // the KS partial results as before).
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

@@ -6,6 +6,7 @@
 // over the row. The sum is formed in 32-bit and the residual stream it
 // starts is 32-bit on both paths.
 #include "common.h"
+#include "launchers.h"
 
 #include <algorithm>
 

@@ -12,6 +12,7 @@
 // store; K must be a multiple of 8 (16-byte pieces). Each output element is
 // a fixed-order sum over k, independent of M.
 #include "common.h"
+#include "launchers.h"
 #include "epilogue.h"
 
 namespace liyab {

@@ -19,6 +19,7 @@
 // leaves it (gemm_skinny.hip). A product with few output tiles and a long K
 // covers the chip that way.
 #include "common.h"
+#include "launchers.h"
 #include "epilogue.h"
 
 #include <type_traits>

@@ -14,6 +14,7 @@
 // element's sum over several waves: gemm_rowwise_f32_kernel below.)
 #include "activations.h"
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

@@ -20,6 +20,7 @@
 // plane of 32-bit sums; the first plane may take the bias and the rows the product is to be
 // added to (themselves a sum of planes), so that the planes together are the new rows.
 #include "common.h"
+#include "launchers.h"
 #include "epilogue.h"
 
 namespace liyab {

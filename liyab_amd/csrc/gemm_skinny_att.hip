@@ -13,6 +13,7 @@
 // from further away). The sums go to one plane a part, the first plane also taking the bias
 // and the rows of the residual stream the product is added to, as in the plain cut product.
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

@@ -18,6 +18,7 @@
 // the norm overlap. Every workgroup repeats the norm: it pays while the rows
 // are few (M * K * planes * 4 bytes from L2 a workgroup).
 #include "common.h"
+#include "launchers.h"
 #include "epilogue.h"
 
 namespace liyab {

@@ -13,6 +13,7 @@
 // and the norm that reads the residual stream next adds the planes up, in their order, as it
 // loads a row.
 #include "common.h"
+#include "launchers.h"
 
 namespace liyab {
 

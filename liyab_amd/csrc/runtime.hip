@@ -1,5 +1,6 @@
 // Error reporting shared by every launcher, and small utility kernels.
 #include "common.h"
+#include "launchers.h"
 
 #include <cstring>
 

@@ -9,6 +9,7 @@ on first use when it is not there.
 from __future__ import annotations
 
 import ctypes
+import struct
 import sys
 from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_uint32, c_void_p
 from typing import Optional
@@ -32,6 +33,8 @@ class EpiParams(ctypes.Structure):
     ]
 
 
+_EPI_PTR = ctypes.POINTER(EpiParams)
+
 _SIGNATURES = {
     "liyab_check_device": [],
     "liyab_fill": [P, c_int, c_uint32, c_int64, P],
@@ -46,17 +49,17 @@ _SIGNATURES = {
     "liyab_sum_parts": [P, c_int, c_int, P, c_int, c_int64, P],
     "liyab_gemm_skinny_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
     "liyab_gemm_simple": [P, c_int, c_int64, P, c_int64, P, c_int, P, P, c_int64, c_int, c_int, c_int, c_int, P],
-    "liyab_gemm_mfma": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
-    "liyab_gemm_mfma_dl": [P, c_int64, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_mfma": [P, c_int64, P, c_int, c_int, c_int, c_int, _EPI_PTR, P],
+    "liyab_gemm_mfma_dl": [P, c_int64, P, c_int, c_int, c_int, c_int, _EPI_PTR, P],
     "liyab_gemm_mfma_dl_parts": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
-    "liyab_gemm_skinny": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_skinny": [P, c_int64, P, c_int, c_int, c_int, c_int, c_int, c_int, _EPI_PTR, P],
     "liyab_attention_generic": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, c_int, P],
     "liyab_attention_decode": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, P],
     "liyab_attention_merge": [P, c_int, c_int64, P, c_int, c_int, c_int, c_int, P],
     "liyab_gemm_att_parts": [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, c_int64, P, P, c_int, c_int64, P],
-    "liyab_gemm_skinny_ln": [P, c_int, c_int64, P, P, c_float, P, c_int, c_int, c_int, c_int, ctypes.POINTER(EpiParams), P],
+    "liyab_gemm_skinny_ln": [P, c_int, c_int64, P, P, c_float, P, c_int, c_int, c_int, c_int, _EPI_PTR, P],
     "liyab_attention_prefill": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
                                 c_int, c_int, c_int, c_int, P],
     "liyab_argmax": [P, P, c_int64, c_int, c_int, P, P, P, P, P],
@@ -101,6 +104,13 @@ def load() -> ctypes.CDLL:
             raise KernelError(f"'{path}' lacks the entry point {name}: rebuild it (python -m liyab_amd.csrc.build)")
         fn.restype = c_int
         fn.argtypes = args
+    for name, args in (("liyab_replay_index", [c_char_p, ctypes.POINTER(c_int)]),
+                       ("liyab_replay", [ctypes.POINTER(ctypes.c_uint64), c_int64])):
+        fn = getattr(lib, name, None)
+        if fn is None:
+            raise KernelError(f"'{path}' lacks the entry point {name}: rebuild it (python -m liyab_amd.csrc.build)")
+        fn.restype = c_int
+        fn.argtypes = args
     _lib, _path = lib, path
     return lib
 
@@ -110,3 +120,82 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(f"{name}: {lib.liyab_last_error().decode('utf-8', 'replace')}")
+    if _recording is not None:
+        _record(name, args)
+
+
+# -- a list of launches, recorded once and run again natively with other tensors ----------------
+_recording: Optional[list] = None  # the words of the list being recorded, or None
+_recording_whole = True  # whether every launch so far could be written down
+_entries: dict = {}  # launcher name -> (index in the native table, encoders of its arguments)
+BLOCK_ARG = 0xB10CB10CB10CB10C  # stands for the argument that points at an epilogue's parameter block (csrc/replay.hip)
+_U64 = (1 << 64) - 1
+
+
+def _encoders(name: str):
+    """(index, [how each argument becomes a 64-bit word]) of a launcher the native replay knows,
+    or None for one it does not."""
+    hit = _entries.get(name)
+    if hit is None:
+        lib = load()
+        n = c_int(0)
+        index = lib.liyab_replay_index(name.encode(), ctypes.byref(n))
+        kinds = []
+        for t in _SIGNATURES[name]:
+            kinds.append("block" if t is _EPI_PTR else ("float" if t is c_float else ("double" if t is c_double else "int")))
+        hit = _entries[name] = (index, kinds) if index >= 0 and n.value == len(kinds) and "double" not in kinds else (-1, kinds)
+    return hit
+
+
+def _record(name: str, args) -> None:
+    global _recording_whole
+    index, kinds = _encoders(name)
+    if index < 0:
+        _recording_whole = False  # a launcher the native replay does not know: the list is of no use
+        return
+    words = [index, len(args)]
+    block = ()
+    for kind, a in zip(kinds, args):
+        if kind == "int":
+            words.append((0 if a is None else int(a)) & _U64)
+        elif kind == "float":
+            words.append(struct.unpack("<I", struct.pack("<f", a))[0])
+        else:
+            raw = bytes(a._obj)  # (the argument is ctypes.byref(params))
+            raw += b"\0" * (-len(raw) % 8)
+            block = struct.unpack(f"<{len(raw) // 8}Q", raw)
+            words.append(BLOCK_ARG)
+    words.append(len(block))
+    words.extend(block)
+    _recording.extend(words)
+
+
+class recording:
+    """Within this context every launch is also written down; `words` holds the list afterwards
+    (a numpy array of uint64, see csrc/replay.hip), or None if a launcher ran that the native
+    replay does not know."""
+
+    def __enter__(self):
+        global _recording, _recording_whole
+        if _recording is not None:
+            raise KernelError("a list of launches is being recorded already")
+        _recording, _recording_whole = [], True
+        self.words = None
+        return self
+
+    def __exit__(self, exc_type, *exc):
+        global _recording
+        import numpy as np
+
+        words, _recording = _recording, None
+        if exc_type is None and _recording_whole:
+            self.words = np.array(words, dtype=np.uint64)
+        return False
+
+
+def replay(words) -> None:
+    """Runs a recorded list of launches (a contiguous numpy array of uint64) again."""
+    lib = load()
+    rc = lib.liyab_replay(words.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)), words.size)
+    if rc != 0:
+        raise KernelError(f"replay: {lib.liyab_last_error().decode('utf-8', 'replace')}")

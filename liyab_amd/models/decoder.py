@@ -15,11 +15,95 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
+import bisect
+import dataclasses
+import os
+
+import numpy as np
+
 from ..cache.pages import KVSpec, StateSpec
+from ..kernels import lib as _lib
 from ..kernels import ops
 from ..config.plan import ModelPlan
-from ..parts.base import StepContext
+from ..parts.base import SplitStream, StepContext
 from ..parts.registry import build_part, find_part
+
+
+_OTHER = object()  # stands for "holds something that may not be run from a recorded list"
+
+
+def _describe(obj, tensors: list, seen: set):
+    """What a part is made of, as a hashable key, its tensors appended to `tensors` in the order
+    they are met: two layers with equal keys hold tensors of equal shapes in the same places
+    and equal constants everywhere else. _OTHER if something in it is not `replayable`."""
+    if isinstance(obj, torch.Tensor):
+        tensors.append(obj)
+        return ("tensor", tuple(obj.shape), str(obj.dtype), tuple(obj.stride()))
+    if obj is None or isinstance(obj, (bool, int, float, str)):
+        return obj
+    if isinstance(obj, torch.dtype):
+        return str(obj)
+    if isinstance(obj, (list, tuple)):
+        items = tuple(_describe(v, tensors, seen) for v in obj)
+        return _OTHER if any(i is _OTHER for i in items) else ("seq", items)
+    if isinstance(obj, dict):
+        items = tuple((str(k), _describe(v, tensors, seen)) for k, v in sorted(obj.items(), key=lambda kv: str(kv[0])))
+        return _OTHER if any(i is _OTHER for _, i in items) else ("dict", items)
+    if dataclasses.is_dataclass(obj) and not isinstance(obj, type):
+        # a spec the part was built from: it names this layer's tensors; what the part computes with
+        # it has copied into attributes of its own
+        return ("spec", type(obj).__name__)
+    if not getattr(type(obj), "replayable", False) or id(obj) in seen or not hasattr(obj, "__dict__"):
+        return _OTHER
+    seen.add(id(obj))
+    fields = []
+    for name in sorted(vars(obj)):
+        key = _describe(vars(obj)[name], tensors, seen)
+        if key is _OTHER:
+            return _OTHER
+        fields.append((name, key))
+    return (type(obj).__module__, type(obj).__qualname__, tuple(fields))
+
+
+class _Recorded:
+    """A layer's launches as a list of words, and where in it the addresses of the layer's own
+    tensors stand (any address inside one of them, as an offset from its start)."""
+
+    def __init__(self, words: np.ndarray, bases: np.ndarray, sizes, pending_out):
+        self.words = words
+        self.pending_out = pending_out
+        order = np.argsort(bases)
+        starts = bases[order].tolist()
+        positions, which, offsets = [], [], []
+        self.usable = True
+        for i in range(1, len(starts)):
+            if starts[i] < starts[i - 1] + sizes[order[i - 1]]:
+                self.usable = False  # two of the layer's tensors overlap: an address would name both
+        for at, word in enumerate(words.tolist()):
+            j = bisect.bisect_right(starts, word) - 1
+            if j >= 0 and word < starts[j] + sizes[order[j]]:
+                positions.append(at)
+                which.append(int(order[j]))
+                offsets.append(word - starts[j])
+        self.positions = np.array(positions, dtype=np.int64)
+        self.which = np.array(which, dtype=np.int64)
+        self.offsets = np.array(offsets, dtype=np.uint64)
+
+    def for_layer(self, bases: np.ndarray) -> np.ndarray:
+        words = self.words.copy()
+        words[self.positions] = bases[self.which] + self.offsets
+        return words
+
+
+class _NoRecording:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_no_recording = _NoRecording()
 
 
 class DecoderModel:
@@ -53,6 +137,16 @@ class DecoderModel:
         for e in self.order:
             if not (0 <= e.layer < len(self.blocks)) or not (0 <= e.cache_layer < len(self.blocks)):
                 raise ValueError(f"the run order names layer {e.layer} / cache of {e.cache_layer}; the model has {len(self.blocks)}")
+        # Layers of one kind run from one recorded list of launches (csrc/replay.hip): a layer's kind
+        # is what its block and parts are made of, its tensors aside; layers whose parts are not all
+        # `replayable` run through their Python every time. LIYAB_REPLAY=0 switches it off.
+        self.replay_layers = os.environ.get("LIYAB_REPLAY", "1") != "0"
+        self._layer_kind, self._layer_tensors = [], []
+        for block in self.blocks:
+            tensors: list = []
+            self._layer_kind.append(_describe(block, tensors, set()))
+            self._layer_tensors.append(tensors)
+        self.replayed_layers = 0  # layers that ran from a recorded list, over the model's lifetime
 
     # -- what the cache manager needs to know ---------------------------------
     def cache_groups(self) -> List[Tuple[KVSpec, List[int]]]:
@@ -91,16 +185,34 @@ class DecoderModel:
         if self.residual_position is not None and fused is None:
             self.residual_position.add(ctx, x)
         pending = None  # the stream as a SplitStream while a layer has left it split (x is then stale)
+        recorded = {}  # this step's lists of launches, by the kind of layer and the state it found the stream in
         for e in self.order:
             block = self.blocks[e.layer]
-            args = (x, ctx, storage.layer(e.cache_layer), storage.state(e.cache_layer))
-            if getattr(block, "takes_pending", False):
-                pending = block.forward(*args, writes_cache=e.writes_cache, pending=pending)
-            else:
-                if pending is not None:
-                    pending.settle()
-                    pending = None
-                block.forward(*args, writes_cache=e.writes_cache)
+            cache, state = storage.layer(e.cache_layer), storage.state(e.cache_layer)
+            key = None
+            if self.replay_layers and phases is None and self._layer_kind[e.layer] is not _OTHER:
+                own = self._layer_tensors[e.layer] + (list(cache.rows.values()) if cache is not None else []) + ([state] if state is not None else [])
+                key = (self._layer_kind[e.layer], cache.group if cache is not None else -1,
+                       tuple((tuple(t.shape), str(t.dtype)) for t in own[len(self._layer_tensors[e.layer]):]), e.writes_cache,
+                       None if pending is None else (pending.planes.data_ptr(), tuple(pending.planes.shape)))
+                bases = np.fromiter((t.data_ptr() for t in own), dtype=np.uint64, count=len(own))
+                hit = recorded.get(key)
+                if hit is not None and hit.usable:
+                    _lib.replay(hit.for_layer(bases))
+                    pending = hit.pending_out
+                    self.replayed_layers += 1
+                    continue
+            args = (x, ctx, cache, state)
+            with _lib.recording() if key is not None and key not in recorded else _no_recording as rec:
+                if getattr(block, "takes_pending", False):
+                    pending = block.forward(*args, writes_cache=e.writes_cache, pending=pending)
+                else:
+                    if pending is not None:
+                        pending.settle()
+                        pending = None
+                    block.forward(*args, writes_cache=e.writes_cache)
+            if rec is not None and rec.words is not None and (pending is None or isinstance(pending, SplitStream)):
+                recorded[key] = _Recorded(rec.words, bases, [t.numel() * t.element_size() for t in own], pending)
         if phases is not None:
             phases.mark("lm_head")
             try:

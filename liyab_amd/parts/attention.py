@@ -104,6 +104,10 @@ class Attention:
     and the cache write, where the reference applies its rotary encoding
     (:3113-3116); GPT-2 has none."""
 
+    # every launch goes through the kernel library and depends on nothing of this object but its
+    # tensors and the constants among its attributes: layers of this kind may run from one recorded list
+    replayable = True
+
     def __init__(self, spec, store, dtype: torch.dtype):
         self.spec = spec
         self.dtype = dtype

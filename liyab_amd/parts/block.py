@@ -13,6 +13,10 @@ class PreNormBlock:
     run_block for a sequential pre-norm layer (src/core/transformer.cpp:5514-5726:
     norm :5565-5577, mixer, residual :5647, norm :5663-5666, ffn, residual :5692)."""
 
+    # every launch goes through the kernel library and depends on nothing of this object but its
+    # tensors and the constants among its attributes: layers of this kind may run from one recorded list
+    replayable = True
+
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
         # phases are named after the parts' kinds (the reference's: attention, dense_ffn, ...)

@@ -15,6 +15,10 @@ class DenseFFN:
     src/core/transformer.cpp:4903-4913; residual :5692). `activation` is
     "gelu_tanh" (:123-130) or "gelu_erf" (:134-142)."""
 
+    # every launch goes through the kernel library and depends on nothing of this object but its
+    # tensors and the constants among its attributes: layers of this kind may run from one recorded list
+    replayable = True
+
     def __init__(self, spec, store, dtype: torch.dtype):
         self.dtype = dtype
         self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation

@@ -46,6 +46,10 @@ class LayerNorm:
     (the reference's layernorm, src/core/transformer.cpp:77-106); weight and
     bias are each optional, as there (:1105-1109). Statistics are 32-bit."""
 
+    # every launch goes through the kernel library and depends on nothing of this object but its
+    # tensors and the constants among its attributes: layers of this kind may run from one recorded list
+    replayable = True
+
     def __init__(self, spec, store, dtype: torch.dtype):
         self.width = spec.width
         self.eps = float(spec.eps)

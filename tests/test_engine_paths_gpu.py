@@ -257,6 +257,81 @@ def test_head_sizes_the_kernels_cannot_take_are_refused_at_load(tmp_path):
 
 
 # ---------------------------------------------------------------------------
+# layers of one kind run from one recorded list of launches
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("use_graphs", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layers_run_from_a_recorded_list_give_the_bits_of_their_own_python(dtype, use_graphs, tmp_path):
+    """Five layers of one kind: the second layer's launches are written down as it runs and the
+    third to fifth run from that list with their own weights and pages in place of the second's
+    (the first finds the stream whole, the others split, so it is a kind of its own in
+    bfloat16). Whole prompts, portions, mixed batches and single tokens, eager and under graphs:
+    the logits have the bits of the same engine with every layer run through its Python, and are
+    the plain implementation's."""
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model
+
+    cfg = {"architectures": ["GPT2LMHeadModel"], "n_layer": 5, "n_embd": 128, "n_head": 4, "n_inner": 320, "vocab_size": 700,
+           "n_positions": 300, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    write_random_model(str(tmp_path), cfg, 41)
+    config, tensors = plain.read_model(str(tmp_path))
+    weights = tensors if dtype == "float32" else plain.round_weights_to_bf16(tensors)
+    reqs = {f"l{i}": tt.random_tokens(70 + i, n, 700) for i, n in enumerate([150, 33, 9, 70, 260])}
+    refs = {rid: plain.forward(config, weights, t) for rid, t in reqs.items()}
+    for label, steps in (("whole", tt.schedule_whole(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=6, decode_tail=8)),
+                         ("bulk+tail", tt.schedule_bulk_tail(reqs, tail=9))):
+        runs = {}
+        for replay in (True, False):
+            core = EngineCore(str(tmp_path), dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=8,
+                              use_graphs=use_graphs)
+            core.model.replay_layers = replay
+            runs[replay] = tt.run_schedule(core, steps)
+            if replay:
+                assert core.model.replayed_layers >= 3 * (len(steps) - core.step_fn.graph_replays) - 3, "the layers ran through their Python"
+            else:
+                assert core.model.replayed_layers == 0
+            core.manager.check()
+            del core
+        for rid, toks in reqs.items():
+            for p in range(len(toks)):
+                assert np.array_equal(runs[True][rid][p], runs[False][rid][p]), f"{label}: request {rid} position {p}: other bits from the recorded list"
+        tt.check_against_plain(runs[True], reqs, refs, TOL[dtype], f"recorded layers {label} {dtype}", family="sizes:odd")
+
+
+def test_layers_with_constants_of_their_own_are_not_run_from_anothers_list(model_dirs):
+    """Configuration B scales attention by 1 / (layer + 1): a constant that differs from layer to
+    layer makes every layer a kind of its own, and each runs through its own Python."""
+    from liyab_amd.engine import EngineCore
+
+    for name, replays in (("A", True), ("B", False)):
+        core = EngineCore(model_dirs[name], dtype="float32", page_size=16, max_tokens=256, max_requests=2, use_graphs=False)
+        kinds = core.model._layer_kind
+        assert (kinds[0] == kinds[1]) == replays
+        core.open("r")
+        core.step([tt_item("r", [1, 2, 3, 4, 5], [4])])
+        assert (core.model.replayed_layers > 0) == replays
+
+
+def tt_item(rid, tokens, want):
+    from liyab_amd.engine import StepItem
+
+    return StepItem(rid, tokens, want)
+
+
+def test_a_malformed_list_of_launches_is_refused_before_anything_runs():
+    from liyab_amd.kernels import lib
+
+    lib.load()
+    index, kinds = lib._encoders("liyab_fill")
+    assert index >= 0 and len(kinds) == 5
+    for words, what in (([index, 5, 0, 4, 0, 0], "cut short"), ([9999, 0, 0], "unknown launcher"), ([index, 4, 0, 4, 0, 0, 0], "takes 5 arguments"),
+                        ([index, 5, lib.BLOCK_ARG, 4, 0, 0, 0, 0], "parameter block")):
+        with pytest.raises(Exception, match=what):
+            lib.replay(np.array(words, dtype=np.uint64))
+    lib.replay(np.array([], dtype=np.uint64))
+
+
+# ---------------------------------------------------------------------------
 # bfloat16 replies that do not depend on the batch
 # ---------------------------------------------------------------------------
 @pytest.fixture(scope="module")

@@ -121,3 +121,46 @@ def test_attention_plans_its_own_words_of_a_step():
     assert words[20:].tolist() == [100, 101]
     # the same sizes cut another way give the same key when they fall into the same tiles
     assert planner.plan(facts([90, 2, 80, 9], [10, 40, 190, 5])).key == p.key
+
+
+def test_what_makes_two_layers_one_kind_and_how_a_recorded_list_gets_another_layers_addresses():
+    """Layers run from one recorded list of launches when their blocks are made of the same parts
+    with the same constants (tensors aside) and every part says it is `replayable`; the list's words
+    that lie inside the recorded layer's tensors become the same places of the other layer's."""
+    import numpy as np
+    import torch
+
+    from liyab_amd.models.decoder import _OTHER, _Recorded, _describe
+
+    class Part:
+        replayable = True
+
+        def __init__(self, scale, w):
+            self.scale, self.w, self.names = scale, w, {"b": [w, None]}
+
+    class Block:
+        replayable = True
+
+        def __init__(self, part):
+            self.part, self.label = part, "x"
+
+    class Foreign:
+        def __init__(self):
+            self.t = torch.zeros(2)
+
+    a, b = torch.zeros(4, 3), torch.ones(4, 3)
+    ta, tb, tc = [], [], []
+    ka, kb = _describe(Block(Part(0.5, a)), ta, set()), _describe(Block(Part(0.5, b)), tb, set())
+    assert ka == kb and ka is not _OTHER and [t.data_ptr() for t in ta] == [a.data_ptr()] * 2 and len(tb) == 2
+    assert _describe(Block(Part(0.25, a)), tc, set()) != ka  # a constant of its own
+    assert _describe(Block(Part(0.5, torch.zeros(4, 4))), [], set()) != ka  # another shape
+    assert _describe(Block(Foreign()), [], set()) is _OTHER  # a part that does not say it may be replayed
+    own = Block(Part(0.5, a))
+    own.part.loop = own
+    assert _describe(own, [], set()) is _OTHER  # an object met twice
+    # a list whose words 2 and 5 point into the first and the second tensor of the recorded layer
+    bases = np.array([1000, 5000], dtype=np.uint64)
+    rec = _Recorded(np.array([7, 3, 1000 + 16, 999, 6000, 5000, 1000 + 64], dtype=np.uint64), bases, [64, 100], None)
+    assert rec.usable and rec.positions.tolist() == [2, 5] and rec.offsets.tolist() == [16, 0]
+    assert rec.for_layer(np.array([20000, 90000], dtype=np.uint64)).tolist() == [7, 3, 20016, 999, 6000, 90000, 1064]
+    assert not _Recorded(np.array([1], dtype=np.uint64), np.array([1000, 1032], dtype=np.uint64), [64, 8], None).usable  # overlapping tensors
