@@ -173,6 +173,18 @@ def test_sampler_rules():
     assert plain.uniform(4, 0) != plain.uniform(5, 0)
 
 
+def test_rng_is_splitmix64s_output_function():
+    """Pinned by the generator's published first outputs from state 0 (0xE220A8397B1DCDAF, then
+    0x6E789E6AA1B965F4): (seed 0, index -1) makes the counter 0 and (seed 1, index -1) one
+    increment, so that a wrong constant or shift in either copy of the formula fails."""
+    from liyab_amd.sampling import uniform
+
+    for fn in (plain.uniform, uniform):
+        assert fn(0, -1) == (0xE220A8397B1DCDAF >> 11) / 2.0 ** 53
+        assert fn(1, -1) == (0x6E789E6AA1B965F4 >> 11) / 2.0 ** 53
+        assert fn(0, 0) != fn(0, -1) and 0.0 <= fn(7, 123) < 1.0
+
+
 def test_rng_agrees_with_the_engine():
     from liyab_amd.sampling import uniform
 
