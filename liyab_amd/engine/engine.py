@@ -139,11 +139,16 @@ class Engine:
         served among equals); the reference's foreground and background sequences
         (include/liyab/engine.h:1034, 1088-1091) are two values of it."""
         params = params or SamplingParams()
-        prompt = [int(t) for t in prompt_ids]
+        import numpy as np
+
+        ids = np.asarray(prompt_ids)
+        if ids.ndim != 1 or (ids.size and ids.dtype.kind not in "iu"):
+            raise InvalidArgument("a prompt is a sequence of token ids")
         V = self.core.vocab_size
-        for t in prompt:
-            if not (0 <= t < V):
-                raise InvalidArgument(f"token id {t} is outside [0, {V})")  # src/core/transformer.cpp:6195-6197
+        if ids.size and (int(ids.min()) < 0 or int(ids.max()) >= V):
+            bad = int(ids[(ids < 0) | (ids >= V)][0])
+            raise InvalidArgument(f"token id {bad} is outside [0, {V})")  # src/core/transformer.cpp:6195-6197
+        prompt = ids.tolist()
         if rid is None:
             rid = f"req-{self._next_id}"
             self._next_id += 1
