@@ -221,16 +221,17 @@ class Engine:
         host = event = None
         if wanting:
             ctx = self.core.step_fn.last_context
-            out = self.sampler.sample_on_device(
-                logits, [r.params for r in wanting], [r.seed for r in wanting],
-                [len(r.generated) + r.pending for r in wanting],
-                scatter=(ctx.logit_slots, ctx.last_tokens))
             host = self._host_tokens[self._turn]
             if host is None or host.numel() < len(wanting):
                 host = self._host_tokens[self._turn] = torch.empty(max(64, 2 * len(wanting)), dtype=torch.int32,
                                                                    pin_memory=True)
             self._turn ^= 1
-            host[:len(wanting)].copy_(out, non_blocking=True)
+            # the sampling kernel writes the tokens into pinned host memory itself (and into the device's
+            # table of last tokens): no copy follows it on the stream
+            self.sampler.sample_on_device(
+                logits, [r.params for r in wanting], [r.seed for r in wanting],
+                [len(r.generated) + r.pending for r in wanting],
+                scatter=(ctx.logit_slots, ctx.last_tokens), out=host)
             event = torch.cuda.Event()
             event.record()
         self.scheduler.advance(batch)

@@ -93,8 +93,9 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
-def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
-    _dev(t, what)
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None, pinned_ok: bool = False) -> None:
+    if not (pinned_ok and not t.is_cuda and t.is_pinned()):  # (pinned host memory is mapped into the device's address space)
+        _dev(t, what)
     if t.dtype != torch.int32 or not t.is_contiguous():
         raise KernelError(f"{what} must be contiguous int32")
     if n is not None and t.numel() < n:
@@ -362,12 +363,13 @@ def _scatter(scatter, rows):
 def argmax(out: torch.Tensor, logits: torch.Tensor, scatter=None) -> None:
     """out[r] = the first maximal element of logits[r] (ties go to the lowest id). With
     scatter = (index, target), target[index[r]] = out[r] too; the caller has checked the
-    indices against the target."""
+    indices against the target. `out` may be pinned host memory: the kernel then writes the
+    tokens where the host reads them, and no copy follows."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
     if logits.dtype != torch.float32:
         raise KernelError("argmax: logits must be float32")
-    _i32(out, "out", rows)
+    _i32(out, "out", rows, pinned_ok=True)
     key = logits.device
     sc = _argmax_scratch.get(key)
     if sc is None or sc[0].numel() < rows * 64:
@@ -382,12 +384,13 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, scatter=None) -> None:
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, uniform: torch.Tensor, scatter=None) -> None:
     """Per-row sampling; temperature/top_p float32 [rows], top_k int32 [rows], uniform float64 [rows] in [0, 1).
-    top_k and top_p may both be None when no row cuts its candidates: a shorter kernel runs then."""
+    top_k and top_p may both be None when no row cuts its candidates: a shorter kernel runs then.
+    `out` may be pinned host memory, as for `argmax`."""
     ld = _rows(logits, "logits")
     rows, V = logits.shape
     if logits.dtype != torch.float32:
         raise KernelError("sample: logits must be float32")
-    _i32(out, "out", rows)
+    _i32(out, "out", rows, pinned_ok=True)
     _f32vec(temperature, "temperature", rows)
     if (top_k is None) != (top_p is None):
         raise KernelError("sample: top_k and top_p are given together or not at all")

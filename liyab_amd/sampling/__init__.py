@@ -85,11 +85,13 @@ class Sampler:
             self._cap = cap
 
     def sample_on_device(self, logits, params: Sequence[SamplingParams], seeds: Sequence[int], indices: Sequence[int],
-                         scatter=None):
+                         scatter=None, out=None):
         """One token per row of `logits` [rows, vocab] (float32, device), left on the device:
         returns an int32 tensor [rows] that stays valid until the next call. `seeds[r]` is row
         r's resolved seed and `indices[r]` how many tokens its request has generated so far.
-        With scatter = (index, target), row r's token also goes to target[index[r]]."""
+        With scatter = (index, target), row r's token also goes to target[index[r]]. `out`: where
+        the tokens go instead (int32, at least `rows` long; pinned host memory is taken: the kernel
+        then writes the tokens where the host reads them once the stream has come that far)."""
         import torch
 
         from ..kernels import ops
@@ -98,7 +100,7 @@ class Sampler:
         if not (len(params) == len(seeds) == len(indices) == rows):
             raise ValueError("one SamplingParams, seed and index per logits row is needed")
         self._buffers(rows)
-        out = self._out[:rows]
+        out = self._out[:rows] if out is None else out[:rows]
         if all(p.greedy for p in params):
             ops.argmax(out, logits, scatter=scatter)
         else:
