@@ -101,6 +101,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 constexpr int kRowwiseRows = 16;     // rows a workgroup
 constexpr int kRowwiseMaxRows = 64;  // steps of at most this many rows take the row-wise kernel
+constexpr int kTiledMinTiles = 512;  // and so do larger ones that would give the tiled kernel fewer tiles than this
 
 template <int NB, int WAVES, int EPI, bool EXACT>
 __global__ void __launch_bounds__(64 * WAVES)
@@ -290,7 +291,13 @@ extern "C" int liyab_gemm_simple(void* out, int out_dtype, int64_t ldo, const vo
     if (M == 0) return 0;
     if (dtype == kF32) {
         LIYAB_REQUIRE(epi == kEpiResidual || out_dtype == kF32, "gemm: 32-bit operands give a 32-bit output");
-        if (M <= kRowwiseMaxRows)
+        // more rows than that take the tiled kernel once its tiles of 64 x 64 are two workgroups for every
+        // compute unit (measured: from there it passes the row-wise kernel's steady 21 TFLOP/s); with fewer tiles
+        // the row-wise kernel's many small workgroups are faster, if its
+        // loads of 16 bytes fit the operands (else it would run one thread an element)
+        const bool vec = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && lda % 4 == 0 && K % 4 == 0;
+        const int64_t tiles = static_cast<int64_t>((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+        if (M <= kRowwiseMaxRows || (vec && tiles < kTiledMinTiles))
             return launch_rowwise_f32(static_cast<float*>(out), ldo, static_cast<const float*>(a), lda, static_cast<const float*>(w),
                                       bias, residual, ldr, M, N, K, epi, stream);
         return launch_simple<float, float, true>(out, ldo, a, lda, w, bias, residual, ldr, M, N, K, epi, stream);

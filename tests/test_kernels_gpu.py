@@ -195,7 +195,10 @@ GEMM_SHAPES = [(1, 64, 64), (7, 200, 96), (33, 777, 144), (130, 50, 320), (64, 1
 # beside those: each width of the row-wise kernel (4, 8 and 16 features a workgroup), chunks of K
 # with a tail, more chunks than waves, a K that is no multiple of 4 (the one-thread-an-element form)
 F32_SHAPES = GEMM_SHAPES + [(16, 1500, 100), (9, 2600, 260), (5, 3000, 72), (12, 40, 6), (40, 2561, 132), (3, 1024, 1028),
-                            (16, 33, 3076), (20, 70, 50)]
+                            (16, 33, 3076), (20, 70, 50),
+                            # 17 to 64 rows in one workgroup: 16 features a workgroup with 2, 3 and 4 rows a thread,
+                            # 8 with 1 and 2, 4 with a long K
+                            (24, 4100, 200), (45, 4097, 68), (64, 4800, 324), (30, 2050, 1604), (17, 100, 3076)]
 
 
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
@@ -218,9 +221,15 @@ def test_gemm_float32(ops, M, N, K, epilogue):
         full = torch.empty(M, N, device=DEV)
         ops.gemm(a, w, bias, out=full)
         assert torch.equal(one[0], full[M // 2])
-        many = torch.empty(40 + M, N, device=DEV)  # among 40 rows more: the tiled kernel
-        ops.gemm(torch.cat([rnd(40, K, seed=9), a]), w, bias, out=many)
-        assert torch.equal(many[40:], full)
+        many = torch.empty(70 + M, N, device=DEV)  # among 70 rows more: the tiled kernel, or the row-wise one again
+        rows = torch.cat([rnd(70, K, seed=9), a])
+        ops.gemm(rows, w, bias, out=many)
+        assert torch.equal(many[70:], full)
+        # from an address that is no multiple of 16 bytes the tiled kernel takes more than 64 rows, however few its tiles
+        shifted = torch.empty(rows.numel() + 1, device=DEV)[1:].view_as(rows).copy_(rows)
+        assert shifted.data_ptr() % 16 != 0
+        ops.gemm(shifted, w, bias, out=many)
+        assert torch.equal(many[70:], full)
 
 
 @pytest.mark.parametrize("kernel", ["simple", "mfma128", "mfma64", "mfma128x64", "auto", "skinny1", "skinny4", "skinny16", "skinny4w", "skinny2w", "skinny8m1", "skinny4m2", "skinny2m4",
