@@ -81,8 +81,8 @@ int liyab_cm_peak_in_use(void* h, int g) { return static_cast<CacheManager*>(h)-
 int liyab_cm_check(void* h) { return static_cast<CacheManager*>(h)->check(&g_error); }
 
 // -- a step's metadata --------------------------------------------------------------
-int liyab_step_shape(void* h, int n_seqs, const int* slots, const int* q_lens, const int* want_counts, StepShape* out) {
-    return step_shape(*static_cast<CacheManager*>(h), n_seqs, slots, q_lens, want_counts, out, &g_error);
+int liyab_step_shape(void* h, int n_seqs, const int* slots, const int* q_lens, const int* want_counts, int pad_rows, StepShape* out) {
+    return step_shape(*static_cast<CacheManager*>(h), n_seqs, slots, q_lens, want_counts, pad_rows, out, &g_error);
 }
 int liyab_step_fill(void* h, const StepShape* shape, const int* slots, const int* q_lens, const int64_t* tokens,
                     const int* want_counts, const int* wants, int vocab_size, int32_t* block) {

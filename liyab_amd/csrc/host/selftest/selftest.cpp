@@ -83,11 +83,17 @@ static int run(unsigned seed, int n_steps) {
             for (int i = 0; i < n; ++i) new_lengths[i] = first[i] + q_lens[i];
             CHECK(m.reserve(slots.data(), new_lengths.data(), n, &err) == kOk, "seed %u step %d: reserve after schedule: %s", seed, step, err.c_str());
             StepShape shape;
-            CHECK(step_shape(m, n, slots.data(), q_lens.data(), wants_n.data(), &shape, &err) == kOk, "step_shape: %s", err.c_str());
+            const int pad = pick(0, 2) == 0 ? pick(1, 70) : 0;  // some steps with padding rows behind their tokens
+            CHECK(step_shape(m, n, slots.data(), q_lens.data(), wants_n.data(), pad, &shape, &err) == kOk, "step_shape: %s", err.c_str());
+            CHECK(shape.n_tokens == budget && shape.n_rows == budget + pad, "step_shape: %d tokens and %d rows for %d + %d", shape.n_tokens, shape.n_rows, budget, pad);
             std::vector<int32_t> block(static_cast<size_t>(shape.total) + 8, -12345);
             CHECK(step_fill(m, shape, slots.data(), q_lens.data(), toks.data(), wants_n.data(), wants.data(), 100, block.data(), &err) == kOk,
                   "step_fill: %s", err.c_str());
             for (int k = 0; k < 8; ++k) CHECK(block[static_cast<size_t>(shape.total) + k] == -12345, "step_fill wrote past its block");
+            for (int j = shape.n_tokens; j < shape.n_rows; ++j) {
+                CHECK(block[shape.off_token_ids + j] == 0 && block[shape.off_positions + j] == 0 && block[shape.off_tok_seq + j] == 0, "a padding row's token, position or request");
+                for (int g = 0; g < shape.n_groups; ++g) CHECK(block[shape.off_slots[g] + j] == -1, "a padding row with a slot");
+            }
             int n_tiles = 0, n_single = 0;
             const int tile = pick(0, 1) ? 64 : 128;
             attn_counts(n, q_lens.data(), 8, tile, &n_tiles, &n_single);

@@ -11,8 +11,9 @@ static Status fail(std::string* err, Status s, const std::string& msg) {
 }
 
 Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int* q_lens, const int* want_counts,
-                  StepShape* out, std::string* err) {
+                  int pad_rows, StepShape* out, std::string* err) {
     if (n_seqs <= 0) return fail(err, kInvalidArgument, "a step needs at least one item");
+    if (pad_rows < 0) return fail(err, kInvalidArgument, "a negative number of padding rows");
     if (m.n_groups() > kMaxGroups) return fail(err, kInvalidArgument, "more cache groups than a step's metadata holds");
     StepShape s{};
     s.n_seqs = n_seqs;
@@ -32,7 +33,8 @@ Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int
         cur += size;
         return at;
     };
-    const int N = s.n_tokens, S = n_seqs, R = s.n_logit_rows;
+    s.n_rows = s.n_tokens + pad_rows;
+    const int N = s.n_rows, S = n_seqs, R = s.n_logit_rows;
     s.off_token_ids = place(N);
     s.off_positions = place(N);
     s.off_tok_seq = place(N);
@@ -84,6 +86,11 @@ Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, co
         row0 += n;
     }
     starts[S] = row0;
+    for (int j = row0; j < s.n_rows; ++j) {  // padding rows
+        tok[j] = 0;
+        pos[j] = 0;
+        seq[j] = 0;
+    }
     for (int g = 0; g < s.n_groups; ++g) {
         int32_t* bt = block + s.off_block_tables[g];
         int32_t* sl = block + s.off_slots[g];
@@ -99,6 +106,7 @@ Status step_fill(const CacheManager& m, const StepShape& s, const int* slots, co
                 sl[starts[i] + j] = pg * page + p % page;
             }
         }
+        for (int j = s.n_tokens; j < s.n_rows; ++j) sl[j] = -1;
     }
     return kOk;
 }

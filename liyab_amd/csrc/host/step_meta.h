@@ -21,7 +21,7 @@ constexpr int kMaxGroups = 16;
 
 // Sizes of a step and where each array starts in the block (offsets in words).
 struct StepShape {
-    int n_tokens, n_seqs, n_logit_rows, n_groups, max_blocks;
+    int n_tokens, n_rows, n_seqs, n_logit_rows, n_groups, max_blocks;  // n_rows: the tokens and the padding rows after them
     int max_q_len, max_context;
     int total;       // words in the block
     int off_token_ids, off_positions, off_tok_seq, off_seq_starts, off_context_lens, off_state_slots;
@@ -29,9 +29,12 @@ struct StepShape {
     int off_block_tables[kMaxGroups], off_slots[kMaxGroups];
 };
 
-// From the items' sizes alone (requests by slot, tokens each brings, logits each wants).
+// From the items' sizes alone (requests by slot, tokens each brings, logits each wants). pad_rows: rows
+// after the last token that belong to no request (a step padded to a size that comes back, so that its
+// captured graph serves every step of that size): token 0 at position 0 of the step's first request, slot
+// -1 in every group, which no kernel writes to; nothing reads what is computed for them.
 Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int* q_lens, const int* want_counts,
-                  StepShape* out, std::string* err);
+                  int pad_rows, StepShape* out, std::string* err);
 
 // Fills the block. `tokens`: the items' token ids one after the other; an id < 0 stands for "the
 // token sampled for slot -1 - id, still on the device". `wants`: places within each item.

@@ -77,6 +77,17 @@ class _Staging:
 GRAPH_AFTER_MIXED = 3  # eager runs of a shape that its parts do not expect to recur before it is captured
 
 
+def padded_rows(n: int) -> int:
+    """The rows of a step of `n` tokens in which some request brings more than one: the next multiple of
+    16 up to 64 rows, of 64 up to 1,024, of 128 beyond. Prompts come in every length, and a step launched
+    kernel by kernel costs the host more than the device (GPT-2 small's sizes, a prompt of 512: 0.9 ms of
+    launches for 0.75 ms of kernels); in steps of these sizes a prompt's length recurs among a few dozen, so
+    that its step is replayed from a captured graph. The products' tiles cover the padding anyway;
+    attention and the cache never see it."""
+    unit = 16 if n <= 64 else 64 if n <= 1024 else 128
+    return -(-n // unit) * unit
+
+
 class StepFunction:
     """`use_graphs`: a step whose shape (tokens, requests, wanted rows, and the key of every
     part's step planner: attention's mode, context bucket and tiles) has been seen before is
@@ -105,6 +116,9 @@ class StepFunction:
         self.last_context: Optional[StepContext] = None
         self.phases: Optional[PhaseTimer] = None  # set: every step is launched kernel by kernel and timed per phase
         self.planners = list(getattr(model, "step_planners", ()))
+        # steps of prompt portions are padded to sizes that recur (padded_rows) where graphs are used and
+        # every part of the model takes padding rows
+        self.pads_rows = bool(use_graphs and getattr(model, "takes_padding_rows", False))
         self._key = None  # the prepared step's shape: what its captured graph is kept under
         self._recurs = True
 
@@ -189,13 +203,18 @@ class StepFunction:
         self.graph_replays += 1
         return logits
 
+    def forget_graphs(self) -> None:
+        """Drops every captured graph and what is known of the shapes seen: the next step of any
+        shape is a first sight (measurements of that case use it)."""
+        self._graphs.clear()
+
     # -- the step -------------------------------------------------------------
     def run(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
         """Runs the items as one batch from the cache earlier steps left.
         Returns float32 logits [wanted, vocab] on the device, rows in the order
         of the items and of each item's `want`, or None when nothing is wanted.
         The tensor is workspace memory: valid until the next step."""
-        ctx, lengths = self.prepare(items)
+        ctx, lengths = self.prepare(items, pad=self.pads_rows)
         logits = self._forward(ctx)
         self.commit(items, lengths)
         self.last_context = ctx
@@ -209,11 +228,12 @@ class StepFunction:
         self.steps += 1
         self.tokens += sum(len(it.tokens) for it in items)
 
-    def prepare(self, items: Sequence[StepItem]):
+    def prepare(self, items: Sequence[StepItem], pad: bool = False):
         """Checks the items, maps their pages (all or nothing) and puts the step's metadata on
         the device. Returns (StepContext, what `commit` needs once the step has run). The
         metadata block is laid out and filled by the host library (csrc/host/step_meta.cpp)
-        straight into pinned memory."""
+        straight into pinned memory. `pad`: a step in which some request brings more than one token
+        gets padding rows behind its tokens up to `padded_rows` of their number (see there)."""
         self._validate(items)
         mgr = self.manager
         S = len(items)
@@ -243,7 +263,9 @@ class StepFunction:
         lib = host.lib()
         shape = host.StepShape()
         ip = lambda a: a.ctypes.data_as(host.IP)  # noqa: E731
-        host.check(lib.liyab_step_shape(mgr.handle, S, ip(slots), ip(q_lens), ip(want_counts), ctypes.byref(shape)))
+        pad_rows = padded_rows(N) - N if pad and N > S and self.phases is None else 0
+        host.check(lib.liyab_step_shape(mgr.handle, S, ip(slots), ip(q_lens), ip(want_counts), pad_rows, ctypes.byref(shape)))
+        rows = shape.n_rows
         # the parts' own words stand behind the common block; their keys join the step's shape
         first_pos = (new_lengths - q_lens).astype(np.intc, copy=False)
         total = shape.total
@@ -255,7 +277,7 @@ class StepFunction:
                 p = planner.plan(facts)
                 plans.append((planner.name, p, total))
                 total += p.n_words
-        self._key = (N, S, R) + tuple((name, p.key, p.n_words) for name, p, _ in plans)
+        self._key = (rows, S, R) + tuple((name, p.key, p.n_words) for name, p, _ in plans)
         self._recurs = all(p.recurs for _, p, _ in plans)
         host_t = self._staging.next(total)
         base = ctypes.cast(host_t.data_ptr(), ctypes.POINTER(ctypes.c_int32))
@@ -278,16 +300,16 @@ class StepFunction:
         W, G, page = shape.max_blocks, shape.n_groups, mgr.page_size
         starts = np.cumsum(q_lens) - q_lens
         ctx = StepContext(
-            n_tokens=N, n_seqs=S,
-            token_ids=dev[shape.off_token_ids:shape.off_token_ids + N],
-            positions=dev[shape.off_positions:shape.off_positions + N],
-            tok_seq=dev[shape.off_tok_seq:shape.off_tok_seq + N],
+            n_tokens=rows, n_seqs=S,
+            token_ids=dev[shape.off_token_ids:shape.off_token_ids + rows],
+            positions=dev[shape.off_positions:shape.off_positions + rows],
+            tok_seq=dev[shape.off_tok_seq:shape.off_tok_seq + rows],
             seq_starts=dev[shape.off_seq_starts:shape.off_seq_starts + S + 1],
             context_lens=dev[shape.off_context_lens:shape.off_context_lens + S],
             state_slots=dev[shape.off_state_slots:shape.off_state_slots + S],
             logit_rows=dev[shape.off_logit_rows:shape.off_logit_rows + max(R, 1)], n_logit_rows=R,
             groups=[GroupStep(block_tables=dev[shape.off_block_tables[g]:shape.off_block_tables[g] + S * W].view(S, W),
-                              slots=dev[shape.off_slots[g]:shape.off_slots[g] + N]) for g in range(G)],
+                              slots=dev[shape.off_slots[g]:shape.off_slots[g] + rows]) for g in range(G)],
             host=StepHost(q_lens=q_lens.tolist(), starts=starts.tolist(), first_pos=first_pos.tolist(),
                           max_q_len=shape.max_q_len, max_context=shape.max_context),
             workspace=self.workspace, dtype=self.model.dtype, page_size=page,

@@ -19,7 +19,7 @@ class StepShape(ctypes.Structure):
     """Mirror of liyab_host::StepShape (csrc/host/step_meta.h)."""
 
     _fields_ = [(n, c_int) for n in (
-        "n_tokens", "n_seqs", "n_logit_rows", "n_groups", "max_blocks", "max_q_len",
+        "n_tokens", "n_rows", "n_seqs", "n_logit_rows", "n_groups", "max_blocks", "max_q_len",
         "max_context", "total", "off_token_ids", "off_positions", "off_tok_seq", "off_seq_starts", "off_context_lens",
         "off_state_slots", "off_logit_rows", "off_logit_slots")] + [
         ("off_block_tables", c_int * MAX_GROUPS), ("off_slots", c_int * MAX_GROUPS)]
@@ -70,7 +70,7 @@ _SIGNATURES = {
     "liyab_sched_get": ([c_void_p, c_int, c_int], c_int),
     "liyab_sched_list": ([c_void_p, c_int, IP, c_int], c_int),
     "liyab_sched_stats": ([c_void_p, POINTER(ctypes.c_longlong)], None),
-    "liyab_step_shape": ([c_void_p, c_int, IP, IP, IP, POINTER(StepShape)], c_int),
+    "liyab_step_shape": ([c_void_p, c_int, IP, IP, IP, c_int, POINTER(StepShape)], c_int),
     "liyab_step_fill": ([c_void_p, POINTER(StepShape), IP, IP, POINTER(c_int64), IP, IP, c_int, POINTER(c_int32)], c_int),
     "liyab_attn_counts": ([c_int, IP, c_int, c_int, IP], None),
     "liyab_attn_fill": ([c_int, IP, IP, c_int, c_int, POINTER(c_int32)], None),

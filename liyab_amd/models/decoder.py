@@ -147,6 +147,14 @@ class DecoderModel:
             self._layer_kind.append(_describe(block, tensors, set()))
             self._layer_tensors.append(tensors)
         self.replayed_layers = 0  # layers that ran from a recorded list, over the model's lifetime
+        # A step may carry padding rows behind its tokens (engine/step.py: padded_rows) when every part that
+        # sees all the step's rows says that it takes them (`takes_padding_rows`): the embedding, a position
+        # encoding of the stream, and every block with its mixer, feed-forward and norms. The final norm and
+        # the head see the wanted rows only.
+        every = [self.embedding, self.residual_position]
+        for block in self.blocks:
+            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn")]
+        self.takes_padding_rows = all(bool(getattr(part, "takes_padding_rows", False)) for part in every if part is not None)
 
     # -- what the cache manager needs to know ---------------------------------
     def cache_groups(self) -> List[Tuple[KVSpec, List[int]]]:

@@ -108,6 +108,12 @@ class Attention:
     # tensors and the constants among its attributes: layers of this kind may run from one recorded list
     replayable = True
 
+    @property
+    def takes_padding_rows(self) -> bool:
+        """Rows behind the step's tokens (token 0 at position 0 of the first request, slot -1) are computed
+        and never read: their keys and values are not written, and no other row attends to them."""
+        return self.position is None or bool(getattr(self.position, "takes_padding_rows", False))
+
     def __init__(self, spec, store, dtype: torch.dtype):
         self.spec = spec
         self.dtype = dtype

@@ -16,6 +16,9 @@ class PreNormBlock:
     # every launch goes through the kernel library and depends on nothing of this object but its
     # tensors and the constants among its attributes: layers of this kind may run from one recorded list
     replayable = True
+    # rows behind the step's tokens (token 0 at position 0 of the first request, slot -1) are computed
+    # and never read: nothing here writes for them or lets them touch another row
+    takes_padding_rows = True
 
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn

@@ -15,6 +15,8 @@ class TokenEmbedding:
     """x[t] = scale * table[id_t] (the reference's embed, src/core/transformer.cpp:5495-5512).
     A residual position table may be folded into the same pass."""
 
+    takes_padding_rows = True  # (they carry token 0)
+
     def __init__(self, spec, store, dtype: torch.dtype):
         self.vocab_size, self.width, self.scale = spec.vocab_size, spec.width, float(spec.scale)
         self.table = store.fetch(spec.tensors["table"], (self.vocab_size, self.width), "table")
@@ -29,6 +31,7 @@ class LearnedPositions:
     The only position encoding that caps the context at its table's rows (:819-823)."""
 
     where = "residual"
+    takes_padding_rows = True  # (they sit at position 0)
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.max_positions, self.width = spec.max_positions, spec.width

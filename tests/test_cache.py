@@ -244,7 +244,8 @@ def test_a_steps_metadata_names_only_pages_and_slots_of_the_pool(seed, page_size
     """Random stories of requests through the step metadata's native layout (liyab_step_shape /
     liyab_step_fill): every page id a block table carries to the device is -1 or a page of the
     pool, every slot a position of a page of the pool, and the slot of a token is its page's
-    place in the table. The kernels follow these words without asking."""
+    place in the table. The kernels follow these words without asking. Some steps carry padding rows
+    behind their tokens: token 0 at position 0 of the first request, with slot -1, which the kernels skip."""
     import ctypes
 
     from liyab_amd import host
@@ -276,7 +277,9 @@ def test_a_steps_metadata_names_only_pages_and_slots_of_the_pool(seed, page_size
                 continue
             wants = np.zeros(len(batch), dtype=np.intc)
             shape = host.StepShape()
-            host.check(lib.liyab_step_shape(m.handle, len(batch), ip(slots), ip(q_lens), ip(wants), ctypes.byref(shape)))
+            pad = rng.choice([0, 0, 1, 15, 63])
+            host.check(lib.liyab_step_shape(m.handle, len(batch), ip(slots), ip(q_lens), ip(wants), pad, ctypes.byref(shape)))
+            assert shape.n_tokens == int(q_lens.sum()) and shape.n_rows == shape.n_tokens + pad
             block = np.full(shape.total, -12345, dtype=np.int32)
             tokens = np.array([rng.randrange(vocab) for _ in range(int(q_lens.sum()))], dtype=np.int64)
             host.check(lib.liyab_step_fill(m.handle, ctypes.byref(shape), ip(slots), ip(q_lens),
@@ -292,6 +295,10 @@ def test_a_steps_metadata_names_only_pages_and_slots_of_the_pool(seed, page_size
                 assert bt.min() >= -1 and bt.max() < num_pages
                 assert sl.min() >= 0 and sl.max() < num_pages * page_size
                 assert (sl == bt[tok_seq, positions // page_size] * page_size + positions % page_size).all()
+                assert (block[shape.off_slots[g] + N:shape.off_slots[g] + N + pad] == -1).all()
+            for off in (shape.off_token_ids, shape.off_positions, shape.off_tok_seq):
+                assert (block[off + N:off + N + pad] == 0).all()
+            assert (block != -12345).all()  # every word of the block is written
             m.commit_slots(slots, new_lengths)
             for r, n in zip(batch, new_lengths):
                 live[r] = int(n)

@@ -160,6 +160,54 @@ def test_replayed_graphs_give_the_eager_logits(dtype, max_graphs, model_dirs):
     assert graphs.manager.pages_in_use() == 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prompts_of_one_padded_size_share_a_graph(dtype, model_dirs):
+    """Steps in which a request brings several tokens are padded to sizes that recur (rows behind
+    their tokens that belong to no request): prompts of 33 to 48 tokens are one shape, launched
+    kernel by kernel three times, then captured once and replayed. Logits have the bits of an engine
+    that neither pads nor captures, also when everything the padding rows might leave behind (the
+    workspace's buffers) is filled with NaN between the steps, and with pages that are used again."""
+    import torch
+
+    from liyab_amd.engine import EngineCore, StepItem
+    from liyab_amd.engine.step import padded_rows
+
+    assert [padded_rows(n) for n in (2, 16, 17, 33, 48, 64, 65, 500, 1024, 1025)] == [16, 16, 32, 48, 48, 64, 128, 512, 1024, 1152]
+    name = "C"
+    cfg, _ = CONFIGS[name]
+    rng = np.random.default_rng(5)
+    plain_core = EngineCore(model_dirs[name], dtype=dtype, page_size=16, max_tokens=64, max_requests=2, use_graphs=False)
+    core = EngineCore(model_dirs[name], dtype=dtype, page_size=16, max_tokens=64, max_requests=2, use_graphs=True)
+    assert core.step_fn.pads_rows and not plain_core.step_fn.pads_rows
+    lengths = [37, 45, 40, 33, 48, 41, 47, 34]
+    for i, n in enumerate(lengths):
+        toks = rng.integers(0, cfg["vocab_size"], n).tolist()
+        want = [0, n // 2, n - 1]
+        out = []
+        for c in (plain_core, core):
+            c.open("r")
+            before = c.step_fn.graph_replays
+            first = c.step([StepItem("r", toks, want)]).float().cpu().numpy().copy()
+            replayed = c.step_fn.graph_replays > before
+            after = c.step([StepItem("r", [toks[0]], [0])]).float().cpu().numpy().copy()  # a decoded token reads the portion's keys
+            c.close("r")
+            out.append((first, after))
+        assert np.array_equal(out[0][0], out[1][0]) and np.array_equal(out[0][1], out[1][1]), f"prompt {i} of {n} tokens"
+        assert np.isfinite(out[1][0]).all()
+        # three sights launched kernel by kernel, then the capture (once more if a buffer of the workspace grew under it)
+        assert not (replayed and i < 3) and (replayed or i < 5), f"prompt {i}: replayed {replayed}"
+        for buf in core.step_fn.workspace._bufs.values():
+            if buf.is_floating_point():
+                buf.fill_(float("nan"))
+        torch.cuda.synchronize()
+    fn = core.step_fn
+    prefill_graphs = [k for k, v in fn._graphs.items() if isinstance(v, tuple) and k[0] == 48]
+    assert len(prefill_graphs) == 1, list(fn._graphs)
+    assert fn.graph_replays >= len(lengths), fn.graph_replays
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+
+
 # ---------------------------------------------------------------------------
 # geometries that take the kernels' fallbacks in bfloat16; a head of its own
 # ---------------------------------------------------------------------------

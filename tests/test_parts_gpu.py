@@ -939,6 +939,7 @@ def test_a_part_with_its_own_step_metadata_runs_under_graphs_and_the_scheduler()
     prompts = [tt.random_tokens(70 + i, n, info["V"]) for i, n in enumerate([30, 5, 41, 17])]
     core = EngineCore.from_plan(plan, tw, dtype="float32", page_size=8, num_pages=14, max_requests=3, use_graphs=True)
     assert [p.name for p in core.model.step_planners] == ["toy_scan", "attention"]
+    assert not core.step_fn.pads_rows  # the toy does not say that it takes padding rows: its steps get none
     ScanPlanner.calls = 0
     engine = Engine(core=core, max_num_seqs=3, max_batched_tokens=24, prefill_chunk=16)
     engine.stop_at_eos = False
