@@ -34,6 +34,12 @@ class EpiParams(ctypes.Structure):
 
 
 _EPI_PTR = ctypes.POINTER(EpiParams)
+# which of the block's 8-byte words are addresses (a pointer field fills one word)
+_EPI_ADDRESS_WORDS = [False] * ((ctypes.sizeof(EpiParams) + 7) // 8)
+for _name, _type in EpiParams._fields_:
+    if _type is P:
+        _EPI_ADDRESS_WORDS[getattr(EpiParams, _name).offset // 8] = True
+_EPI_ADDRESS_WORDS = tuple(_EPI_ADDRESS_WORDS)
 
 _SIGNATURES = {
     "liyab_check_device": [],
@@ -126,6 +132,7 @@ def call(name: str, *args) -> None:
 
 # -- a list of launches, recorded once and run again natively with other tensors ----------------
 _recording: Optional[list] = None  # the words of the list being recorded, or None
+_recording_addresses: Optional[list] = None  # for each of them: whether it is an address (a pointer argument or field)
 _recording_whole = True  # whether every launch so far could be written down
 _entries: dict = {}  # launcher name -> (index in the native table, encoders of its arguments)
 BLOCK_ARG = 0xB10CB10CB10CB10C  # stands for the argument that points at an epilogue's parameter block (csrc/replay.hip)
@@ -142,7 +149,8 @@ def _encoders(name: str):
         index = lib.liyab_replay_index(name.encode(), ctypes.byref(n))
         kinds = []
         for t in _SIGNATURES[name]:
-            kinds.append("block" if t is _EPI_PTR else ("float" if t is c_float else ("double" if t is c_double else "int")))
+            kinds.append("block" if t is _EPI_PTR else "float" if t is c_float else "double" if t is c_double else
+                         "address" if t is P else "int")
         hit = _entries[name] = (index, kinds) if index >= 0 and n.value == len(kinds) and "double" not in kinds else (-1, kinds)
     return hit
 
@@ -153,10 +161,11 @@ def _record(name: str, args) -> None:
     if index < 0:
         _recording_whole = False  # a launcher the native replay does not know: the list is of no use
         return
-    words = [index, len(args)]
-    block = ()
+    words, addresses = [index, len(args)], [False, False]
+    block, block_addresses = (), ()
     for kind, a in zip(kinds, args):
-        if kind == "int":
+        addresses.append(kind == "address")
+        if kind == "int" or kind == "address":
             words.append((0 if a is None else int(a)) & _U64)
         elif kind == "float":
             words.append(struct.unpack("<I", struct.pack("<f", a))[0])
@@ -164,32 +173,39 @@ def _record(name: str, args) -> None:
             raw = bytes(a._obj)  # (the argument is ctypes.byref(params))
             raw += b"\0" * (-len(raw) % 8)
             block = struct.unpack(f"<{len(raw) // 8}Q", raw)
+            block_addresses = _EPI_ADDRESS_WORDS
             words.append(BLOCK_ARG)
     words.append(len(block))
     words.extend(block)
+    addresses.append(False)
+    addresses.extend(block_addresses)
     _recording.extend(words)
+    _recording_addresses.extend(addresses)
 
 
 class recording:
     """Within this context every launch is also written down; `words` holds the list afterwards
-    (a numpy array of uint64, see csrc/replay.hip), or None if a launcher ran that the native
-    replay does not know."""
+    (a numpy array of uint64, see csrc/replay.hip) and `addresses` which of them are addresses
+    (pointer arguments and pointer fields of a parameter block; a size or a constant never is), or
+    None if a launcher ran that the native replay does not know."""
 
     def __enter__(self):
-        global _recording, _recording_whole
+        global _recording, _recording_addresses, _recording_whole
         if _recording is not None:
             raise KernelError("a list of launches is being recorded already")
-        _recording, _recording_whole = [], True
-        self.words = None
+        _recording, _recording_addresses, _recording_whole = [], [], True
+        self.words = self.addresses = None
         return self
 
     def __exit__(self, exc_type, *exc):
-        global _recording
+        global _recording, _recording_addresses
         import numpy as np
 
         words, _recording = _recording, None
+        addresses, _recording_addresses = _recording_addresses, None
         if exc_type is None and _recording_whole:
             self.words = np.array(words, dtype=np.uint64)
+            self.addresses = np.array(addresses, dtype=bool)
         return False
 
 

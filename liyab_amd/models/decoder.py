@@ -67,9 +67,10 @@ def _describe(obj, tensors: list, seen: set):
 
 class _Recorded:
     """A layer's launches as a list of words, and where in it the addresses of the layer's own
-    tensors stand (any address inside one of them, as an offset from its start)."""
+    tensors stand (any address inside one of them, as an offset from its start). `addresses`: which
+    words are addresses at all; a size or a constant that happens to lie in a tensor's range is not one."""
 
-    def __init__(self, words: np.ndarray, bases: np.ndarray, sizes, pending_out):
+    def __init__(self, words: np.ndarray, addresses: np.ndarray, bases: np.ndarray, sizes, pending_out):
         self.words = words
         self.pending_out = pending_out
         order = np.argsort(bases)
@@ -79,7 +80,9 @@ class _Recorded:
         for i in range(1, len(starts)):
             if starts[i] < starts[i - 1] + sizes[order[i - 1]]:
                 self.usable = False  # two of the layer's tensors overlap: an address would name both
-        for at, word in enumerate(words.tolist()):
+        listed = words.tolist()
+        for at in np.flatnonzero(addresses).tolist():
+            word = listed[at]
             j = bisect.bisect_right(starts, word) - 1
             if j >= 0 and word < starts[j] + sizes[order[j]]:
                 positions.append(at)
@@ -220,7 +223,7 @@ class DecoderModel:
                         pending = None
                     block.forward(*args, writes_cache=e.writes_cache)
             if rec is not None and rec.words is not None and (pending is None or isinstance(pending, SplitStream)):
-                recorded[key] = _Recorded(rec.words, bases, [t.numel() * t.element_size() for t in own], pending)
+                recorded[key] = _Recorded(rec.words, rec.addresses, bases, [t.numel() * t.element_size() for t in own], pending)
         if phases is not None:
             phases.mark("lm_head")
             try:

@@ -158,9 +158,12 @@ def test_what_makes_two_layers_one_kind_and_how_a_recorded_list_gets_another_lay
     own = Block(Part(0.5, a))
     own.part.loop = own
     assert _describe(own, [], set()) is _OTHER  # an object met twice
-    # a list whose words 2 and 5 point into the first and the second tensor of the recorded layer
+    # a list whose words 2 and 5 point into the first and the second tensor of the recorded layer; word 7 is
+    # a size that happens to lie in the first tensor's range and stays what it is
     bases = np.array([1000, 5000], dtype=np.uint64)
-    rec = _Recorded(np.array([7, 3, 1000 + 16, 999, 6000, 5000, 1000 + 64], dtype=np.uint64), bases, [64, 100], None)
+    words = np.array([7, 3, 1000 + 16, 999, 6000, 5000, 1000 + 64, 1008], dtype=np.uint64)
+    addresses = np.array([False, False, True, True, True, True, False, False])
+    rec = _Recorded(words, addresses, bases, [64, 100], None)
     assert rec.usable and rec.positions.tolist() == [2, 5] and rec.offsets.tolist() == [16, 0]
-    assert rec.for_layer(np.array([20000, 90000], dtype=np.uint64)).tolist() == [7, 3, 20016, 999, 6000, 90000, 1064]
-    assert not _Recorded(np.array([1], dtype=np.uint64), np.array([1000, 1032], dtype=np.uint64), [64, 8], None).usable  # overlapping tensors
+    assert rec.for_layer(np.array([20000, 90000], dtype=np.uint64)).tolist() == [7, 3, 20016, 999, 6000, 90000, 1064, 1008]
+    assert not _Recorded(np.array([1], dtype=np.uint64), np.array([True]), np.array([1000, 1032], dtype=np.uint64), [64, 8], None).usable  # overlapping tensors
