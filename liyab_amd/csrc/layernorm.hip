@@ -87,7 +87,9 @@ template <typename T, int MAXV, bool PARTS>
 __global__ void __launch_bounds__(256)
 layernorm_wave_kernel(T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
                       const float* __restrict__ b, const int* __restrict__ rows, int n, int d, float eps, PartSums ps) {
-    const int lane = threadIdx.x % kWave, r = blockIdx.x * 4 + threadIdx.x / kWave;
+    // a wave a row, blockDim.x / 64 rows a workgroup (one while the rows are few: a compute unit draws
+    // its rows at a tenth of what the chip can, and 64 rows of five planes are a megabyte)
+    const int lane = threadIdx.x % kWave, r = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (r >= n) return;
     const int64_t src = rows != nullptr ? rows[r] : r;
     const float* row0 = x + src * d;
@@ -215,9 +217,10 @@ __global__ void __launch_bounds__(256) sum_parts_kernel(float* out, const float*
 template <typename T, int MAXV>
 void launch_wave(T* out, const float* x, const float* w, const float* b, const int* rows, int n, int d, float eps,
                  const PartSums& ps, hipStream_t stream) {
-    const int grid = (n + 3) / 4;
-    if (ps.n_parts > 1) layernorm_wave_kernel<T, MAXV, true><<<grid, 256, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
-    else layernorm_wave_kernel<T, MAXV, false><<<grid, 256, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
+    const int waves = n <= 512 ? 1 : 4;  // rows a workgroup
+    const int grid = (n + waves - 1) / waves;
+    if (ps.n_parts > 1) layernorm_wave_kernel<T, MAXV, true><<<grid, kWave * waves, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
+    else layernorm_wave_kernel<T, MAXV, false><<<grid, kWave * waves, 0, stream>>>(out, x, w, b, rows, n, d, eps, ps);
 }
 
 // Whether the kernels that keep a row in registers take these operands (the only ones that add planes up):
