@@ -14,6 +14,7 @@
 // The argument that points at the epilogue's parameter block holds kBlockArg instead; the block's
 // bytes follow the arguments, and the launcher gets their address.
 #include "launchers.h"
+#include "epilogue.h"
 
 #include <cstring>
 #include <utility>
@@ -123,6 +124,8 @@ extern "C" int liyab_replay(const uint64_t* list, int64_t n_words) {
         LIYAB_REQUIRE(at + 2 + static_cast<int64_t>(n_args) + 1 <= n_words, "replay: a record is cut short at word %lld", static_cast<long long>(at));
         const uint64_t n_block = list[at + 2 + n_args];
         LIYAB_REQUIRE(n_block <= kMaxBlockWords && at + 3 + static_cast<int64_t>(n_args + n_block) <= n_words, "replay: a parameter block of %llu words",
+                      static_cast<unsigned long long>(n_block));
+        LIYAB_REQUIRE(n_block == 0 || n_block * sizeof(uint64_t) >= sizeof(EpiParams), "replay: a parameter block of %llu words is shorter than the launchers read",
                       static_cast<unsigned long long>(n_block));
         int blocks = 0;
         for (uint64_t i = 0; i < n_args; ++i) blocks += list[at + 2 + i] == kBlockArg ? 1 : 0;

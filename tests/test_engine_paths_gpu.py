@@ -376,6 +376,10 @@ def test_a_malformed_list_of_launches_is_refused_before_anything_runs():
                         ([index, 5, lib.BLOCK_ARG, 4, 0, 0, 0, 0], "parameter block")):
         with pytest.raises(Exception, match=what):
             lib.replay(np.array(words, dtype=np.uint64))
+    product, kinds = lib._encoders("liyab_gemm_mfma")
+    assert product >= 0 and kinds[7] == "block" and len(kinds) == 9
+    with pytest.raises(Exception, match="shorter than the launchers read"):  # one word where the epilogue's parameters stand
+        lib.replay(np.array([product, 9, 0, 0, 0, 0, 0, 0, 0, lib.BLOCK_ARG, 0, 1, 0], dtype=np.uint64))
     lib.replay(np.array([], dtype=np.uint64))
 
 
