@@ -1,7 +1,8 @@
 """Each part alone against its plain formula, and the generality of the layer plan: a toy
 mixer with state of its own, a feed-forward that routes and a position encoding without a
-table, defined here, are registered, built and stepped without touching the framework's files; a layer reads another layer's cache; the run order names a layer twice
-(needs the GPU)."""
+table, defined here, are registered, built and stepped without touching the framework's files; a layer
+reads another layer's cache; the run order names a layer twice; a norm of another kind and blocks arranged
+otherwise (parallel, post-norm) (needs the GPU)."""
 
 import math
 
@@ -1125,6 +1126,143 @@ def test_split_streams_reach_parts_that_cannot_take_them(monkeypatch):
         tt.check_against_plain(got, reqs, ref, TOL_TOY["bfloat16"], f"toy with forced cuts, {name}")
         core.manager.check()
     assert 2 in cut and 1 in cut  # both ways were taken
+
+
+# ---------------------------------------------------------------------------
+# another norm and two other arrangements of a block
+# ---------------------------------------------------------------------------
+class RmsSpec:
+    kind = "toy_rms"
+
+    def __init__(self, width, eps, prefix):
+        self.width, self.eps, self.prefix = width, eps, prefix
+
+
+class RmsNorm:
+    """y = x / sqrt(mean(x^2) + eps) * weight: no mean taken off, no bias. A test's toy in torch with
+    only what a norm must have: forward(x, ctx, rows, n_rows, name) -> rows in the compute dtype."""
+
+    def __init__(self, spec, store, dtype):
+        from liyab_amd.config import TensorSource
+
+        self.width, self.eps, self.dtype = spec.width, float(spec.eps), dtype
+        self.weight = store.fetch(TensorSource(spec.prefix + ".w"), (self.width,), "vector")
+
+    def forward(self, x, ctx, rows=None, n_rows=None, name="normed"):
+        x = x.float()
+        if rows is not None:
+            x = x[rows.long()[:n_rows if n_rows is not None else rows.numel()]]
+        out = ctx.workspace.get(name, tuple(x.shape), self.dtype)
+        out.copy_(self.stream(x))
+        return out
+
+    def stream(self, x):
+        """The same in 32-bit, for a block that keeps the norm's output as the stream."""
+        return x * torch.rsqrt((x * x).mean(dim=1, keepdim=True) + self.eps) * self.weight.float()
+
+
+class ParallelBlock:
+    """x += mixer(norm(x)) + ffn(norm(x)): one norm, both parts read its rows."""
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
+        assert norm_ffn is None
+        self.mixer, self.ffn, self.norm = mixer, ffn, norm_mixer
+
+    def forward(self, x, ctx, cache, state, writes_cache=True):
+        h = self.norm.forward(x, ctx, name="parallel_in").clone()  # (both parts read it: not the workspace's next view of that name)
+        self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
+        self.ffn.forward(h, ctx, x)
+
+
+class PostNormBlock:
+    """x = norm_mixer(x + mixer(x)); x = norm_ffn(x + ffn(x)): the norms come after the sums and
+    the stream itself is what they leave."""
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
+        self.dtype = mixer.dtype
+
+    def forward(self, x, ctx, cache, state, writes_cache=True):
+        self.mixer.forward(x.to(self.dtype), ctx, cache, state, x, writes_cache=writes_cache)
+        x.copy_(self.norm_mixer.stream(x))
+        self.ffn.forward(x.to(self.dtype), ctx, x)
+        x.copy_(self.norm_ffn.stream(x))
+
+
+def arranged_model(dtype="float32"):
+    """Layer 0: a parallel block behind the framework's LayerNorm (4 query heads on 2 key/value heads
+    of 16, tanh feed-forward); layer 1: a post-norm block with root-mean-square norms (3 heads of 32,
+    erf feed-forward); the final norm is the toy's too."""
+    from liyab_amd.config import HeadSpec, LayerSpec, ModelPlan, OrderEntry, PositionSpec, TokenEmbeddingSpec
+    from liyab_amd.parts import register_block, register_norm
+
+    register_norm("toy_rms", RmsNorm)
+    register_block("toy_parallel", ParallelBlock)
+    register_block("toy_post_norm", PostNormBlock)
+    d, V, P, eps = 96, 211, 160, 2e-5
+    rng = np.random.default_rng(31)
+    layers = [
+        LayerSpec(attention_spec("a0", d, 4, 2, 16, 0.3), ffn_spec("f0", d, 120, "gelu_tanh"), norm_spec("n0", d, eps), None, arrangement="toy_parallel"),
+        LayerSpec(attention_spec("a1", d, 3, 3, 32, 0.05), ffn_spec("f1", d, 88, "gelu_erf"), RmsSpec(d, eps, "r1a"), RmsSpec(d, eps, "r1b"),
+                  arrangement="toy_post_norm"),
+    ]
+    tw = {"emb": rand(rng, V, d, scale=0.5), "pos": rand(rng, P, d, scale=0.3), "r1a.w": rand(rng, d, scale=0.1, mean=1.0),
+          "r1b.w": rand(rng, d, scale=0.1, mean=1.0), "rf.w": rand(rng, d, scale=0.1, mean=1.0), **norm_tensors(rng, "n0", d),
+          **attention_tensors(rng, "a0", d, 4, 2, 16), **attention_tensors(rng, "a1", d, 3, 3, 32),
+          **ffn_tensors(rng, "f0", d, 120), **ffn_tensors(rng, "f1", d, 88)}
+    if dtype == "bfloat16":
+        tw = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v) for k, v in tw.items()}
+    plan = ModelPlan(architecture="toy_arranged", width=d, vocab_size=V, max_positions=P,
+                     embedding=TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": T("emb")}),
+                     residual_position=PositionSpec("learned_positions", "residual", P, d, {"table": T("pos")}),
+                     layers=layers, order=[OrderEntry(0), OrderEntry(1)], final_norm=RmsSpec(d, eps, "rf"),
+                     head=HeadSpec("lm_head", d, V, 1.0, {"weight": T("emb")}))
+    return plan, tw, dict(d=d, V=V, eps=eps)
+
+
+def arranged_plain(tw, info, ids):
+    eps = info["eps"]
+
+    def rms(x, name):
+        return x / np.sqrt((x * x).mean(axis=1, keepdims=True) + eps) * f64(tw[name + ".w"])
+
+    x = f64(tw["emb"])[ids] + f64(tw["pos"])[:len(ids)]
+    h = plain_norm(x, tw, "n0", eps)
+    a, _ = plain_attention(h, tw, "a0", 4, 2, 16, 0.3)
+    x = x + a + plain_ffn(h, tw, "f0", "gelu_tanh")
+    a, _ = plain_attention(x, tw, "a1", 3, 3, 32, 0.05)  # (it reads the stream as it is, several units large: a small scale keeps the scores moderate)
+    x = rms(x + a, "r1a")
+    x = rms(x + plain_ffn(x, tw, "f1", "gelu_erf"), "r1b")
+    return rms(x, "rf") @ f64(tw["emb"]).T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_other_arrangements_of_a_block(dtype):
+    """A root-mean-square norm, a parallel block and a post-norm block, all defined here, are
+    registered and built around the framework's attention and feed-forward and stepped under every
+    way of cutting the work: the norm's kind, where it stands and what the stream holds between the
+    parts belong to the plan, not to the model class. (The parts here say nothing of padding rows, split
+    streams or recorded lists: the engine then pads nothing, adds planes up first and runs their Python.)"""
+    from liyab_amd.engine import EngineCore
+
+    plan, tw, info = arranged_model(dtype)
+    reqs = {f"p{i}": tt.random_tokens(60 + i, n, info["V"]) for i, n in enumerate([35, 160, 3, 81])}
+    ref = {rid: arranged_plain(tw, info, toks) for rid, toks in reqs.items()}
+    # (a plausible mistake fails it: a mean taken off in the toy norm, or the second part reading the stream
+    # after the first has added to it, moves the logits by far more than the tolerance)
+    x = f64(tw["emb"])[reqs["p0"]] + f64(tw["pos"])[:35]
+    assert tt.rel_err((x - x.mean(axis=1, keepdims=True)) @ f64(tw["emb"]).T, x @ f64(tw["emb"]).T) > 1e-2
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs, (7, 2, 31, 3))),
+                        ("mixed", tt.schedule_mixed(reqs, seed=7))):
+        for use_graphs in (False, True):
+            core = EngineCore.from_plan(plan, tw, dtype=dtype, page_size=16, max_tokens=tt.max_live_tokens(steps), max_requests=4,
+                                        use_graphs=use_graphs)
+            assert not core.step_fn.pads_rows and core.model.replayed_layers == 0
+            got = tt.run_schedule(core, steps)
+            tt.check_against_plain(got, reqs, ref, TOL_TOY[dtype], f"arranged toy {name} {dtype}")
+            assert core.model.replayed_layers == 0
+            core.manager.check()
+            assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
 
 
 def test_unknown_kinds_are_refused_by_name():
