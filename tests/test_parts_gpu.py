@@ -5,6 +5,7 @@ reads another layer's cache; the run order names a layer twice; a norm of anothe
 otherwise (parallel, post-norm) (needs the GPU)."""
 
 import math
+import os
 
 import numpy as np
 import pytest
@@ -1263,6 +1264,158 @@ def test_toy_norm_and_other_arrangements_of_a_block(dtype):
             assert core.model.replayed_layers == 0
             core.manager.check()
             assert all(core.manager.pages_in_use(g.index) == 0 for g in core.manager.groups)
+
+
+# ---------------------------------------------------------------------------
+# a whole architecture of a test's own, from its config.json to greedy tokens
+# ---------------------------------------------------------------------------
+class ToyWindowConfig:
+    """An architecture of this test's own: config.json keys of its own, a plan made of the
+    package's parts in a mix GPT-2 has not: layers alternate between attention over all keys and
+    grouped attention over a window (two cache groups), the head is a matrix of its own with a bias,
+    the feed-forward's width and activation alternate too. Nothing of it is in the package's files."""
+
+    architecture = "ToyWindowLM"
+
+    def __init__(self, raw):
+        self.raw = dict(raw)
+        for key in ("layers", "width", "heads", "kv_heads", "inner", "vocab", "positions", "window"):
+            if not isinstance(raw.get(key), int) or raw[key] <= 0:
+                from liyab_amd.errors import InvalidModel
+
+                raise InvalidModel(f"missing or invalid {key}")
+        self.eps = float(raw.get("eps", 1e-5))
+
+    @classmethod
+    def from_json(cls, raw):
+        return cls(raw)
+
+    def to_json(self):
+        return dict(self.raw, architectures=[self.architecture])
+
+    def plan(self):
+        from liyab_amd.config import (AttentionSpec, DenseFFNSpec, HeadSpec, LayerSpec, ModelPlan, NormSpec, OrderEntry, PositionSpec,
+                                      TensorSource, TokenEmbeddingSpec)
+        from liyab_amd.config.plan import Init
+
+        r = self.raw
+        d, H, V, P = r["width"], r["heads"], r["vocab"], r["positions"]
+        hd = d // H
+        small, unit = Init(0.08), Init(0.05, 1.0)
+
+        def norm(name):
+            return NormSpec("layernorm", d, self.eps, {"weight": TensorSource(name + ".gain", init=unit), "bias": TensorSource(name + ".shift", init=small)})
+
+        layers = []
+        for i in range(r["layers"]):
+            windowed = i % 2 == 1
+            Hkv = r["kv_heads"] if windowed else H
+            p = f"blocks.{i}"
+            mixer = AttentionSpec("attention", d, H, Hkv, hd, 1.0 / math.sqrt(hd), r["window"] if windowed else 0,
+                                  {"qkv_weight": TensorSource(p + ".qkv", init=small), "qkv_bias": TensorSource(p + ".qkv_b", init=small),
+                                   "out_weight": TensorSource(p + ".out", init=small), "out_bias": TensorSource(p + ".out_b", init=small)})
+            F = r["inner"] + 16 * (i % 2)
+            ffn = DenseFFNSpec("dense_ffn", d, F, "gelu_erf" if windowed else "gelu_tanh",
+                               {"up_weight": TensorSource(p + ".up", init=small), "up_bias": TensorSource(p + ".up_b", init=small),
+                                "down_weight": TensorSource(p + ".down", init=small), "down_bias": TensorSource(p + ".down_b", init=small)})
+            layers.append(LayerSpec(mixer, ffn, norm(p + ".norm_a"), norm(p + ".norm_f")))
+        return ModelPlan(architecture=self.architecture, width=d, vocab_size=V, max_positions=P,
+                         embedding=TokenEmbeddingSpec("token_embedding", V, d, 1.0, {"table": TensorSource("tokens", init=Init(0.3))}),
+                         residual_position=PositionSpec("learned_positions", "residual", P, d, {"table": TensorSource("places", init=Init(0.2))}),
+                         layers=layers, order=[OrderEntry(i) for i in range(r["layers"])], final_norm=norm("norm_out"),
+                         head=HeadSpec("lm_head", d, V, 1.0, {"weight": TensorSource("unembed", init=Init(0.1)), "bias": TensorSource("unembed_b", init=small)}))
+
+
+def toy_window_plain(raw, t, ids):
+    """The toy architecture's logits for a whole sequence, float64, from the folder's tensors by name."""
+    d, H, eps = raw["width"], raw["heads"], float(raw.get("eps", 1e-5))
+    hd = d // H
+    x = t["tokens"][ids] + t["places"][:len(ids)]
+    for i in range(raw["layers"]):
+        windowed = i % 2 == 1
+        Hkv = raw["kv_heads"] if windowed else H
+        p = f"blocks.{i}"
+        h = plain.layer_norm(x, t[p + ".norm_a.gain"], t[p + ".norm_a.shift"], eps)
+        qkv = h @ t[p + ".qkv"].T + t[p + ".qkv_b"]
+        q, k, v = qkv[:, :H * hd], qkv[:, H * hd:(H + Hkv) * hd], qkv[:, (H + Hkv) * hd:]
+        rep = H // Hkv
+        kk = np.concatenate([k[:, (hh // rep) * hd:(hh // rep + 1) * hd] for hh in range(H)], axis=1)
+        vv = np.concatenate([v[:, (hh // rep) * hd:(hh // rep + 1) * hd] for hh in range(H)], axis=1)
+        x = x + plain.causal_attention(q, kk, vv, H, 1.0 / math.sqrt(hd), raw["window"] if windowed else 0) @ t[p + ".out"].T + t[p + ".out_b"]
+        h = plain.layer_norm(x, t[p + ".norm_f.gain"], t[p + ".norm_f.shift"], eps)
+        act = plain.gelu_erf if windowed else plain.gelu_tanh
+        x = x + act(h @ t[p + ".up"].T + t[p + ".up_b"]) @ t[p + ".down"].T + t[p + ".down_b"]
+    return plain.layer_norm(x, t["norm_out.gain"], t["norm_out.shift"], eps) @ t["unembed"].T + t["unembed_b"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_architecture_of_the_tests_own_from_config_json_to_greedy_tokens(dtype, tmp_path):
+    """What adding an architecture takes: a configuration class (from_json, to_json, plan) and one call
+    of register_architecture, here from a test. From then on the name in config.json finds it: the
+    random-weights mode writes its folder from the plan's tensor names and rules, the loader reads it back by
+    name (and says what is missing when a tensor is taken out), the cache manager gives its two kinds of layers
+    groups of pages of their own, the step function runs it whole, in portions and mixed under graphs, and the
+    engine's loop generates greedy tokens with it; all against a plain implementation written here."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+
+    from liyab_amd import Engine, InvalidModel, SamplingParams, Unsupported
+    from liyab_amd.config import register_architecture
+    from liyab_amd.config.registry import load_config
+    from liyab_amd.engine import EngineCore
+    from liyab_amd.weights import write_random_model
+
+    raw = {"architectures": ["ToyWindowLM"], "layers": 3, "width": 96, "heads": 6, "kv_heads": 2, "inner": 136, "vocab": 333,
+           "positions": 200, "window": 40, "eps": 3e-5}
+    register_architecture("ToyWindowLM", ToyWindowConfig)
+    folder = write_random_model(str(tmp_path / "model"), raw, seed=4)
+    assert isinstance(load_config(folder), ToyWindowConfig)
+    with pytest.raises(Unsupported, match="ToyWindowLM"):  # the list of what is supported names it now
+        load_config(write_bad_config(tmp_path / "other", {"architectures": ["NoSuchLM"]}))
+    with pytest.raises(InvalidModel, match="missing or invalid kv_heads"):
+        load_config(write_bad_config(tmp_path / "incomplete", {k: v for k, v in raw.items() if k != "kv_heads"}))
+    config, tensors = plain.read_model(folder)
+    assert tensors["blocks.1.qkv"].shape == ((6 + 2 * 2) * 16, 96) and tensors["blocks.0.up"].shape == (136, 96) and tensors["blocks.1.up"].shape == (152, 96)
+    if dtype == "bfloat16":
+        tensors = plain.round_weights_to_bf16(tensors)
+    reqs = {f"w{i}": tt.random_tokens(20 + i, n, raw["vocab"]) for i, n in enumerate([200, 47, 3, 120])}
+    ref = {rid: toy_window_plain(raw, tensors, toks) for rid, toks in reqs.items()}
+    for name, steps in (("whole", tt.schedule_whole(reqs)), ("portions", tt.schedule_portions(reqs)), ("mixed", tt.schedule_mixed(reqs, seed=9))):
+        core = EngineCore(folder, dtype=dtype, page_size=8, max_tokens=tt.max_live_tokens(steps), max_requests=4, use_graphs=True)
+        assert sorted(g.spec.window for g in core.manager.groups) == [0, 40] and [len(g.layers) for g in core.manager.groups if g.spec.window == 0] == [2]
+        got = tt.run_schedule(core, steps)
+        tt.check_against_plain(got, reqs, ref, TOL[dtype], f"architecture {name} {dtype}", family="toy:architecture")
+        core.manager.check()
+        del core
+    # greedy tokens through the engine's loop and the scheduler
+    prompts = [reqs["w1"], reqs["w2"], reqs["w3"][:60]]
+    engine = Engine(folder, dtype=dtype, page_size=8, max_num_seqs=3, max_batched_tokens=48, prefill_chunk=32)
+    engine.stop_at_eos = False
+    for prompt, res in zip(prompts, engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16))):
+        assert len(res.tokens) == 16
+        rows = toy_window_plain(raw, tensors, prompt + res.tokens[:-1])[len(prompt) - 1:]
+        tol = 1e-5 if dtype == "float32" else TOL[dtype]
+        assert all(row[tok] >= row.max() - tol * np.abs(row).max() for row, tok in zip(rows, res.tokens))
+    # a folder with a tensor taken out: one error that names it
+    kept = {}
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        for key in f.keys():
+            if key != "blocks.2.norm_f.shift":
+                kept[key] = f.get_tensor(key)
+    broken = tmp_path / "broken"
+    broken.mkdir()
+    save_file(kept, str(broken / "model.safetensors"))
+    (broken / "config.json").write_text((tmp_path / "model" / "config.json").read_text())
+    with pytest.raises(InvalidModel, match="blocks.2.norm_f.shift"):
+        EngineCore(str(broken), dtype=dtype, page_size=8, max_tokens=64, max_requests=2)
+
+
+def write_bad_config(folder, raw):
+    import json
+
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(raw))
+    return str(folder)
 
 
 def test_unknown_kinds_are_refused_by_name():
