@@ -12,6 +12,8 @@
 // starts from zero; the chunks' sums added in ascending order. (Chunks, so that
 // a step of few rows, which has few output elements, can still spread one
 // element's sum over several waves: gemm_rowwise_f32_kernel below.)
+#include <type_traits>
+
 #include "activations.h"
 #include "common.h"
 #include "launchers.h"
@@ -89,6 +91,84 @@ gemm_simple_kernel(OutT* __restrict__ out, int64_t ldo, const T* __restrict__ a,
     }
 }
 
+// The tiled kernel for large 32-bit products: tiles of 128 x 128, a thread 8 x 8 output elements (rows
+// ty * 4 + {0..3} and 64 + the same, columns likewise), so that a step of k costs four 16-byte reads from
+// LDS for 64 multiply-adds where the 64 x 64 tiles above read two for 16: there the reads set the pace
+// (35 TFLOP/s). The chains and the order of sums are the ones above, bit for bit.
+constexpr int BM2 = 128, BN2 = 128;
+
+template <int EPI, bool EXACT>
+__global__ void __launch_bounds__(256)
+gemm_simple128_f32_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ a, int64_t lda, const float* __restrict__ w,
+                          const float* __restrict__ bias, float* __restrict__ residual, int64_t ldr, int M, int N, int K) {
+    __shared__ float As[BK][BM2 + 4];
+    __shared__ float Ws[BK][BN2 + 4];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * BM2, n0 = blockIdx.x * BN2;
+    const int ty = tid / 16, tx = tid % 16;
+    const int lrow = tid / 4, lk = (tid % 4) * 4;  // this thread loads 4 k of rows lrow and lrow + 64
+    float acc[8][8] = {}, tot[8][8] = {};
+    for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = m0 + lrow + 64 * h, n = n0 + lrow + 64 * h;
+            const float* p = a + static_cast<int64_t>(m) * lda + k0 + lk;
+            const float* q = w + static_cast<int64_t>(n) * K + k0 + lk;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool in = k0 + lk + i < K;
+                As[lk + i][lrow + 64 * h] = (m < M && in) ? p[i] : 0.0f;
+                Ws[lk + i][lrow + 64 * h] = (n < N && in) ? q[i] : 0.0f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float av[8], wv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                av[i] = As[k][ty * 4 + i];
+                av[4 + i] = As[k][64 + ty * 4 + i];
+                wv[i] = Ws[k][tx * 4 + i];
+                wv[4 + i] = Ws[k][64 + tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        if ((k0 + BK) % kChunk == 0 || k0 + BK >= K) {  // the chunk's chain ends: its sum joins the others'
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    tot[i][j] += acc[i][j];
+                    acc[i][j] = 0.0f;
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + (i / 4) * 64 + ty * 4 + i % 4;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int n = n0 + (j / 4) * 64 + tx * 4 + j % 4;
+            if (n >= N) continue;
+            float v = tot[i][j];
+            if (bias != nullptr) v += bias[n];
+            if constexpr (EPI == kEpiGeluTanh) v = gelu_tanh(v);
+            if constexpr (EPI == kEpiGeluErf) v = EXACT ? gelu_erf_exact(v) : gelu_erf_fast(v);
+            if constexpr (EPI == kEpiResidual) {
+                residual[static_cast<int64_t>(m) * ldr + n] += v;
+            } else {
+                out[static_cast<int64_t>(m) * ldo + n] = v;
+            }
+        }
+    }
+}
+
 // The same product for steps of few rows (decoding), in the same order of sums, so a row's
 // result has the same bits whichever of the two kernels computed it. A workgroup of four or
 // eight waves takes NB output features and 16 rows (blockIdx.y: which 16); the chunks of K go round the waves. A wave
@@ -101,6 +181,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 constexpr int kRowwiseRows = 16;     // rows a workgroup
 constexpr int kRowwiseMaxRows = 64;  // steps of at most this many rows take the row-wise kernel
+constexpr int kTiled128MinTiles = 512;  // tiles of 128 x 128 from this many on: two a compute unit (288 of them, 2,048 x 2,304 x 768: 305 us against 222 in tiles of 64 x 64; 576, 4,096 rows: 349 against 440)
 constexpr int kTiledMinTiles = 512;  // and so do larger ones that would give the tiled kernel fewer tiles than this
 
 template <int NB, int WAVES, int EPI, bool EXACT>
@@ -258,6 +339,22 @@ int launch_simple(void* out, int64_t ldo, const void* a, int64_t lda, const void
     auto* o = static_cast<OutT*>(out);
     auto* pa = static_cast<const T*>(a);
     auto* pw = static_cast<const T*>(w);
+    if constexpr (std::is_same<T, float>::value && std::is_same<OutT, float>::value) {
+        // large 32-bit products in tiles of 128 x 128 once those are two a compute unit (45-57 TFLOP/s against 31-37)
+        const dim3 grid2((N + BN2 - 1) / BN2, (M + BM2 - 1) / BM2);
+        if (static_cast<int64_t>(grid2.x) * grid2.y >= kTiled128MinTiles) {
+#define LIYAB_GO2(E) gemm_simple128_f32_kernel<E, EXACT><<<grid2, 256, 0, stream>>>(o, ldo, pa, lda, pw, bias, residual, ldr, M, N, K)
+            switch (epi) {
+                case kEpiNone: LIYAB_GO2(kEpiNone); break;
+                case kEpiGeluTanh: LIYAB_GO2(kEpiGeluTanh); break;
+                case kEpiGeluErf: LIYAB_GO2(kEpiGeluErf); break;
+                case kEpiResidual: LIYAB_GO2(kEpiResidual); break;
+                default: return fail(1, "gemm: unknown epilogue %d", epi);
+            }
+#undef LIYAB_GO2
+            return check_launch("gemm_simple128");
+        }
+    }
 #define LIYAB_GO(E) \
     gemm_simple_kernel<T, OutT, E, EXACT><<<grid, 256, 0, stream>>>(o, ldo, pa, lda, pw, bias, residual, ldr, M, N, K)
     switch (epi) {

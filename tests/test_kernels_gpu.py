@@ -198,7 +198,9 @@ F32_SHAPES = GEMM_SHAPES + [(16, 1500, 100), (9, 2600, 260), (5, 3000, 72), (12,
                             (16, 33, 3076), (20, 70, 50),
                             # 17 to 64 rows in one workgroup: 16 features a workgroup with 2, 3 and 4 rows a thread,
                             # 8 with 1 and 2, 4 with a long K
-                            (24, 4100, 200), (45, 4097, 68), (64, 4800, 324), (30, 2050, 1604), (17, 100, 3076)]
+                            (24, 4100, 200), (45, 4097, 68), (64, 4800, 324), (30, 2050, 1604), (17, 100, 3076),
+                            # large enough for the tiles of 128 x 128 (528 of them), with edges on both sides and a K that ends inside a step of 16
+                            (1100, 7300, 68)]
 
 
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
