@@ -167,3 +167,14 @@ def test_what_makes_two_layers_one_kind_and_how_a_recorded_list_gets_another_lay
     assert rec.usable and rec.positions.tolist() == [2, 5] and rec.offsets.tolist() == [16, 0]
     assert rec.for_layer(np.array([20000, 90000], dtype=np.uint64)).tolist() == [7, 3, 20016, 999, 6000, 90000, 1064, 1008]
     assert not _Recorded(np.array([1], dtype=np.uint64), np.array([True]), np.array([1000, 1032], dtype=np.uint64), [64, 8], None).usable  # overlapping tensors
+
+
+def test_padded_sizes_of_steps_with_prompt_portions():
+    """The rows of a step in which some request brings more than one token: multiples of 16 up to 64,
+    of 64 up to 1,024, of 128 beyond; never fewer than the tokens, never a whole unit more."""
+    from liyab_amd.engine.step import padded_rows
+
+    assert [padded_rows(n) for n in (2, 16, 17, 33, 48, 64, 65, 500, 1024, 1025, 2048)] == [16, 16, 32, 48, 48, 64, 128, 512, 1024, 1152, 2048]
+    for n in range(1, 3000):
+        unit = 16 if n <= 64 else 64 if n <= 1024 else 128
+        assert n <= padded_rows(n) < n + unit and padded_rows(n) % unit == 0 and padded_rows(padded_rows(n)) == padded_rows(n)
