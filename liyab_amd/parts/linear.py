@@ -21,7 +21,10 @@ from .norms import Normed
 # Folding the norm into a decode step's products saves a launch of the seven a layer has; every
 # workgroup of the product then repeats the norm of all rows ahead of its multiplies, which
 # pays while the rows are few (us a decode step at GPT-2 small's sizes, folded and not: 8 rows
-# 420 / 471, 16 rows 498 / 524, 24 rows 657 / 679, 32 rows 711 / 694, 64 rows 954 / 810).
+# 420 / 471, 16 rows 498 / 524, 24 rows 657 / 679, 32 rows 711 / 694, 64 rows 954 / 810; and 64 rows
+# with a workgroup normalising 32 of them for 32 output features, a wave asking for its four rows
+# together, where the stream is whole (the feed-forward's first product): 721 against 713, 48 rows 656
+# against 652. That form was taken out again.)
 FOLD_NORM = True
 FOLD_NORM_ROWS = 24
 TILED_PARTS = True  # products of 33 to 64 rows that are added to the stream: tiled and cut over K (ops.tiled_k_parts)
