@@ -7,6 +7,7 @@
 
 #include "cache_manager.h"
 #include "scheduler.h"
+#include "attention_plan.h"
 #include "step_meta.h"
 
 using namespace liyab_host;
@@ -88,7 +89,7 @@ int liyab_step_fill(void* h, const StepShape* shape, const int* slots, const int
                     const int* want_counts, const int* wants, int vocab_size, int32_t* block) {
     return step_fill(*static_cast<CacheManager*>(h), *shape, slots, q_lens, tokens, want_counts, wants, vocab_size, block, &g_error);
 }
-// attention's own words of a step (step_meta.h): counts[0] tiles, counts[1] single rows
+// attention's own words of a step (attention_plan.h): counts[0] tiles, counts[1] single rows
 void liyab_attn_counts(int n_seqs, const int* q_lens, int decode_q_len, int attn_tile, int* counts) {
     attn_counts(n_seqs, q_lens, decode_q_len, attn_tile, &counts[0], &counts[1]);
 }

@@ -14,6 +14,7 @@
 
 #include "../cache_manager.h"
 #include "../scheduler.h"
+#include "../attention_plan.h"
 #include "../step_meta.h"
 
 using namespace liyab_host;

@@ -42,14 +42,4 @@ Status step_shape(const CacheManager& m, int n_seqs, const int* slots, const int
 Status step_fill(const CacheManager& m, const StepShape& shape, const int* slots, const int* q_lens, const int64_t* tokens,
                  const int* want_counts, const int* wants, int vocab_size, int32_t* block, std::string* err);
 
-// Attention's own words of a step in which some request brings more than decode_q_len tokens:
-// the long portions cut into tiles of up to attn_tile consecutive queries (4 words a tile: request
-// index, first row, first position, queries; the tile that ends at the latest position first, so
-// that the short ones fill the gaps at the end), and the rows of the short portions, which are
-// attended one by one. attn_counts gives (tiles, single rows); attn_fill writes 4 * max(tiles, 1)
-// words of tiles followed by max(single rows, 1) words of rows. first_pos: each request's length
-// before the step.
-void attn_counts(int n_seqs, const int* q_lens, int decode_q_len, int attn_tile, int* n_tiles, int* n_single);
-void attn_fill(int n_seqs, const int* q_lens, const int* first_pos, int decode_q_len, int attn_tile, int32_t* words);
-
 }  // namespace liyab_host

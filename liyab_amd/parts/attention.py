@@ -61,7 +61,7 @@ class AttentionStepPlanner:
     """Attention's words of a step's metadata and its term of the graph key: the reference cuts a
     pass's attention into per-segment work the same way, on the host, before its kernels run
     (src/core/transformer.cpp:2169-2174, 2396-2452). The lists are laid out natively
-    (csrc/host/step_meta.cpp: attn_counts, attn_fill)."""
+    (csrc/host/attention_plan.cpp: attn_counts, attn_fill)."""
 
     name = "attention"
 
