@@ -89,11 +89,13 @@ def padded_rows(n: int) -> int:
 
 
 class StepFunction:
-    """`use_graphs`: a step whose shape (tokens, requests, wanted rows, and the key of every
+    """`use_graphs`: a step whose shape (rows, requests, wanted rows, and the key of every
     part's step planner: attention's mode, context bucket and tiles) has been seen before is
     captured into a HIP graph the second time and replayed from then on; what varies between
     such steps lives in the metadata block, whose address and layout the shape fixes. Kernels
-    must then depend on the host only through the shape: the ones in this package do."""
+    must then depend on the host only through the shape: the ones in this package do. Steps
+    that bring prompt portions are padded with rows of no request to sizes that come back
+    (`padded_rows`), where every part of the model takes such rows (`pads_rows`)."""
 
     def __init__(self, model, manager: CacheManager, storage: CacheStorage, device="cuda:0", use_graphs: bool = True,
                  max_graphs: int = 256, batch_invariant: bool = False):
